@@ -1,0 +1,371 @@
+/*
+ * CPU oracle for the MoE routing hot path.  TEST INFRASTRUCTURE ONLY.
+ *
+ * Sequential, plain-C restatement of what the reference's CUDA kernels compute,
+ * written from their source text (paths are relative to the reference tree):
+ *
+ *   src/router/location.cu   generate_indices_and_loads, throttle_hotmask,
+ *                            convert_{seat_to_tag,tag_to_seat}_indices
+ *   src/router/route.cu      dispatch_with_{seat,tag}_indices_{1d,2d},
+ *                            combine_with_seat_indices, init_with_seat_indices
+ *   src/backend/torch/router.cc   shape/dtype conventions around them
+ *
+ * Only tests, the smoke check and the bench's cpu_baseline leg may link or call
+ * this file; the product path never does.
+ *
+ * Parity status: every function here is pinned by checks that do not retype
+ * its formula (reference notebook vectors, the reference test-suite's own
+ * closed forms, permutation/round-trip invariants, brute force on tiny
+ * inputs); see tests/test_oracle_*.py.  No function is "parity unpinned".
+ *
+ * Index conventions (location.cu:132-195): all index tensors are int32
+ * row-major [T,E]; values are 1-based and 0 means "not routed / empty slot".
+ *
+ * Build: gcc -O2 -ffp-contract=off -shared -fPIC (no FMA contraction, so the
+ * fp32 combine keeps one rounding per multiply and one per add, like the
+ * reference's `in * gate` followed by atomicAdd, route.cu:236-243).
+ */
+#include <stdint.h>
+#include <stddef.h>
+#include <string.h>
+
+enum { ORACLE_F32 = 0, ORACLE_F16 = 1, ORACLE_BF16 = 2 };
+
+/* ---------- 16-bit float helpers (round-to-nearest-even) ---------- */
+
+static float bits_to_float(uint32_t u) {
+  float f;
+  memcpy(&f, &u, 4);
+  return f;
+}
+static uint32_t float_to_bits(float f) {
+  uint32_t u;
+  memcpy(&u, &f, 4);
+  return u;
+}
+
+static float bf16_to_float(uint16_t h) { return bits_to_float((uint32_t)h << 16); }
+
+static uint16_t float_to_bf16(float f) {
+  uint32_t u = float_to_bits(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u); /* quiet NaN */
+  uint32_t lsb = (u >> 16) & 1u;
+  u += 0x7fffu + lsb;
+  return (uint16_t)(u >> 16);
+}
+
+static float f16_to_float(uint16_t h) {
+  uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+  uint32_t exp = (h >> 10) & 0x1fu;
+  uint32_t man = h & 0x3ffu;
+  if (exp == 0) {
+    if (man == 0) return bits_to_float(sign);
+    /* subnormal: value = man * 2^-24 */
+    float v = (float)man * (1.0f / 16777216.0f);
+    return sign ? -v : v;
+  }
+  if (exp == 31) return bits_to_float(sign | 0x7f800000u | (man << 13));
+  return bits_to_float(sign | ((exp + 112u) << 23) | (man << 13));
+}
+
+static uint16_t float_to_f16(float f) {
+  uint32_t u = float_to_bits(f);
+  uint16_t sign = (uint16_t)((u >> 16) & 0x8000u);
+  uint32_t a = u & 0x7fffffffu;
+  if (a > 0x7f800000u) return (uint16_t)(sign | 0x7e00u);  /* NaN */
+  if (a >= 0x47800000u) return (uint16_t)(sign | 0x7c00u); /* >= 65536 (or inf) -> inf */
+  if (a >= 0x477ff000u) return (uint16_t)(sign | 0x7c00u); /* rounds up to inf */
+  if (a < 0x33000001u) return sign;                        /* <= 2^-25 rounds to zero */
+  int32_t e = (int32_t)(a >> 23) - 127;
+  uint32_t m = (a & 0x7fffffu) | 0x800000u; /* 24-bit significand */
+  int shift;                                /* bits dropped from m */
+  uint32_t hexp;
+  if (e < -14) { /* subnormal half */
+    shift = 13 + (-14 - e);
+    hexp = 0;
+  } else {
+    shift = 13;
+    hexp = (uint32_t)(e + 15);
+  }
+  uint32_t kept = m >> shift;
+  uint32_t rem = m & ((1u << shift) - 1u);
+  uint32_t half = 1u << (shift - 1);
+  if (rem > half || (rem == half && (kept & 1u))) kept++;
+  uint32_t out;
+  if (hexp == 0) {
+    out = kept; /* may carry into exponent 1: correct encoding */
+  } else {
+    out = ((hexp - 1u) << 10) + kept; /* kept includes the hidden bit (1<<10) */
+  }
+  return (uint16_t)(sign | out);
+}
+
+static size_t elem_size(int dtype) { return dtype == ORACLE_F32 ? 4 : 2; }
+
+static float load_elem(const void* p, int dtype, size_t i) {
+  if (dtype == ORACLE_F32) return ((const float*)p)[i];
+  if (dtype == ORACLE_F16) return f16_to_float(((const uint16_t*)p)[i]);
+  return bf16_to_float(((const uint16_t*)p)[i]);
+}
+
+static void store_elem(void* p, int dtype, size_t i, float v) {
+  if (dtype == ORACLE_F32)
+    ((float*)p)[i] = v;
+  else if (dtype == ORACLE_F16)
+    ((uint16_t*)p)[i] = float_to_f16(v);
+  else
+    ((uint16_t*)p)[i] = float_to_bf16(v);
+}
+
+/* exported so tests can pin the converters against numpy/torch */
+float oracle_f16_to_float(uint16_t h) { return f16_to_float(h); }
+uint16_t oracle_float_to_f16(float f) { return float_to_f16(f); }
+float oracle_bf16_to_float(uint16_t h) { return bf16_to_float(h); }
+uint16_t oracle_float_to_bf16(float f) { return float_to_bf16(f); }
+
+/* ---------- location.cu ---------- */
+
+/*
+ * generate_indices_and_loads  (location.cu:132-257, launcher :335-379)
+ *
+ * Per column e: a running inclusive sum of the mask values ("location"),
+ * index = location * mask (location.cu:177-178).  Seat mode writes it at
+ * [t,e]; tag mode writes t+1 at [index-1,e] (:180-185).  `indices` must be
+ * zero-filled by the caller (router.cc:74).  Load rules: location.cu:222-256;
+ * path_wise_padding is honoured only together with capacity_padding (:349-358).
+ */
+void oracle_generate_indices_and_loads(const int32_t* mask, int32_t* indices, int32_t* loads,
+                                       int T, int E, const int32_t* caps, int C,
+                                       int capacity_padding, int path_wise_padding,
+                                       int is_tag_index) {
+  if (caps == NULL) C = 0;
+  if (!capacity_padding) path_wise_padding = 0;
+  for (int e = 0; e < E; ++e) {
+    int prefix = 0;
+    for (int t = 0; t < T; ++t) {
+      int m = mask[(size_t)t * E + e];
+      prefix += m;
+      int index = prefix * m;
+      if (index != 0) {
+        if (is_tag_index) {
+          if (index >= 1 && index <= T) indices[(size_t)(index - 1) * E + e] = t + 1;
+        } else {
+          indices[(size_t)t * E + e] = index;
+        }
+      }
+    }
+    int real_load = prefix;
+    if (path_wise_padding) {
+      loads[e] = caps[e];
+      continue;
+    }
+    if (real_load == 0) {
+      loads[e] = 0;
+      continue;
+    }
+    if (capacity_padding) {
+      int v = caps[C - 1];
+      for (int i = 0; i < C; ++i)
+        if (real_load <= caps[i]) {
+          v = caps[i];
+          break;
+        }
+      loads[e] = v;
+    } else {
+      if (C == 0) {
+        loads[e] = real_load;
+        continue;
+      }
+      int v = caps[C - 1];
+      for (int i = 0; i < C; ++i)
+        if (real_load <= caps[i]) {
+          v = real_load;
+          break;
+        }
+      loads[e] = v;
+    }
+  }
+}
+
+/*
+ * throttle_hotmask  (location.cu:59-130)
+ *
+ * The reference walks each column in chunks of 1024 rows; inside a chunk a row
+ * is kept iff mask==1 and prefix+rank <= threshold; after a chunk, the running
+ * prefix absorbs the chunk's sum and the walk stops once it reaches the
+ * threshold (then prefix := threshold).  `out` must be zero-filled by the
+ * caller (router.cc:26); prefix is updated in place.
+ */
+void oracle_throttle_hotmask(const int32_t* mask, int32_t* out, int32_t* prefix,
+                             const int32_t* threshold, int T, int E) {
+  const int chunk = 1024;
+  for (int e = 0; e < E; ++e) {
+    int run = prefix[e];
+    int thr = threshold[e];
+    for (int s = 0; s < T; s += chunk) {
+      int loc = run;
+      int end = s + chunk < T ? s + chunk : T;
+      for (int t = s; t < end; ++t) {
+        int m = mask[(size_t)t * E + e];
+        loc += m;
+        if (m == 1 && loc <= thr) out[(size_t)t * E + e] = 1;
+      }
+      run = loc;
+      if (run >= thr) {
+        run = thr;
+        break;
+      }
+    }
+    prefix[e] = run;
+  }
+}
+
+/*
+ * convert_seat_to_tag_indices (location.cu:259-278): tag[seat-1,e] = t+1.
+ * convert_tag_to_seat_indices (location.cu:280-302): slot s (< loads[e]) is
+ * handled by thread s%1024, which walks s, s+1024, ... and stops at its first
+ * zero tag; so slot s is converted iff tags at s, s-1024, s-2048, ... are all
+ * non-zero.  `dst` must be zero-filled by the caller (router.cc:102).
+ */
+void oracle_convert_index_format(const int32_t* src, int32_t* dst, const int32_t* loads, int T,
+                                 int E, int tag_to_seat) {
+  if (!tag_to_seat) {
+    for (int e = 0; e < E; ++e)
+      for (int t = 0; t < T; ++t) {
+        int seat = src[(size_t)t * E + e];
+        if (seat != 0 && seat >= 1 && seat <= T) dst[(size_t)(seat - 1) * E + e] = t + 1;
+      }
+    return;
+  }
+  for (int e = 0; e < E; ++e) {
+    int load = loads[e];
+    if (load > T) load = T;
+    for (int lane = 0; lane < 1024; ++lane)
+      for (int s = lane; s < load; s += 1024) {
+        int tag = src[(size_t)s * E + e];
+        if (tag == 0) break;
+        if (tag >= 1 && tag <= T) dst[(size_t)(tag - 1) * E + e] = s + 1;
+      }
+  }
+}
+
+/* ---------- route.cu ---------- */
+
+static void copy_row(const void* src, size_t src_row, void* dst, size_t dst_row, int cell,
+                     int dtype, int weighted, float gate) {
+  size_t es = elem_size(dtype);
+  if (!weighted) {
+    memcpy((char*)dst + dst_row * cell * es, (const char*)src + src_row * cell * es, cell * es);
+    return;
+  }
+  for (int j = 0; j < cell; ++j) {
+    float v = load_elem(src, dtype, src_row * cell + j) * gate;
+    store_elem(dst, dtype, dst_row * cell + j, v);
+  }
+}
+
+/*
+ * dispatch_with_indices_and_loads  (route.cu:13-206; shapes router.cc:131-273)
+ *
+ *   src   1-d: [T, cell];  2-d: [T, E, cell] (expert e reads slice [:, e, :];
+ *         the binding transposes to [E,T,cell] first, router.cc:212)
+ *   dst   [P, cell], zero-filled by the caller (router.cc:219)
+ *   gates [T, E] in the data dtype or NULL (1-d only, route.cu:362)
+ *   start[e] = e*max_path_load when max_path_load != 0, else sum(loads[:e])
+ *   seat mode: every (t,e) with 1 <= idx <= loads[e] copies row t to
+ *         start[e]+idx-1 (route.cu:37-50)
+ *   tag mode: slot i < loads[e] is handled by block i%512, which walks
+ *         i, i+512, ... and stops at its first zero tag (route.cu:84-92);
+ *         dst row start[e]+i receives row tag-1
+ *   new_tags (zero-filled by the caller) receive old_tags[source row]
+ *         (route.cu:51-53); old_tags NULL means "no tag generation".
+ *   Rows >= P are never written (guard added here; the reference would write
+ *   out of bounds).
+ */
+void oracle_dispatch(const void* src, void* dst, const void* gates, const int32_t* idx,
+                     const int32_t* loads, const int32_t* old_tags, int32_t* new_tags, int T,
+                     int cell, int E, int P, int max_path_load, int is_1d, int is_tag_index,
+                     int dtype) {
+  int weighted = gates != NULL;
+  long start = 0;
+  for (int e = 0; e < E; ++e) {
+    long load_start = max_path_load != 0 ? (long)e * max_path_load : start;
+    int path_load = loads[e];
+    if (!is_tag_index) {
+      for (int t = 0; t < T; ++t) {
+        int seat = idx[(size_t)t * E + e];
+        if (seat == 0 || seat > path_load || seat < 0) continue;
+        long row = load_start + seat - 1;
+        if (row >= P) continue;
+        size_t src_row = is_1d ? (size_t)t : (size_t)t * E + e;
+        float g = weighted ? load_elem(gates, dtype, (size_t)t * E + e) : 1.0f;
+        copy_row(src, src_row, dst, (size_t)row, cell, dtype, weighted, g);
+        if (old_tags) new_tags[row] = old_tags[t];
+      }
+    } else {
+      for (int blk = 0; blk < 512; ++blk)
+        for (int i = blk; i < T; i += 512) {
+          if (i >= path_load) continue;
+          int tag = idx[(size_t)i * E + e];
+          if (tag == 0) break;
+          if (tag < 1 || tag > T) continue;
+          long row = load_start + i;
+          if (row >= P) continue;
+          int t = tag - 1;
+          size_t src_row = is_1d ? (size_t)t : (size_t)t * E + e;
+          float g = weighted ? load_elem(gates, dtype, (size_t)t * E + e) : 1.0f;
+          copy_row(src, src_row, dst, (size_t)row, cell, dtype, weighted, g);
+          if (old_tags) new_tags[row] = old_tags[t];
+        }
+    }
+    start += path_load;
+  }
+}
+
+/*
+ * combine_with_indices_and_loads, seat mode  (route.cu:208-282, 467-518)
+ *
+ *   src [P, cell] in in_dtype; dst [T, cell] in out_dtype; gates [T,E] in
+ *   gate_dtype or NULL.
+ *   For token t the accumulator starts at 0 (non-residual: dst is torch::zeros,
+ *   router.cc:460; residual: init_with_seat_indices zeroes the rows of routed
+ *   tokens, route.cu:250-282) and adds, for e ascending with
+ *   1 <= idx <= loads[e], src[start[e]+idx-1] * gate: one fp32 multiply, then
+ *   one fp32 add (the atomicAdd of route.cu:243 is issued by one thread per
+ *   element in program order, so the order is ascending e).  Residual rows of
+ *   tokens with no valid route are left untouched.
+ *   The reference binding only instantiates fp32 (router.cc:435,443); for
+ *   16-bit inputs this oracle defines: widen to fp32, accumulate in fp32 in the
+ *   same order, round once on store.
+ */
+void oracle_combine(const void* src, void* dst, const void* gates, const int32_t* idx,
+                    const int32_t* loads, int T, int cell, int E, int P, int max_path_load,
+                    int is_residual, int in_dtype, int out_dtype, int gate_dtype) {
+  for (int t = 0; t < T; ++t) {
+    int routed = 0;
+    for (int j = 0; j < cell; ++j) {
+      float acc = 0.0f;
+      long start = 0;
+      int any = 0;
+      for (int e = 0; e < E; ++e) {
+        int seat = idx[(size_t)t * E + e];
+        int load = loads[e];
+        long load_start = max_path_load != 0 ? (long)e * max_path_load : start;
+        start += load;
+        if (seat == 0 || seat > load || seat < 0) continue;
+        long row = load_start + seat - 1;
+        if (row >= P) continue;
+        any = 1;
+        float v = load_elem(src, in_dtype, (size_t)row * cell + j);
+        if (gates) {
+          float g = load_elem(gates, gate_dtype, (size_t)t * E + e);
+          v = v * g;
+        }
+        acc = acc + v;
+      }
+      routed = any;
+      if (any || !is_residual) store_elem(dst, out_dtype, (size_t)t * cell + j, acc);
+    }
+    (void)routed;
+  }
+}
