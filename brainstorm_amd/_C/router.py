@@ -1,0 +1,456 @@
+"""``brt._C.router`` -- same names, arguments, defaults and error behaviour as the
+pybind11 module of the reference (src/backend/torch/router.cc:479-513,
+python/brt/_C/router.pyi), implemented over the C ABI of ``libbrt_hip.so``.
+
+PyTorch is used for tensor allocation and stream handles only; every device
+computation of the seat-index path is a hand-written HIP kernel.  Work is
+enqueued on the current PyTorch stream (the reference uses the default stream,
+router.cc:78; identical when no stream context is active).
+"""
+from __future__ import annotations
+
+import weakref
+from typing import List, Optional, Tuple
+
+import torch
+
+from brainstorm_amd import _lib
+
+_DT = {torch.float32: _lib.F32, torch.float16: _lib.F16, torch.bfloat16: _lib.BF16}
+
+__all__ = [
+    "throttle_hotmask",
+    "generate_indices_and_loads",
+    "convert_index_format",
+    "dispatch_with_indices_and_loads",
+    "split_fused_cells_to_paths",
+    "fuse_split_cells_from_paths",
+    "combine_with_indices_and_loads",
+    "combine_with_src_indices",
+]
+
+
+# --------------------------------------------------------------------- helpers
+def _check_on_device(t: torch.Tensor, name: str) -> None:
+    # CHECK_ON_CUDA, src/backend/torch/torch.h:16-21
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must be a CUDA tensor")
+
+
+def _check_int32(t: torch.Tensor, name: str) -> None:
+    if t.dtype != torch.int32:  # data_ptr<int>() in the reference throws likewise
+        raise RuntimeError(f"{name} must be an int32 tensor, got {t.dtype}")
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else t.data_ptr()
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+_workspaces = {}
+
+
+def _scan_workspace(device: torch.device, T: int, E: int) -> torch.Tensor:
+    """Zero-initialised scan workspace, one per (device, stream), grown on demand."""
+    need = _lib.lib().brt_hip_scan_workspace_bytes(T, E)
+    key = (device.index, _stream())
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < need:
+        ws = torch.zeros(max(need, 1 << 16), dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
+class _Pairing:
+    """Remembers which (indices, loads) pair one index-generation call produced,
+    together with the true per-path counts, so that dispatch can zero-fill the
+    padding rows itself instead of clearing the whole output first."""
+
+    __slots__ = ("indices_ref", "indices_ptr", "indices_version", "loads_version", "counts")
+
+    def __init__(self, indices, loads, counts):
+        self.indices_ref = weakref.ref(indices)
+        self.indices_ptr = indices.data_ptr()
+        self.indices_version = indices._version
+        self.loads_version = loads._version
+        self.counts = counts
+
+
+def _paired_counts(route_indices: torch.Tensor, loads: torch.Tensor) -> Optional[torch.Tensor]:
+    pairing = getattr(loads, "_brt_pairing", None)
+    if (
+        pairing is None
+        or pairing.indices_ref() is not route_indices
+        or pairing.indices_ptr != route_indices.data_ptr()
+        or pairing.indices_version != route_indices._version
+        or pairing.loads_version != loads._version
+    ):
+        return None
+    return pairing.counts
+
+
+# ------------------------------------------------------------------------- ops
+def throttle_hotmask(
+    hot_mask: torch.Tensor, prefix: torch.Tensor, threshold: torch.Tensor
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """router.cc:15-31.  ``prefix`` is updated in place and returned."""
+    _check_on_device(hot_mask, "hot_mask")
+    _check_on_device(prefix, "prefix")
+    _check_on_device(threshold, "threshold")
+    for t, n in ((hot_mask, "hot_mask"), (prefix, "prefix"), (threshold, "threshold")):
+        _check_int32(t, n)
+    if hot_mask.size(1) != prefix.size(0) or hot_mask.size(1) != threshold.size(0):
+        raise RuntimeError("prefix/threshold must have one entry per path")
+    hot_mask = hot_mask.contiguous()
+    T, E = hot_mask.shape
+    with torch.cuda.device(hot_mask.device):
+        throttled = torch.empty_like(hot_mask)
+        if T > 0:
+            ws = _scan_workspace(hot_mask.device, T, E)
+            _lib.check(_lib.lib().brt_hip_throttle_hotmask(
+                _ptr(hot_mask), _ptr(throttled), _ptr(prefix), _ptr(threshold.contiguous()),
+                T, E, _ptr(ws), ws.numel(), _stream()))
+    return throttled, prefix
+
+
+def generate_indices_and_loads(
+    hot_mask: torch.Tensor,
+    supported_capacities: Optional[torch.Tensor] = None,
+    capacity_padding: bool = False,
+    path_wise_padding: bool = False,
+    is_tag_index: bool = False,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """router.cc:48-80."""
+    _check_on_device(hot_mask, "hot_mask")
+    _check_int32(hot_mask, "hot_mask")
+    T, E = hot_mask.size(0), hot_mask.size(1)
+    with torch.cuda.device(hot_mask.device):
+        if hot_mask.numel() == 0:  # router.cc:59-62
+            return (torch.zeros((0, E), dtype=hot_mask.dtype, device=hot_mask.device),
+                    torch.zeros((E,), dtype=hot_mask.dtype, device=hot_mask.device))
+        caps = None
+        n_caps = 0
+        if supported_capacities is not None:
+            _check_on_device(supported_capacities, "supported_capacities")
+            _check_int32(supported_capacities, "supported_capacities")
+            caps = supported_capacities.contiguous()
+            n_caps = caps.size(0)
+        if capacity_padding and n_caps < 1:  # CHECK_GE, location.cu:350,365
+            raise RuntimeError("capacity_padding requires at least one supported capacity")
+        hot_mask = hot_mask.contiguous()
+        # seat mode writes every element; the tag list is sparse and starts from zeros
+        indices = torch.zeros_like(hot_mask) if is_tag_index else torch.empty_like(hot_mask)
+        loads_and_counts = torch.empty((2, E), dtype=torch.int32, device=hot_mask.device)
+        loads, counts = loads_and_counts[0], loads_and_counts[1]
+        ws = _scan_workspace(hot_mask.device, T, E)
+        _lib.check(_lib.lib().brt_hip_generate_indices_and_loads(
+            _ptr(hot_mask), _ptr(indices), _ptr(loads), _ptr(counts), T, E, _ptr(caps), n_caps,
+            int(capacity_padding), int(path_wise_padding), int(is_tag_index),
+            _ptr(ws), ws.numel(), _stream()))
+        if not is_tag_index:
+            loads._brt_pairing = _Pairing(indices, loads, counts)
+    return indices, loads
+
+
+def convert_index_format(
+    origin_indices: torch.Tensor, loads: torch.Tensor, is_to_tag: bool
+) -> torch.Tensor:
+    """router.cc:90-110.
+
+    As built, the reference forwards ``is_to_tag`` into the launcher's
+    ``tag_to_seat`` parameter (router.cc:104-107 vs location.cu:317-333), so
+    ``is_to_tag=True`` runs the tag->seat kernel.  This entry point keeps that
+    behaviour; use :func:`seat_to_tag_indices` / :func:`tag_to_seat_indices` for
+    the direction their names say.
+    """
+    return _convert(origin_indices, loads, tag_to_seat=bool(is_to_tag))
+
+
+def seat_to_tag_indices(seat_indices: torch.Tensor, loads: torch.Tensor) -> torch.Tensor:
+    return _convert(seat_indices, loads, tag_to_seat=False)
+
+
+def tag_to_seat_indices(tag_indices: torch.Tensor, loads: torch.Tensor) -> torch.Tensor:
+    return _convert(tag_indices, loads, tag_to_seat=True)
+
+
+def _convert(origin_indices, loads, tag_to_seat: bool) -> torch.Tensor:
+    _check_on_device(origin_indices, "origin_indices")
+    _check_int32(origin_indices, "origin_indices")
+    origin_indices = origin_indices.contiguous()
+    T, E = origin_indices.shape
+    with torch.cuda.device(origin_indices.device):
+        dev_loads = loads
+        if tag_to_seat:
+            _check_int32(loads, "loads")
+            dev_loads = loads.to(origin_indices.device, non_blocking=True).contiguous()
+        new_indices = torch.zeros_like(origin_indices)
+        _lib.check(_lib.lib().brt_hip_convert_index_format(
+            _ptr(origin_indices), _ptr(new_indices), _ptr(dev_loads) if tag_to_seat else None,
+            T, E, int(tag_to_seat), _stream()))
+    return new_indices
+
+
+def dispatch_with_indices_and_loads(
+    in_data: torch.Tensor,
+    route_indices: torch.Tensor,
+    loads: torch.Tensor,
+    gates: Optional[torch.Tensor] = None,
+    tag_generating: bool = False,
+    tags: Optional[torch.Tensor] = None,
+    max_path_padding: bool = False,
+    max_path_load: int = 0,
+    is_1d_routing: bool = True,
+    is_tag_index: bool = False,
+) -> List[torch.Tensor]:
+    """router.cc:131-273.  Returns ``[out]`` or ``[out, new_tags]``."""
+    _check_on_device(in_data, "in_data")
+    _check_on_device(route_indices, "route_indices")
+    _check_int32(route_indices, "route_indices")
+    device = in_data.device
+    T = in_data.size(0)
+    E = route_indices.size(1)
+    with torch.cuda.device(device):
+        if T == 0:  # router.cc:150-168
+            shape = list(in_data.shape)
+            if is_1d_routing:
+                shape[0] = 0
+            else:
+                if len(shape) == 2:
+                    shape.append(1)
+                shape[1] = 0
+                shape = shape[1:]
+            out = torch.zeros(shape, dtype=in_data.dtype, device=device)
+            if tag_generating:
+                return [out, torch.zeros((0,), dtype=route_indices.dtype, device=device)]
+            return [out]
+        if in_data.dtype not in _DT:  # TORCH_CHECK_NOT_IMPLEMENTED, router.cc:266
+            raise NotImplementedError("data type is not supported")
+        dtype = _DT[in_data.dtype]
+        cell = in_data.numel() // T
+        if not is_1d_routing:
+            cell //= E
+
+        counts = None if is_tag_index else _paired_counts(route_indices, loads)
+        _check_int32(loads, "loads")
+        dev_loads = loads if loads.is_cuda else loads.to(device, non_blocking=True)
+
+        # rows of the dispatched buffer (router.cc:189-202); data dependent, so one
+        # host read of the loads unless a fixed per-path stride was given
+        mpl = 0
+        if max_path_padding:
+            mpl = int(max_path_load) if max_path_load > 0 else int(loads.max().item())
+            total = mpl * E
+        else:
+            total = int(loads.sum().item())
+
+        in_data = in_data.contiguous()
+        route_indices = route_indices.contiguous()
+        shape = list(in_data.shape)
+        if is_1d_routing:
+            shape[0] = total
+        else:
+            if len(shape) == 2:
+                shape.append(1)
+            shape[1] = total
+            shape = shape[1:]
+        alloc = torch.empty if counts is not None else torch.zeros
+        out = alloc(shape, dtype=in_data.dtype, device=device)
+
+        dev_gates = None
+        if gates is not None:
+            if not is_1d_routing:
+                raise RuntimeError("gates are only supported with 1-d routing")  # route.cu:362
+            _check_on_device(gates, "gates")
+            if gates.dtype != in_data.dtype:  # CHECK_EQ, router.cc:226
+                raise RuntimeError("gates must have the dtype of in_data")
+            dev_gates = gates.contiguous()
+
+        old_tags = new_tags = None
+        if tag_generating:
+            if tags is not None:
+                _check_on_device(tags, "tags")
+                if tags.dtype != route_indices.dtype:
+                    raise RuntimeError("tags must have the dtype of route_indices")
+                old_tags = tags.contiguous()
+            # old_tags None = arange(1, T+1) (router.cc:240-241), generated in the kernel
+            new_tags = alloc((total,), dtype=route_indices.dtype, device=device)
+
+        _lib.check(_lib.lib().brt_hip_dispatch(
+            _ptr(in_data), _ptr(out), _ptr(dev_gates), _ptr(route_indices), _ptr(dev_loads),
+            _ptr(counts), _ptr(old_tags), _ptr(new_tags), T, cell, E, total, mpl,
+            int(is_1d_routing), int(is_tag_index), dtype, _stream()))
+    if tag_generating:
+        return [out, new_tags]
+    return [out]
+
+
+def split_fused_cells_to_paths(
+    in_data: torch.Tensor,
+    loads: torch.Tensor,
+    max_path_padding: bool = False,
+    is_load_split: bool = False,
+    is_tag_split: bool = False,
+    tags: Optional[torch.Tensor] = None,
+) -> List[List[torch.Tensor]]:
+    """router.cc:285-335: per-path views (``narrow``) of the fused buffer."""
+    path_num = loads.numel()
+    if is_tag_split:
+        is_load_split = True
+        if tags is None:
+            raise RuntimeError("is_tag_split needs tags")
+    datas, load_list, tag_list = [], [], []
+    if max_path_padding:
+        stride = in_data.size(0) // path_num
+        bounds = [(i * stride, stride) for i in range(path_num)]
+    else:
+        host_loads = loads.cpu().tolist()
+        bounds, start = [], 0
+        for load in host_loads:
+            bounds.append((start, load))
+            start += load
+    for i, (start, length) in enumerate(bounds):
+        datas.append(in_data.narrow(0, start, length))
+        if is_load_split:
+            load_list.append(loads.narrow(0, i, 1))
+        if is_tag_split:
+            tag_list.append(tags.narrow(0, start, length))
+    if is_tag_split:
+        return [datas, load_list, tag_list]
+    if is_load_split:
+        return [datas, load_list]
+    return [datas]
+
+
+def fuse_split_cells_from_paths(
+    in_data: List[torch.Tensor],
+    is_load_fuse: bool = False,
+    is_tag_fuse: bool = False,
+    loads: Optional[List[torch.Tensor]] = None,
+    tags: Optional[List[torch.Tensor]] = None,
+) -> List[torch.Tensor]:
+    """router.cc:348-369."""
+    out_data = torch.cat(in_data, 0)
+    if is_load_fuse:
+        if loads is None:
+            raise RuntimeError("is_load_fuse needs loads")
+        return [out_data, torch.cat(loads, 0)]
+    if is_tag_fuse:
+        if tags is None:
+            raise RuntimeError("is_tag_fuse needs tags")
+        out_tags = torch.cat(tags, 0)
+        new_tags, global_seat_indices = torch.unique(out_tags, sorted=True, return_inverse=True)
+        return [out_data, new_tags, global_seat_indices]
+    return [out_data]
+
+
+def combine_with_indices_and_loads(
+    in_data: torch.Tensor,
+    route_indices: torch.Tensor,
+    loads: Optional[torch.Tensor] = None,
+    gates: Optional[torch.Tensor] = None,
+    out_data: Optional[torch.Tensor] = None,
+    max_path_padding: bool = False,
+    ever_padded: bool = True,
+    is_tag_index: bool = False,
+    tags: Optional[torch.Tensor] = None,
+    *,
+    out_dtype: Optional[torch.dtype] = None,
+) -> List[torch.Tensor]:
+    """router.cc:372-473.
+
+    Seat mode runs the HIP gather kernel (fp32 accumulation in ascending path
+    order).  ``out_dtype`` (keyword only, not in the reference) selects an fp32
+    result for 16-bit inputs; with ``out_data`` the result dtype is that of
+    ``out_data``.  Tag mode is the reference's ``scatter_reduce`` formulation.
+    """
+    _check_on_device(in_data, "in_data")
+    _check_on_device(route_indices, "route_indices")
+    device = in_data.device
+    T = route_indices.size(0)
+    with torch.cuda.device(device):
+        if T == 0:  # router.cc:386-397
+            if not is_tag_index:
+                return [out_data if out_data is not None else torch.empty_like(in_data)]
+            return [torch.empty_like(in_data), torch.empty_like(tags), torch.zeros_like(tags)]
+        if T == 1:  # router.cc:402-412
+            if not is_tag_index:
+                return [out_data + in_data if out_data is not None else in_data]
+            return [in_data, tags, torch.ones_like(tags)]
+
+        if is_tag_index:
+            return _combine_with_tags(in_data, route_indices, out_data, ever_padded, tags)
+
+        if loads is None:
+            raise RuntimeError("seat-index combine needs loads")
+        _check_int32(route_indices, "route_indices")
+        _check_int32(loads, "loads")
+        if in_data.dtype not in _DT:
+            raise NotImplementedError("data type is not supported")
+        E = route_indices.size(1)
+        dev_loads = loads.to(device, non_blocking=True).contiguous()
+        in_data = in_data.contiguous()
+        route_indices = route_indices.contiguous()
+        P = in_data.size(0)
+        cell = in_data.numel() // P if P > 0 else 0
+        mpl = P // E if max_path_padding else 0  # router.cc:427-430
+        dev_gates = None
+        gate_dtype = _lib.F32
+        if gates is not None:
+            _check_on_device(gates, "gates")
+            if gates.dtype not in _DT:
+                raise NotImplementedError("gate data type is not supported")
+            dev_gates = gates.contiguous()
+            gate_dtype = _DT[gates.dtype]
+        if out_data is not None:
+            _check_on_device(out_data, "out_data")
+            if not out_data.is_contiguous():
+                raise RuntimeError("out_data must be contiguous (it is updated in place)")
+            result = out_data
+            residual = 1
+        else:
+            shape = list(in_data.shape)
+            shape[0] = T
+            result = torch.empty(shape, dtype=out_dtype or in_data.dtype, device=device)
+            residual = 0
+        if result.dtype not in _DT or result.numel() != T * cell:
+            raise RuntimeError("out_data does not match [cell_num, *cell_shape]")
+        _lib.check(_lib.lib().brt_hip_combine(
+            _ptr(in_data), _ptr(result), _ptr(dev_gates), _ptr(route_indices), _ptr(dev_loads),
+            T, cell, E, P, mpl, residual, _DT[in_data.dtype], _DT[result.dtype], gate_dtype,
+            _stream()))
+        return [result]
+
+
+def _combine_with_tags(in_data, route_indices, out_data, ever_padded, tags):
+    # router.cc:449-472
+    if tags is None:
+        raise RuntimeError("tag-index combine needs tags")
+    cell = in_data.numel() // in_data.size(0)
+    index = route_indices.view(-1, 1).repeat(1, cell).view_as(in_data)
+    tags_value = tags
+    n = tags_value.size(0)
+    if out_data is not None:
+        _check_on_device(out_data, "out_data")
+        if out_data.size(0) != n:
+            raise RuntimeError("out_data must hold one row per unique tag")
+        result = out_data
+        # out-of-place and discarded, as in the reference (router.cc:456)
+        torch.scatter_reduce(result, 0, index, in_data, "sum", include_self=False)
+    else:
+        shape = list(in_data.shape)
+        shape[0] = n
+        result = torch.zeros(shape, dtype=in_data.dtype, device=in_data.device)
+        result = torch.scatter_reduce(result, 0, index, in_data, "sum")
+        if ever_padded and int(tags_value[0].item()) == 0:
+            result = result.narrow(0, 1, n - 1)
+            tags_value = tags_value.narrow(0, 1, n - 1)
+    out_loads = torch.tensor([tags_value.numel()], dtype=torch.int32, device=in_data.device)
+    return [result, tags_value, out_loads]
+
+
+# legacy name (sample/cpp/router.ipynb:258-266) of the seat-index combine
+combine_with_src_indices = combine_with_indices_and_loads

@@ -1,0 +1,90 @@
+// Shared host/device helpers for libbrt_hip.so (gfx950, wave64).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "brt_hip.h"
+
+namespace brt {
+
+// ---- host side: per-thread error text -------------------------------------
+int fail(int code, const char* fmt, ...);  // records the message, returns code
+int check_launch(const char* what);        // hipGetLastError -> BRT_E_LAUNCH
+
+inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
+inline bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+
+// ---- device side ------------------------------------------------------------
+constexpr int kWave = 64;
+
+__device__ __forceinline__ int lane_id() { return threadIdx.x & (kWave - 1); }
+
+// Inclusive prefix sum across the 64 lanes of a wavefront.
+__device__ __forceinline__ int wave_inclusive_scan(int v) {
+  const int lane = lane_id();
+#pragma unroll
+  for (int d = 1; d < kWave; d <<= 1) {
+    int n = __shfl_up(v, d, kWave);
+    if (lane >= d) v += n;
+  }
+  return v;
+}
+
+// bf16 <-> fp32 (round to nearest even; NaN stays NaN).
+__device__ __forceinline__ float bf16_to_float(uint32_t h) { return __uint_as_float(h << 16); }
+__device__ __forceinline__ uint32_t float_to_bf16(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x0040u;
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return u >> 16;
+}
+__device__ __forceinline__ float f16_to_float(uint32_t h) {
+  union { uint16_t u; _Float16 f; } c;
+  c.u = static_cast<uint16_t>(h);
+  return static_cast<float>(c.f);
+}
+__device__ __forceinline__ uint32_t float_to_f16(float f) {
+  union { uint16_t u; _Float16 f; } c;
+  c.f = static_cast<_Float16>(f);
+  return c.u;
+}
+
+template <int DT>
+__device__ __forceinline__ float half_bits_to_float(uint32_t h) {
+  return DT == BRT_F16 ? f16_to_float(h) : bf16_to_float(h);
+}
+template <int DT>
+__device__ __forceinline__ uint32_t float_to_half_bits(float f) {
+  return DT == BRT_F16 ? float_to_f16(f) : float_to_bf16(f);
+}
+
+// Scalar load of one gate value of a runtime dtype.
+__device__ __forceinline__ float load_gate(const void* gates, int dtype, size_t i) {
+  if (dtype == BRT_F32) return static_cast<const float*>(gates)[i];
+  uint32_t h = static_cast<const uint16_t*>(gates)[i];
+  return dtype == BRT_F16 ? f16_to_float(h) : bf16_to_float(h);
+}
+
+// Fills s_val[e] = g[e] and s_start[e] = exclusive prefix of g (or e*stride when
+// stride != 0) for e < E, using the first wavefront of the block.  The caller
+// must __syncthreads() afterwards.
+__device__ __forceinline__ void load_and_scan_paths(const int* __restrict__ g, int* s_val,
+                                                    int* s_start, int E, int stride) {
+  if (threadIdx.x < kWave) {
+    const int lane = threadIdx.x;
+    int carry = 0;
+    for (int base = 0; base < E; base += kWave) {
+      const int e = base + lane;
+      const int v = e < E ? g[e] : 0;
+      const int incl = wave_inclusive_scan(v);
+      if (e < E) {
+        s_val[e] = v;
+        s_start[e] = stride != 0 ? e * stride : carry + incl - v;
+      }
+      carry += __shfl(incl, kWave - 1, kWave);
+    }
+  }
+}
+
+}  // namespace brt

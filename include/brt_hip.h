@@ -1,0 +1,170 @@
+/*
+ * libbrt_hip.so -- C ABI of the MI355X (gfx950) MoE routing hot path.
+ *
+ * Each entry point replaces one raw-pointer launcher of the reference's native
+ * layer (paths relative to the reference tree); the reference-side binding
+ * that would call it is the torch extension src/backend/torch/router.cc.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless stated otherwise; `stream` is a
+ *     hipStream_t passed as void* (NULL = the null stream);
+ *   - index tensors are int32 row-major [T,E], values 1-based, 0 = not routed;
+ *   - entry points return 0 on success and a negative BRT_E_* code otherwise
+ *     (brt_hip_last_error() gives the message of the calling thread's last
+ *     failure); they never throw, never allocate device memory, never
+ *     synchronise the stream, and only enqueue work on `stream`;
+ *   - the caller owns every buffer, including workspaces.
+ */
+#ifndef BRT_HIP_H_
+#define BRT_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+  BRT_OK = 0,
+  BRT_E_INVALID = -1,     /* bad argument (shape, flag combination, null pointer) */
+  BRT_E_WORKSPACE = -2,   /* workspace missing or too small */
+  BRT_E_LAUNCH = -3,      /* HIP reported a launch error */
+  BRT_E_UNSUPPORTED = -4  /* dtype / layout not implemented */
+};
+
+enum { BRT_F32 = 0, BRT_F16 = 1, BRT_BF16 = 2 };
+
+/* activation fused into the grouped GEMM epilogue */
+enum { BRT_ACT_NONE = 0, BRT_ACT_GELU = 1, BRT_ACT_RELU = 2 };
+
+/* Message of this thread's most recent failing call ("" if none). */
+const char* brt_hip_last_error(void);
+
+/* Library version, "major.minor". */
+const char* brt_hip_version(void);
+
+/*
+ * Bytes of scan workspace needed by brt_hip_generate_indices_and_loads /
+ * brt_hip_throttle_hotmask for a [T,E] mask.  The workspace must be
+ * zero-filled ONCE after allocation; the kernels leave it reusable (records
+ * are stamped with a launch epoch kept inside the workspace).  One workspace
+ * must not be used by two calls that can run concurrently (two streams).
+ */
+size_t brt_hip_scan_workspace_bytes(int T, int E);
+
+/*
+ * Replaces router::GenerateIndicesAndLoads (include/brt/router/location.h:28-38,
+ * src/router/location.cu:212-257,335-379).
+ *
+ *   mask     [T,E] int32 hot mask
+ *   indices  [T,E] int32 out.  Seat mode (is_tag_index=0): every element is
+ *            written (cumsum(mask,0)*mask), no pre-zeroing needed.  Tag mode:
+ *            must be zero-filled by the caller; slot [s-1,e] receives row+1 of
+ *            the s-th routed row of column e.
+ *   loads    [E] int32 out, after the capacity rules of location.cu:222-256
+ *   counts   [E] int32 out or NULL: the un-clipped, un-padded per-path counts
+ *            (sum(mask,0)); brt_hip_dispatch uses them to zero-fill padding rows
+ *   caps     [C] int32 ascending supported capacities or NULL (C=0)
+ *   capacity_padding requires C>=1; path_wise_padding is honoured only together
+ *   with capacity_padding and requires C>=E (location.cu:349-358,227-230).
+ *   T==0 writes loads=counts=0.
+ */
+int brt_hip_generate_indices_and_loads(const int32_t* mask, int32_t* indices, int32_t* loads,
+                                       int32_t* counts, int T, int E, const int32_t* caps, int C,
+                                       int capacity_padding, int path_wise_padding,
+                                       int is_tag_index, void* workspace, size_t workspace_bytes,
+                                       void* stream);
+
+/*
+ * Replaces router::ThrottleHotmask (location.h:13-19, location.cu:59-130,304-315).
+ *   out[t,e] = 1 iff mask[t,e]==1 and prefix[e] + cumsum(mask)[t,e] <= threshold[e]
+ *   prefix[e] <- min(prefix[e] + sum(mask[:,e]), threshold[e])   (in place)
+ * `out` is fully written (no pre-zeroing needed).  T==0 leaves prefix untouched.
+ */
+int brt_hip_throttle_hotmask(const int32_t* mask, int32_t* out, int32_t* prefix,
+                             const int32_t* threshold, int T, int E, void* workspace,
+                             size_t workspace_bytes, void* stream);
+
+/*
+ * Replaces router::ConvertIndexFormat (location.h:21-27, location.cu:259-302,317-333).
+ *   tag_to_seat=0: dst[src[t,e]-1, e] = t+1 for src[t,e] != 0
+ *   tag_to_seat=1: dst[src[s,e]-1, e] = s+1 for s < loads[e], under the
+ *                  reference's stop rule (slot s is converted iff the tags at
+ *                  s, s-1024, s-2048, ... are all non-zero)
+ * `dst` must be zero-filled by the caller.  `loads` is only read when
+ * tag_to_seat=1.
+ */
+int brt_hip_convert_index_format(const int32_t* src, int32_t* dst, const int32_t* loads, int T,
+                                 int E, int tag_to_seat, void* stream);
+
+/*
+ * Replaces router::DispatchWithIndicesAndLoads<dtype> (include/brt/router/route.h:14-28,
+ * src/router/route.cu:13-206,284-465).
+ *
+ *   src       1-d routing: [T, cell]; 2-d routing: [T, E, cell] (path e reads
+ *             src[:, e, :]; no transposed copy is needed)
+ *   dst       [P, cell]
+ *   gates     [T,E] in `dtype`, or NULL (unweighted); 1-d routing only
+ *   indices   [T,E] seat indices (is_tag_index=0) or tag lists (is_tag_index=1)
+ *   loads     [E]
+ *   counts    [E] or NULL.  Non-NULL (seat mode only): the routed rows of path e
+ *             are exactly seats 1..min(counts[e],loads[e]); the kernel then
+ *             writes every row of dst (data rows, and zeros for the padding
+ *             rows) and dst/new_tags need no pre-zeroing.  NULL: dst and
+ *             new_tags must be zero-filled by the caller (the reference's
+ *             contract, router.cc:219,246).
+ *   old_tags  [T] or NULL; new_tags [P] or NULL.  new_tags non-NULL enables tag
+ *             generation: new_tags[row] = old_tags ? old_tags[t] : t+1.
+ *   cell      elements per row, in units of `dtype`
+ *   P         rows of dst (rows >= P are never written)
+ *   max_path_load  0 = paths packed back to back (start[e] = sum(loads[:e]));
+ *             otherwise start[e] = e*max_path_load
+ *   Weighted rows are src*gate rounded once to `dtype`; unweighted rows are
+ *   byte copies.
+ */
+int brt_hip_dispatch(const void* src, void* dst, const void* gates, const int32_t* indices,
+                     const int32_t* loads, const int32_t* counts, const int32_t* old_tags,
+                     int32_t* new_tags, int T, int cell, int E, int P, int max_path_load,
+                     int is_1d_routing, int is_tag_index, int dtype, void* stream);
+
+/*
+ * Replaces router::CombineWithIndicesAndLoads<dtype>, seat-index mode
+ * (route.h:30-44, route.cu:208-282,467-518).
+ *
+ *   src [P, cell] in in_dtype; dst [T, cell] in out_dtype; gates [T,E] in
+ *   gate_dtype or NULL.
+ *   dst[t] = sum over e ascending with 1 <= indices[t,e] <= loads[e] of
+ *            src[start[e]+indices[t,e]-1] (* gates[t,e]),
+ *   each product rounded to fp32, accumulated in fp32 in that order from 0, and
+ *   rounded once to out_dtype.  is_residual=0: tokens without a valid route get
+ *   a zero row (dst needs no pre-zeroing).  is_residual=1: such rows of dst are
+ *   left untouched, rows of routed tokens are overwritten.
+ */
+int brt_hip_combine(const void* src, void* dst, const void* gates, const int32_t* indices,
+                    const int32_t* loads, int T, int cell, int E, int P, int max_path_load,
+                    int is_residual, int in_dtype, int out_dtype, int gate_dtype, void* stream);
+
+/*
+ * Replaces the homo-fused expert kernel launch jit::CUDACompiler::HomoExecute
+ * (src/jit/compiler.cu:151-246, binding src/backend/torch/jit.cc:54-75) for
+ * Linear branches (python/brt/jit/modules/linear.py:15-61):
+ *
+ *   out[start[e] : start[e]+loads[e], :] =
+ *        act( x[start[e] : start[e]+loads[e], :] @ W_e^T + b_e ),  start[e] = sum(loads[:e])
+ *
+ *   x [P,K], out [P,N] bf16 row-major; `weights` is a device array of E
+ *   pointers to W_e [N,K] bf16 row-major (torch Linear layout); `biases` is a
+ *   device array of E pointers to b_e [N] bf16, or NULL; `loads` [E] int32 is
+ *   read on the device (no host copy, any non-negative values, sum <= P).
+ *   One launch covers all experts; accumulation is fp32 on the bf16 MFMA units.
+ *   K must be a multiple of 32 and N a multiple of 16.
+ */
+int brt_hip_grouped_gemm(const void* x, const void* const* weights, const void* const* biases,
+                         void* out, const int32_t* loads, int E, int P, int K, int N, int act,
+                         void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BRT_HIP_H_ */

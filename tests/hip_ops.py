@@ -1,0 +1,159 @@
+"""Thin test-side callers of the C ABI (include/brt_hip.h) on torch device memory.
+
+numpy in, numpy out: inputs are uploaded, the entry point is called through
+ctypes exactly as a foreign binding would, outputs are downloaded.  16-bit data
+travel as uint16 bit patterns like in the oracle.
+"""
+import numpy as np
+import torch
+
+from brainstorm_amd import _lib
+
+DT = {"f32": _lib.F32, "f16": _lib.F16, "bf16": _lib.BF16}
+_TORCH_BITS = {"f32": torch.float32, "f16": torch.int16, "bf16": torch.int16}
+
+
+def dev(a, dtype=None):
+    if a is None:
+        return None
+    a = np.ascontiguousarray(a)
+    if a.dtype == np.uint16:
+        a = a.view(np.int16)
+    return torch.from_numpy(a).cuda()
+
+
+def host(t, bits16=False):
+    a = t.cpu().numpy()
+    if bits16 and a.dtype == np.int16:
+        a = a.view(np.uint16)
+    return a
+
+
+def ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+_ws = {}
+
+
+def workspace(T, E):
+    need = _lib.lib().brt_hip_scan_workspace_bytes(T, E)
+    ws = _ws.get("ws")
+    if ws is None or ws.numel() < need:
+        ws = torch.zeros(max(need, 1 << 20), dtype=torch.uint8, device="cuda")
+        _ws["ws"] = ws
+    return ws
+
+
+def generate_indices_and_loads(mask, caps=None, capacity_padding=False, path_wise_padding=False,
+                               is_tag_index=False, want_counts=False, misalign=False):
+    mask = np.ascontiguousarray(mask, dtype=np.int32)
+    T, E = mask.shape
+    if misalign:  # 4-byte aligned views: exercises the non-vector tile copy
+        buf = torch.zeros(T * E + 1, dtype=torch.int32, device="cuda")
+        d_mask = buf[1:].view(T, E)
+        d_mask.copy_(torch.from_numpy(mask))
+        obuf = torch.full((T * E + 1,), -7, dtype=torch.int32, device="cuda")
+        d_idx = obuf[1:].view(T, E)
+        if is_tag_index:
+            d_idx.zero_()
+    else:
+        d_mask = dev(mask)
+        d_idx = (torch.zeros if is_tag_index else torch.empty)((T, E), dtype=torch.int32, device="cuda")
+        if not is_tag_index:
+            d_idx.fill_(-7)  # poison: seat mode must overwrite everything
+    d_loads = torch.full((E,), -1, dtype=torch.int32, device="cuda")
+    d_counts = torch.full((E,), -1, dtype=torch.int32, device="cuda") if want_counts else None
+    d_caps = None if caps is None else dev(np.asarray(caps, dtype=np.int32))
+    ws = workspace(T, E)
+    _lib.check(_lib.lib().brt_hip_generate_indices_and_loads(
+        ptr(d_mask), ptr(d_idx), ptr(d_loads), ptr(d_counts), T, E, ptr(d_caps),
+        0 if caps is None else len(caps), int(capacity_padding), int(path_wise_padding),
+        int(is_tag_index), ptr(ws), ws.numel(), stream()))
+    torch.cuda.synchronize()
+    assert int(ws[64 * 8:64 * 8 + 8].view(torch.int64).item()) == 0, "look-back spin bound hit"
+    out = (host(d_idx), host(d_loads))
+    if want_counts:
+        out = out + (host(d_counts),)
+    return out
+
+
+def throttle_hotmask(mask, prefix, threshold):
+    mask = np.ascontiguousarray(mask, dtype=np.int32)
+    T, E = mask.shape
+    d_mask = dev(mask)
+    d_out = torch.full((T, E), -7, dtype=torch.int32, device="cuda")
+    d_prefix = dev(np.asarray(prefix, dtype=np.int32))
+    d_thr = dev(np.asarray(threshold, dtype=np.int32))
+    ws = workspace(T, E)
+    _lib.check(_lib.lib().brt_hip_throttle_hotmask(
+        ptr(d_mask), ptr(d_out), ptr(d_prefix), ptr(d_thr), T, E, ptr(ws), ws.numel(), stream()))
+    torch.cuda.synchronize()
+    return host(d_out), host(d_prefix)
+
+
+def convert_index_format(indices, loads, tag_to_seat):
+    indices = np.ascontiguousarray(indices, dtype=np.int32)
+    T, E = indices.shape
+    d_src = dev(indices)
+    d_dst = torch.zeros((T, E), dtype=torch.int32, device="cuda")
+    d_loads = dev(np.asarray(loads, dtype=np.int32))
+    _lib.check(_lib.lib().brt_hip_convert_index_format(
+        ptr(d_src), ptr(d_dst), ptr(d_loads), T, E, int(tag_to_seat), stream()))
+    torch.cuda.synchronize()
+    return host(d_dst)
+
+
+def dispatch(x_bits, idx, loads, gates_bits=None, counts=None, tag_generating=False, tags=None,
+             max_path_load=0, P=None, is_1d=True, is_tag_index=False, dtype="f32"):
+    idx = np.ascontiguousarray(idx, dtype=np.int32)
+    T, E = idx.shape
+    loads = np.asarray(loads, dtype=np.int32)
+    x_bits = np.ascontiguousarray(x_bits)
+    cell = x_bits.size // max(T, 1) // (1 if is_1d else E)
+    if P is None:
+        P = E * max_path_load if max_path_load else int(loads.sum())
+    d_x = dev(x_bits.reshape(T, -1))
+    prezero = counts is None
+    poison = 0 if prezero else 0x55
+    d_out = torch.full((P, cell), poison, dtype=_TORCH_BITS[dtype], device="cuda") if dtype != "f32" \
+        else (torch.zeros((P, cell), device="cuda") if prezero else torch.full((P, cell), float("nan"), device="cuda"))
+    d_new = None
+    if tag_generating:
+        d_new = torch.full((P,), 0 if prezero else -9, dtype=torch.int32, device="cuda")
+    d_old = None if tags is None else dev(np.asarray(tags, dtype=np.int32))
+    _lib.check(_lib.lib().brt_hip_dispatch(
+        ptr(d_x), ptr(d_out), ptr(dev(gates_bits)), ptr(dev(idx)), ptr(dev(loads)),
+        ptr(None if counts is None else dev(np.asarray(counts, dtype=np.int32))),
+        ptr(d_old), ptr(d_new), T, cell, E, P, max_path_load, int(is_1d), int(is_tag_index),
+        DT[dtype], stream()))
+    torch.cuda.synchronize()
+    return host(d_out, True), (None if d_new is None else host(d_new))
+
+
+def combine(y_bits, idx, loads, gates_bits=None, residual_bits=None, max_path_load=0,
+            in_dtype="f32", out_dtype=None, gate_dtype=None):
+    out_dtype = out_dtype or in_dtype
+    gate_dtype = gate_dtype or in_dtype
+    idx = np.ascontiguousarray(idx, dtype=np.int32)
+    T, E = idx.shape
+    y_bits = np.ascontiguousarray(y_bits)
+    P = y_bits.shape[0]
+    cell = y_bits.size // max(P, 1)
+    d_y = dev(y_bits.reshape(P, -1))
+    if residual_bits is not None:
+        d_out = dev(np.ascontiguousarray(residual_bits).reshape(T, -1)).clone()
+    elif out_dtype == "f32":
+        d_out = torch.full((T, cell), float("nan"), device="cuda")
+    else:
+        d_out = torch.full((T, cell), 0x55, dtype=torch.int16, device="cuda")
+    _lib.check(_lib.lib().brt_hip_combine(
+        ptr(d_y), ptr(d_out), ptr(dev(gates_bits)), ptr(dev(idx)),
+        ptr(dev(np.asarray(loads, dtype=np.int32))), T, cell, E, P, max_path_load,
+        int(residual_bits is not None), DT[in_dtype], DT[out_dtype], DT[gate_dtype], stream()))
+    torch.cuda.synchronize()
+    return host(d_out, True)

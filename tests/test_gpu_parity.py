@@ -1,0 +1,350 @@
+"""GPU parity: HIP kernels (called through the C ABI) against the CPU oracle on the
+same seeded inputs.  Integer / byte / index results must be bit-exact; the
+floating-point combine is compared bit-exactly too (fixed summation order) and
+additionally against an fp64 evaluation within 1e-6 (fp32) / 1e-2 (16-bit).
+"""
+import json
+import os
+
+import numpy as np
+import pytest
+
+import oracle
+from routing_cases import as_dtype_bits, bernoulli_mask, bits_to_f32, softmax, topk_mask, zipf_bias
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "notebook_vectors.json")))
+
+
+@pytest.fixture(scope="module")
+def hip():
+    import hip_ops
+
+    return hip_ops
+
+
+def same_bits(a, b):
+    a, b = np.ascontiguousarray(a), np.ascontiguousarray(b)
+    return a.shape == b.shape and np.array_equal(a.view(np.uint8), b.view(np.uint8))
+
+
+# ------------------------------------------------------------ indices / loads
+def test_notebook_vectors(hip):
+    g = GOLDEN["generate_indices"]
+    idx, loads = hip.generate_indices_and_loads(g["mask"])
+    assert np.array_equal(idx, np.array(g["seat_indices"], dtype=np.int32))
+    assert loads.tolist() == g["loads"]
+    t = GOLDEN["throttle"]
+    out, prefix = hip.throttle_hotmask(t["mask"], t["prefix"], t["threshold"])
+    assert np.array_equal(out, np.array(t["throttled"], dtype=np.int32))
+    assert prefix.tolist() == t["new_prefix"]
+
+
+INDEX_SHAPES = [
+    (1, 1, 1), (1, 3, 1), (5, 2, 1), (37, 7, 3), (1023, 16, 1), (1024, 16, 4), (4096, 16, 1),
+    (4096, 8, 4), (8192, 64, 1), (16384, 32, 2), (3000, 100, 5), (2500, 128, 2), (700, 300, 3),
+    (333, 257, 1), (100352, 8, 1), (20000, 3, 1), (50000, 1, 1),
+]
+
+
+@pytest.mark.parametrize("T,E,k", INDEX_SHAPES)
+def test_seat_and_tag_indices_bit_exact(hip, T, E, k):
+    mask, _ = topk_mask(T, E, k, seed=T * 7 + E)
+    for tag in (False, True):
+        want_idx, want_loads = oracle.generate_indices_and_loads(mask, is_tag_index=tag)
+        for _ in range(2):  # second launch reuses the workspace (next epoch)
+            idx, loads, counts = hip.generate_indices_and_loads(mask, is_tag_index=tag, want_counts=True)
+            assert np.array_equal(idx, want_idx), f"indices differ T={T} E={E} tag={tag}"
+            assert np.array_equal(loads, want_loads)
+            assert np.array_equal(counts, mask.sum(0))
+
+
+def test_indices_general_mask_values_and_misaligned_buffers(hip):
+    mask = bernoulli_mask(2049, 12, 0.4, seed=5)
+    mask[::7, 3] = 2  # the scan sums mask values and multiplies by them (location.cu:177-178)
+    want = oracle.generate_indices_and_loads(mask)
+    got = hip.generate_indices_and_loads(mask)
+    assert np.array_equal(got[0], want[0]) and np.array_equal(got[1], want[1])
+    mask = bernoulli_mask(3001, 10, 0.2, seed=6)
+    for tag in (False, True):
+        want = oracle.generate_indices_and_loads(mask, is_tag_index=tag)
+        got = hip.generate_indices_and_loads(mask, is_tag_index=tag, misalign=True)
+        assert np.array_equal(got[0], want[0]) and np.array_equal(got[1], want[1])
+
+
+@pytest.mark.parametrize("tag", [False, True])
+def test_capacity_rules_bit_exact(hip, tag):
+    caps = [1, 2, 4, 8, 16, 32, 64, 128, 256, 512]
+    cases = [
+        (topk_mask(4096, 8, 4, seed=7)[0], caps, False, False),
+        (topk_mask(4096, 8, 4, seed=7)[0], caps, True, False),
+        (topk_mask(512, 8, 1, seed=8)[0], caps, True, False),
+        (topk_mask(256, 8, 4, seed=9)[0], [2, 4, 8, 16, 32, 64, 128, 256], True, True),
+        (topk_mask(1024, 16, 1, seed=1)[0], [64], False, False),
+        (topk_mask(8192, 64, 1, seed=2)[0], [160], True, False),
+    ]
+    empty = topk_mask(300, 6, 1, seed=3)[0]
+    empty[:, 2] = 0
+    cases.append((empty, [50, 100], True, False))
+    cases.append((empty, [5, 6, 7, 8, 9, 10], True, True))
+    cases.append((empty, [5, 6, 7, 8, 9, 10], False, True))
+    for mask, c, pad, pw in cases:
+        want = oracle.generate_indices_and_loads(mask, c, pad, pw, tag)
+        got = hip.generate_indices_and_loads(mask, c, pad, pw, tag)
+        assert np.array_equal(got[0], want[0]) and np.array_equal(got[1], want[1])
+
+
+def test_index_generation_rejects_bad_arguments(hip):
+    from brainstorm_amd import _lib
+
+    mask = topk_mask(16, 4, 1, seed=0)[0]
+    with pytest.raises(RuntimeError):
+        hip.generate_indices_and_loads(mask, None, True)  # padding without capacities
+    with pytest.raises(RuntimeError):
+        hip.generate_indices_and_loads(mask, [4, 8], True, True)  # fewer capacities than paths
+    assert b"capacity" in _lib.lib().brt_hip_last_error()
+
+
+@pytest.mark.parametrize("T,E", [(1, 4), (1000, 6), (1025, 6), (5000, 64), (30000, 8), (4000, 300)])
+def test_throttle_bit_exact(hip, T, E):
+    mask = bernoulli_mask(T, E, 0.3, seed=T + E)
+    rng = np.random.default_rng(T)
+    prefix = rng.integers(0, 50, E).astype(np.int32)
+    threshold = rng.integers(0, max(2, T // 2), E).astype(np.int32)
+    want = oracle.throttle_hotmask(mask, prefix, threshold)
+    got = hip.throttle_hotmask(mask, prefix, threshold)
+    assert np.array_equal(got[0], want[0]) and np.array_equal(got[1], want[1])
+
+
+@pytest.mark.parametrize("T,E,k", [(300, 4, 2), (3000, 3, 1), (8192, 64, 1)])
+def test_convert_index_format_bit_exact(hip, T, E, k):
+    mask, _ = topk_mask(T, E, k, seed=3)
+    seat, loads = oracle.generate_indices_and_loads(mask)
+    tag, _ = oracle.generate_indices_and_loads(mask, is_tag_index=True)
+    assert np.array_equal(hip.convert_index_format(seat, loads, False), tag)
+    assert np.array_equal(hip.convert_index_format(tag, loads, True), seat)
+    perm = np.random.default_rng(4).permutation(T)
+    assert np.array_equal(hip.convert_index_format(seat[perm], loads, False),
+                          oracle.convert_index_format(seat[perm], loads, False))
+    clipped = np.minimum(loads, 5)
+    holes = tag.copy()
+    holes[2::5] = 0  # malformed lists: the stop rule of the reference applies
+    for t in (tag, holes):
+        assert np.array_equal(hip.convert_index_format(t, clipped, True),
+                              oracle.convert_index_format(t, clipped, True))
+        assert np.array_equal(hip.convert_index_format(t, loads, True),
+                              oracle.convert_index_format(t, loads, True))
+
+
+# -------------------------------------------------------------------- dispatch
+DISPATCH_SHAPES = [  # T, E, k, cell
+    (1024, 16, 1, 512), (777, 5, 2, 33), (64, 2, 2, 1), (2048, 64, 1, 768), (3000, 32, 2, 256),
+    (5000, 8, 1, 96), (100, 128, 3, 48), (50, 300, 2, 10),
+]
+
+
+@pytest.mark.parametrize("T,E,k,cell", DISPATCH_SHAPES)
+@pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
+def test_dispatch_bit_exact(hip, T, E, k, cell, dtype):
+    mask, logits = topk_mask(T, E, k, seed=T + cell)
+    rng = np.random.default_rng(T)
+    x = as_dtype_bits(rng.standard_normal((T, cell)), dtype)
+    gates = as_dtype_bits(softmax(logits), dtype)
+    cap = max(1, int(1.25 * T * k / E))
+    for caps, pad in ((None, False), ([cap], False), ([cap, 2 * cap, 64 * cap], True)):
+        idx, loads = oracle.generate_indices_and_loads(mask, caps, pad)
+        counts = mask.sum(0).astype(np.int32)
+        for g in (None, gates):
+            want, want_tags = oracle.dispatch(x, idx, loads, gates=g, tag_generating=True, dtype=dtype)
+            # (a) reference contract: caller pre-zeroes
+            got, got_tags = hip.dispatch(x, idx, loads, g, None, True, dtype=dtype)
+            assert same_bits(got, want) and np.array_equal(got_tags, want_tags)
+            # (b) counts given: the kernel writes every row itself (output is poisoned)
+            got, got_tags = hip.dispatch(x, idx, loads, g, counts, True, dtype=dtype)
+            assert same_bits(got, want) and np.array_equal(got_tags, want_tags)
+        mpl = int(loads.max()) + 3
+        want, want_tags = oracle.dispatch(x, idx, loads, tag_generating=True, max_path_padding=True,
+                                          max_path_load=mpl, dtype=dtype)
+        for c in (None, counts):
+            got, got_tags = hip.dispatch(x, idx, loads, None, c, True, max_path_load=mpl, dtype=dtype)
+            assert same_bits(got, want) and np.array_equal(got_tags, want_tags)
+
+
+def test_dispatch_custom_tags_2d_and_tag_mode(hip):
+    T, E, cell = 1500, 4, 6
+    mask, _ = topk_mask(T, E, 2, seed=41)
+    seat, loads = oracle.generate_indices_and_loads(mask)
+    tag, _ = oracle.generate_indices_and_loads(mask, is_tag_index=True)
+    rng = np.random.default_rng(42)
+    x = rng.standard_normal((T, cell)).astype(np.float32)
+    tags = rng.integers(1, 10**6, T).astype(np.int32)
+    want = oracle.dispatch(x, seat, loads, tag_generating=True, tags=tags)
+    got = hip.dispatch(x, seat, loads, tag_generating=True, tags=tags)
+    assert same_bits(got[0], want[0]) and np.array_equal(got[1], want[1])
+    # tag-index dispatch, also with holes (stop rule of the reference) and gates
+    g = rng.random((T, E)).astype(np.float32)
+    holes = tag.copy()
+    holes[3::11] = 0
+    for t in (tag, holes):
+        for gates in (None, g):
+            want = oracle.dispatch(x, t, loads, gates=gates, tag_generating=True, tags=tags, is_tag_index=True)
+            got = hip.dispatch(x, t, loads, gates, None, True, tags, is_tag_index=True)
+            assert same_bits(got[0], want[0]) and np.array_equal(got[1], want[1])
+    # 2-d routing: path e reads in[:, e, :]
+    x2 = rng.standard_normal((T, E, 3)).astype(np.float32)
+    for idx, is_tag in ((seat, False), (tag, True)):
+        want = oracle.dispatch(x2, idx, loads, is_1d_routing=False, is_tag_index=is_tag)
+        got = hip.dispatch(x2, idx, loads, is_1d=False, is_tag_index=is_tag)
+        assert same_bits(got[0], want[0])
+    s = rng.standard_normal((T, E)).astype(np.float32)  # the score tensor itself: cell = 1
+    want = oracle.dispatch(s, seat, loads, is_1d_routing=False)
+    got = hip.dispatch(s, seat, loads, is_1d=False)
+    assert same_bits(got[0], want[0])
+
+
+def test_dispatch_odd_row_sizes_use_narrower_accesses(hip):
+    T, E = 400, 6
+    mask, logits = topk_mask(T, E, 2, seed=77)
+    idx, loads = oracle.generate_indices_and_loads(mask)
+    rng = np.random.default_rng(78)
+    for dtype, cells in (("f32", [1, 2, 3, 6]), ("f16", [1, 2, 3, 4, 6, 7, 12]), ("bf16", [1, 5, 8])):
+        for cell in cells:
+            x = as_dtype_bits(rng.standard_normal((T, cell)), dtype)
+            g = as_dtype_bits(softmax(logits), dtype)
+            for gates in (None, g):
+                want, _ = oracle.dispatch(x, idx, loads, gates=gates, dtype=dtype)
+                got, _ = hip.dispatch(x, idx, loads, gates, dtype=dtype)
+                assert same_bits(got, want), (dtype, cell)
+
+
+# --------------------------------------------------------------------- combine
+@pytest.mark.parametrize("T,E,k,cell", DISPATCH_SHAPES)
+@pytest.mark.parametrize("in_dtype,out_dtype,gate_dtype", [
+    ("f32", "f32", "f32"), ("bf16", "bf16", "bf16"), ("bf16", "f32", "f32"), ("f16", "f16", "f16"),
+    ("f16", "f32", "f16"),
+])
+def test_combine_bit_exact(hip, T, E, k, cell, in_dtype, out_dtype, gate_dtype):
+    mask, logits = topk_mask(T, E, k, seed=T + cell + 1)
+    rng = np.random.default_rng(T + 1)
+    cap = max(1, int(1.25 * T * k / E))
+    idx, loads = oracle.generate_indices_and_loads(mask, [cap])
+    P = int(loads.sum())
+    y = as_dtype_bits(rng.standard_normal((P, cell)), in_dtype)
+    gates = as_dtype_bits(softmax(logits), gate_dtype)
+    res = as_dtype_bits(rng.standard_normal((T, cell)), out_dtype)
+    for g in (None, gates):
+        for r in (None, res):
+            want = oracle.combine(y, idx, loads, gates=g, out_data=r, in_dtype=in_dtype,
+                                  out_dtype=out_dtype, gate_dtype=gate_dtype)
+            got = hip.combine(y, idx, loads, g, r, in_dtype=in_dtype, out_dtype=out_dtype,
+                              gate_dtype=gate_dtype)
+            assert same_bits(got, want), (g is None, r is None)
+    # fp64 evaluation of the same sum: the tolerance the north star states
+    yf, gf = bits_to_f32(y, in_dtype).astype(np.float64), bits_to_f32(gates, gate_dtype).astype(np.float64)
+    start = np.concatenate([[0], np.cumsum(loads)[:-1]])
+    ref = np.zeros((T, cell))
+    for e in range(E):
+        rows = np.nonzero((idx[:, e] >= 1) & (idx[:, e] <= loads[e]))[0]
+        ref[rows] += yf[start[e] + idx[rows, e] - 1] * gf[rows, e][:, None]
+    got = bits_to_f32(hip.combine(y, idx, loads, gates, None, in_dtype=in_dtype, out_dtype=out_dtype,
+                                  gate_dtype=gate_dtype), out_dtype)
+    tol = 1e-6 if out_dtype == "f32" and in_dtype == "f32" else 1e-2
+    assert np.allclose(got, ref, rtol=tol, atol=tol)
+
+
+def test_combine_max_path_padding_and_odd_rows(hip):
+    T, E = 300, 4
+    mask, logits = topk_mask(T, E, 2, seed=91)
+    idx, loads = oracle.generate_indices_and_loads(mask)
+    rng = np.random.default_rng(92)
+    for cell in (1, 3, 8, 10):
+        x = rng.standard_normal((T, cell)).astype(np.float32)
+        mpl = int(loads.max()) + 1
+        y, _ = oracle.dispatch(x, idx, loads, max_path_padding=True, max_path_load=mpl)
+        want = oracle.combine(y, idx, loads, max_path_padding=True)
+        got = hip.combine(y, idx, loads, max_path_load=mpl)
+        assert same_bits(got, want)
+        assert np.array_equal(got, 2 * x)
+        for dtype in ("f16", "bf16"):
+            yb = as_dtype_bits(y, dtype)
+            gb = as_dtype_bits(softmax(logits), dtype)
+            want = oracle.combine(yb, idx, loads, gates=gb, max_path_padding=True, in_dtype=dtype)
+            got = hip.combine(yb, idx, loads, gb, max_path_load=mpl, in_dtype=dtype)
+            assert same_bits(got, want)
+
+
+# ------------------------------------------------- full-size configurations
+def _route(hip, mask, caps=None, pad=False):
+    idx, loads, counts = hip.generate_indices_and_loads(mask, caps, pad, want_counts=True)
+    return idx, loads, counts
+
+
+def test_config1_top1_capacity_drop_roundtrip(hip):
+    # 1024 tokens x 512 fp32, 16 paths, capacity 64 with drop, identity experts
+    T, E, d, cap = 1024, 16, 512, 64
+    mask, _ = topk_mask(T, E, 1, seed=1)
+    x = np.random.default_rng(1).standard_normal((T, d)).astype(np.float32)
+    idx, loads, counts = _route(hip, mask, [cap])
+    want_idx, want_loads = oracle.generate_indices_and_loads(mask, [cap])
+    assert np.array_equal(idx, want_idx) and np.array_equal(loads, want_loads)
+    y, _ = hip.dispatch(x, idx, loads, counts=counts)
+    assert same_bits(y, oracle.dispatch(x, idx, loads)[0])
+    out = hip.combine(y, idx, loads)
+    assert same_bits(out, oracle.combine(y, idx, loads))
+    kept = ((idx >= 1) & (idx <= loads[None, :])).any(1)
+    assert np.array_equal(out[kept], x[kept]) and not out[~kept].any()
+
+
+def test_config2_switch_full_size(hip):
+    # 8192 tokens x 768 bf16, 64 paths, top-1, capacity 160 (clip and pad variants)
+    T, E, d, cap = 8192, 64, 768, 160
+    mask, logits = topk_mask(T, E, 1, seed=2)
+    x = as_dtype_bits(np.random.default_rng(2).standard_normal((T, d)), "bf16")
+    for pad in (False, True):
+        idx, loads, counts = _route(hip, mask, [cap], pad)
+        want_idx, want_loads = oracle.generate_indices_and_loads(mask, [cap], pad)
+        assert np.array_equal(idx, want_idx) and np.array_equal(loads, want_loads)
+        y, _ = hip.dispatch(x, idx, loads, counts=counts, dtype="bf16")
+        assert same_bits(y, oracle.dispatch(x, idx, loads, dtype="bf16")[0])
+        res = as_dtype_bits(np.random.default_rng(3).standard_normal((T, d)), "bf16")
+        out = hip.combine(y, idx, loads, residual_bits=res, in_dtype="bf16")
+        assert same_bits(out, oracle.combine(y, idx, loads, out_data=res, in_dtype="bf16"))
+        kept = ((idx >= 1) & (idx <= loads[None, :])).any(1)
+        assert np.array_equal(out[kept], x[kept]) and np.array_equal(out[~kept], res[~kept])
+
+
+def test_config3_top2_skewed_fp32_combine(hip):
+    # 16384 tokens x 1024 bf16, 32 paths, Zipf-skewed top-2, throttled to capacity 2048
+    T, E, d, cap = 16384, 32, 1024, 2048
+    mask, logits = topk_mask(T, E, 2, seed=3, bias=zipf_bias(E, 1.2, seed=3))
+    thr, _ = hip.throttle_hotmask(mask, np.zeros(E, np.int32), np.full(E, cap, np.int32))
+    want_thr, _ = oracle.throttle_hotmask(mask, np.zeros(E, np.int32), np.full(E, cap, np.int32))
+    assert np.array_equal(thr, want_thr) and thr.sum(0).max() == cap
+    idx, loads, counts = _route(hip, thr)
+    assert np.array_equal(idx, oracle.generate_indices_and_loads(thr)[0])
+    p = softmax(logits) * mask
+    gates = (p / p.sum(1, keepdims=True)).astype(np.float32)
+    x = as_dtype_bits(np.random.default_rng(3).standard_normal((T, d)), "bf16")
+    y, _ = hip.dispatch(x, idx, loads, counts=counts, dtype="bf16")
+    assert same_bits(y, oracle.dispatch(x, idx, loads, dtype="bf16")[0])
+    out = hip.combine(y, idx, loads, gates, in_dtype="bf16", out_dtype="f32", gate_dtype="f32")
+    assert same_bits(out, oracle.combine(y, idx, loads, gates=gates, in_dtype="bf16",
+                                         out_dtype="f32", gate_dtype="f32"))
+
+
+def test_config4_swin_small_rows_full_size(hip):
+    # 100352 tokens x 96 fp16, 8 paths, top-1, capacity 12544 with padding
+    T, E, d, cap = 100352, 8, 96, 12544
+    mask, _ = topk_mask(T, E, 1, seed=4)
+    thr, _ = hip.throttle_hotmask(mask, np.zeros(E, np.int32), np.full(E, cap, np.int32))
+    idx, loads, counts = _route(hip, thr, [cap], True)
+    want_idx, want_loads = oracle.generate_indices_and_loads(thr, [cap], True)
+    assert np.array_equal(idx, want_idx) and np.array_equal(loads, want_loads)
+    x = as_dtype_bits(np.random.default_rng(4).standard_normal((T, d)), "f16")
+    y, _ = hip.dispatch(x, idx, loads, counts=counts, max_path_load=cap, dtype="f16")
+    assert same_bits(y, oracle.dispatch(x, idx, loads, max_path_padding=True, max_path_load=cap, dtype="f16")[0])
+    out = hip.combine(y, idx, loads, max_path_load=cap, in_dtype="f16")
+    assert same_bits(out, oracle.combine(y, idx, loads, max_path_padding=True, in_dtype="f16"))
+    kept = thr.any(1)
+    assert np.array_equal(out[kept], x[kept]) and not out[~kept].any()
