@@ -10,6 +10,11 @@ import ctypes
 import os
 import subprocess
 
+# torch bundles its own HIP runtime (same soname as the system one).  Streams and
+# device pointers handed to the library come from torch, so torch's runtime must
+# be the one already resident in the process when the library is loaded.
+import torch  # noqa: F401
+
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libbrt_hip.so")
 CSRC_DIR = os.path.join(_HERE, "csrc")

@@ -20,24 +20,34 @@ constexpr int kWave = 64;
 
 __device__ __forceinline__ int lane_id() { return threadIdx.x & (kWave - 1); }
 
-// Inclusive prefix sum across the 64 lanes of a wavefront.
+// Inclusive prefix sum across the 64 lanes of a wavefront, on the DPP network
+// (no LDS, no cross-lane memory traffic): Kogge-Stone inside each row of 16 lanes
+// with row_shr, then the row totals are carried over with row_bcast15/31.
 __device__ __forceinline__ int wave_inclusive_scan(int v) {
-  const int lane = lane_id();
-#pragma unroll
-  for (int d = 1; d < kWave; d <<= 1) {
-    int n = __shfl_up(v, d, kWave);
-    if (lane >= d) v += n;
-  }
+  v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, false);  // row_shr:1
+  v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, false);  // row_shr:2
+  v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, false);  // row_shr:4
+  v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, false);  // row_shr:8
+  v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false);  // row_bcast:15 -> rows 1,3
+  v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false);  // row_bcast:31 -> rows 2,3
   return v;
+}
+
+// Value of `v` held by lane `src_lane`; src_lane must be wave-uniform.
+__device__ __forceinline__ int read_lane(int v, int src_lane) {
+  return __builtin_amdgcn_readlane(v, src_lane);
+}
+__device__ __forceinline__ float read_lane(float v, int src_lane) {
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), src_lane));
 }
 
 // bf16 <-> fp32 (round to nearest even; NaN stays NaN).
 __device__ __forceinline__ float bf16_to_float(uint32_t h) { return __uint_as_float(h << 16); }
 __device__ __forceinline__ uint32_t float_to_bf16(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x0040u;
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return u >> 16;
+  // gfx950 converts in hardware (v_cvt_pk_bf16_f32, round to nearest even)
+  union { __bf16 h; uint16_t u; } c;
+  c.h = static_cast<__bf16>(f);
+  return c.u;
 }
 __device__ __forceinline__ float f16_to_float(uint32_t h) {
   union { uint16_t u; _Float16 f; } c;

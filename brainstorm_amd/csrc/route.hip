@@ -21,13 +21,24 @@ namespace brt {
 namespace {
 
 constexpr int kBlock = 256;
-constexpr int kUnroll = 4;
+
+// Copy units are native vector types, so that arrays of them live in registers.
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
 
 template <int BYTES> struct Unit;
-template <> struct Unit<16> { using type = uint4; };
-template <> struct Unit<8> { using type = uint2; };
+template <> struct Unit<16> { using type = u32x4; };
+template <> struct Unit<8> { using type = u32x2; };
 template <> struct Unit<4> { using type = uint32_t; };
 template <> struct Unit<2> { using type = uint16_t; };
+
+template <int BYTES>
+__device__ __forceinline__ uint32_t unit_word(const typename Unit<BYTES>::type& v, int i) {
+  if constexpr (BYTES >= 8) return v[i];
+  else return v;
+}
 
 constexpr int elem_bytes(int dt) { return dt == BRT_F32 ? 4 : 2; }
 
@@ -38,14 +49,14 @@ __device__ __forceinline__ void unpack(const typename Unit<BYTES>::type& v,
   if constexpr (BYTES == 2) {
     x[0] = half_bits_to_float<DT>(v);
   } else {
-    const uint32_t* w = reinterpret_cast<const uint32_t*>(&v);
 #pragma unroll
     for (int i = 0; i < BYTES / 4; ++i) {
+      const uint32_t w = unit_word<BYTES>(v, i);
       if constexpr (DT == BRT_F32) {
-        x[i] = __uint_as_float(w[i]);
+        x[i] = __uint_as_float(w);
       } else {
-        x[2 * i] = half_bits_to_float<DT>(w[i] & 0xffffu);
-        x[2 * i + 1] = half_bits_to_float<DT>(w[i] >> 16);
+        x[2 * i] = half_bits_to_float<DT>(w & 0xffffu);
+        x[2 * i + 1] = half_bits_to_float<DT>(w >> 16);
       }
     }
   }
@@ -57,10 +68,13 @@ __device__ __forceinline__ void pack_store(void* p, const float (&x)[N]) {
   if constexpr (DT == BRT_F32) {
     if constexpr (N % 4 == 0) {
 #pragma unroll
-      for (int i = 0; i < N / 4; ++i)
-        static_cast<float4*>(p)[i] = make_float4(x[4 * i], x[4 * i + 1], x[4 * i + 2], x[4 * i + 3]);
+      for (int i = 0; i < N / 4; ++i) {
+        f32x4 o = {x[4 * i], x[4 * i + 1], x[4 * i + 2], x[4 * i + 3]};
+        static_cast<f32x4*>(p)[i] = o;
+      }
     } else if constexpr (N == 2) {
-      *static_cast<float2*>(p) = make_float2(x[0], x[1]);
+      f32x2 o = {x[0], x[1]};
+      *static_cast<f32x2*>(p) = o;
     } else {
       *static_cast<float*>(p) = x[0];
     }
@@ -73,9 +87,11 @@ __device__ __forceinline__ void pack_store(void* p, const float (&x)[N]) {
       for (int i = 0; i < N / 2; ++i)
         w[i] = float_to_half_bits<DT>(x[2 * i]) | (float_to_half_bits<DT>(x[2 * i + 1]) << 16);
       if constexpr (N == 8) {
-        *static_cast<uint4*>(p) = make_uint4(w[0], w[1], w[2], w[3]);
+        u32x4 o = {w[0], w[1], w[2], w[3]};
+        *static_cast<u32x4*>(p) = o;
       } else if constexpr (N == 4) {
-        *static_cast<uint2*>(p) = make_uint2(w[0], w[1]);
+        u32x2 o = {w[0], w[1]};
+        *static_cast<u32x2*>(p) = o;
       } else {
         *static_cast<uint32_t*>(p) = w[0];
       }
@@ -85,9 +101,67 @@ __device__ __forceinline__ void pack_store(void* p, const float (&x)[N]) {
 
 template <int BYTES>
 __device__ __forceinline__ typename Unit<BYTES>::type zero_unit() {
-  if constexpr (BYTES == 16) return make_uint4(0, 0, 0, 0);
-  else if constexpr (BYTES == 8) return make_uint2(0, 0);
-  else return 0;
+  typename Unit<BYTES>::type z = {};
+  return z;
+}
+
+// ------------------------------------------------------- wave-level plumbing
+// Every wavefront works on its own: it owns `rows_pw` consecutive rows of the
+// index matrix, keeps its tables in a private slice of LDS and never meets a
+// block barrier.  LDS traffic of one wavefront is executed in order, so a
+// wave-scope fence between the "write list" and "read list" phases is all the
+// synchronisation that is needed.
+constexpr int kSteps = 8;  // index words fetched per lane before any is used
+
+__device__ __forceinline__ void wave_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+}
+
+// How one wave-wide load of 64 index words maps to (row, path): for E <= 64 a
+// step covers 64/ep whole rows (ep = E rounded up to a power of two, lanes
+// beyond E idle); for E > 64 a row takes ceil(E/64) steps.
+struct StepMap {
+  int ep_shift;  // log2(ep), E <= 64 only
+  int chunks;    // steps per row, E > 64 only (1 otherwise)
+  int E;
+  __device__ __forceinline__ int rows_per_step() const { return E <= kWave ? kWave >> ep_shift : 1; }
+  __device__ __forceinline__ int steps(int rows) const {
+    return E <= kWave ? (rows + rows_per_step() - 1) >> (6 - ep_shift) : rows * chunks;
+  }
+  // row (relative) and path handled by `lane` in `step`; path >= E means idle
+  __device__ __forceinline__ void locate(int step, int lane, int& row, int& e) const {
+    if (E <= kWave) {
+      row = step * rows_per_step() + (lane >> ep_shift);
+      e = lane & ((1 << ep_shift) - 1);
+    } else {
+      row = step / chunks;
+      e = (step - row * chunks) * kWave + lane;
+    }
+  }
+  // lanes that belong to the same row as `lane` within a step
+  __device__ __forceinline__ unsigned long long segment(int lane) const {
+    if (E > kWave || ep_shift == 6) return ~0ull;
+    const int ep = 1 << ep_shift;
+    return ((1ull << ep) - 1ull) << ((lane >> ep_shift) * ep);
+  }
+};
+
+// Per-wave copy of loads[] and the path start offsets (exclusive prefix of the
+// loads, or e*stride for fixed-stride layouts).
+__device__ __forceinline__ void wave_path_tables(const int* __restrict__ loads, int* s_loads,
+                                                 int* s_start, int E, int stride, int lane) {
+  int carry = 0;
+  for (int base = 0; base < E; base += kWave) {
+    const int e = base + lane;
+    const int v = e < E ? loads[e] : 0;
+    const int incl = wave_inclusive_scan(v);
+    if (e < E) {
+      s_loads[e] = v;
+      s_start[e] = stride != 0 ? e * stride : carry + incl - v;
+    }
+    carry += __shfl(incl, kWave - 1, kWave);
+  }
 }
 
 // ---------------------------------------------------------------- dispatch
@@ -101,9 +175,10 @@ struct DispatchArgs {
   const int* old_tags;
   int* new_tags;
   int T, E, P, mpl;
-  int cpr;       // units (BYTES each) per row
-  int rows_pb;   // rows of the index matrix per block
-  int list_cap;  // work-list capacity (>= rows_pb * E)
+  int cpr;      // units (BYTES each) per row
+  int rows_pw;  // rows of the index matrix per wavefront
+  int lds_pw;   // ints of LDS per wavefront
+  StepMap map;
   int is_1d, is_tag_index;
 };
 
@@ -113,21 +188,37 @@ __global__ __launch_bounds__(kBlock) void dispatch_kernel(DispatchArgs a) {
   using U = typename Unit<BYTES>::type;
   extern __shared__ int smem[];
   const int E = a.E;
-  int* s_loads = smem;
-  int* s_start = smem + E;
-  int* s_zstart = smem + 2 * E;  // E + 1 entries: padding rows before path e
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave_in_block = threadIdx.x >> 6;
+  const int waves_pb = blockDim.x >> 6;
+  const long wave = static_cast<long>(blockIdx.x) * waves_pb + wave_in_block;
+  const long n_waves = static_cast<long>(gridDim.x) * waves_pb;
+  int* s_loads = smem + wave_in_block * a.lds_pw;
+  int* s_start = s_loads + E;
+  int* s_zstart = s_start + E;  // E + 1 entries: padding rows before path e
   int* s_dst = s_zstart + E + 1;
-  int* s_src = s_dst + a.list_cap;
-  float* s_gate = reinterpret_cast<float*>(s_src + a.list_cap);
-  __shared__ int s_n;
+  int* s_src = s_dst + a.rows_pw * E;
+  float* s_gate = reinterpret_cast<float*>(s_src + a.rows_pw * E);
+  const unsigned long long lt = (1ull << lane) - 1ull;
 
-  const int tid = threadIdx.x;
-  if (tid == 0) s_n = 0;
-  load_and_scan_paths(a.loads, s_loads, s_start, E, a.mpl);
-  if (a.counts != nullptr && tid < kWave) {
+  const long r0 = wave * a.rows_pw;
+  const int nr = static_cast<int>(max(0l, min(static_cast<long>(a.rows_pw), a.T - r0)));
+  const int* __restrict__ idx0 = a.idx + r0 * E;
+  const int n_steps = a.map.steps(nr);
+
+  // ---- 1. fetch the first batch of index words, then build the path tables ------
+  int v[kSteps];
+#pragma unroll
+  for (int j = 0; j < kSteps; ++j) {
+    int row, e;
+    a.map.locate(j, lane, row, e);
+    v[j] = (j < n_steps && row < nr && e < E) ? idx0[row * E + e] : 0;
+  }
+  wave_path_tables(a.loads, s_loads, s_start, E, a.mpl, lane);
+  if (a.counts != nullptr) {
     int carry = 0;
     for (int base = 0; base < E; base += kWave) {
-      const int e = base + tid;
+      const int e = base + lane;
       int z = 0;
       if (e < E) {
         const int load = a.loads[e];
@@ -139,65 +230,80 @@ __global__ __launch_bounds__(kBlock) void dispatch_kernel(DispatchArgs a) {
       if (e < E) s_zstart[e] = carry + incl - z;
       carry += __shfl(incl, kWave - 1, kWave);
     }
-    if (tid == 0) s_zstart[E] = carry;
+    if (lane == 0) s_zstart[E] = carry;
   }
-  __syncthreads();
+  wave_sync();
 
-  // ---- 1. index rows -> work list (destination row, source row, gate) --------
-  const int r0 = blockIdx.x * a.rows_pb;
-  const int nr = max(0, min(a.rows_pb, a.T - r0));
-  const int* idx0 = a.idx + static_cast<size_t>(r0) * E;
-  for (int i = tid; i < nr * E; i += kBlock) {
-    const int rl = i / E, e = i - rl * E;
-    const int r = r0 + rl;
-    const int v = idx0[i];
-    bool ok;
-    int dst_row, tok;
-    if (!a.is_tag_index) {  // v = seat of token r on path e
-      ok = v >= 1 && v <= s_loads[e];
-      dst_row = s_start[e] + v - 1;
-      tok = r;
-    } else {  // v = 1-based token held by slot r of path e
-      ok = r < s_loads[e] && v >= 1 && v <= a.T;
-      dst_row = s_start[e] + r;
-      tok = v - 1;
-      // the reference walks slots r, r+512, ... per block and stops at the first
-      // empty one (route.cu:84-92): an empty slot above in that chain hides r
-      if (ok)
-        for (int k = r - 512; k >= 0; k -= 512)
-          if (a.idx[static_cast<size_t>(k) * E + e] == 0) {
-            ok = false;
-            break;
+  // ---- 2. index words -> compact list of (destination row, source row, gate) -----
+  int n = 0;
+  for (int s0 = 0; s0 < n_steps; s0 += kSteps) {
+    if (s0 > 0) {
+#pragma unroll
+      for (int j = 0; j < kSteps; ++j) {
+        int row, e;
+        a.map.locate(s0 + j, lane, row, e);
+        v[j] = (s0 + j < n_steps && row < nr && e < E) ? idx0[row * E + e] : 0;
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < kSteps; ++j) {
+      if (s0 + j < n_steps) {  // wave-uniform
+        int row, e;
+        a.map.locate(s0 + j, lane, row, e);
+        bool ok = false;
+        int dst_row = 0, tok = 0;
+        if (row < nr && e < E) {
+          const long r = r0 + row;
+          if (!a.is_tag_index) {  // v = seat of token r on path e
+            ok = v[j] >= 1 && v[j] <= s_loads[e];
+            dst_row = s_start[e] + v[j] - 1;
+            tok = static_cast<int>(r);
+          } else {  // v = 1-based token held by slot r of path e
+            ok = r < s_loads[e] && v[j] >= 1 && v[j] <= a.T;
+            dst_row = s_start[e] + static_cast<int>(r);
+            tok = v[j] - 1;
+            // the reference walks slots r, r+512, ... per block and stops at the
+            // first empty one (route.cu:84-92): an empty slot above hides r
+            if (ok)
+              for (long k = r - 512; k >= 0; k -= 512)
+                if (a.idx[k * E + e] == 0) {
+                  ok = false;
+                  break;
+                }
           }
-    }
-    ok = ok && dst_row >= 0 && dst_row < a.P;
-    if (ok) {
-      const int pos = atomicAdd(&s_n, 1);
-      s_dst[pos] = dst_row;
-      s_src[pos] = a.is_1d ? tok : tok * E + e;
-      if constexpr (DT >= 0) s_gate[pos] = load_gate(a.gates, DT, static_cast<size_t>(tok) * E + e);
-      if (a.new_tags != nullptr) a.new_tags[dst_row] = a.old_tags ? a.old_tags[tok] : tok + 1;
+          ok = ok && dst_row >= 0 && dst_row < a.P;
+        }
+        const unsigned long long m = __ballot(ok);
+        if (ok) {
+          const int pos = n + __popcll(m & lt);
+          s_dst[pos] = dst_row;
+          s_src[pos] = a.is_1d ? tok : tok * E + e;
+          if constexpr (DT >= 0)
+            s_gate[pos] = load_gate(a.gates, DT, static_cast<size_t>(tok) * E + e);
+          if (a.new_tags != nullptr) a.new_tags[dst_row] = a.old_tags ? a.old_tags[tok] : tok + 1;
+        }
+        n += __popcll(m);
+      }
     }
   }
-  __syncthreads();
+  wave_sync();
 
-  // ---- 2. move rows: flat loop over (entry, unit) pairs -----------------------
-  const int n = s_n;
+  // ---- 3. move rows: flat loop over (entry, unit) pairs, loads first ---------------
   const int cpr = a.cpr;
   const U* __restrict__ src = static_cast<const U*>(a.src);
   U* __restrict__ dst = static_cast<U*>(a.dst);
-  int ent = tid / cpr, off = tid - ent * cpr;
-  const int d_ent = kBlock / cpr, d_off = kBlock - d_ent * cpr;
+  int ent = lane / cpr, off = lane - ent * cpr;
+  const int d_ent = kWave / cpr, d_off = kWave - d_ent * cpr;
   while (ent < n) {
-    U v[kUnroll];
-    size_t to[kUnroll];
-    float g[kUnroll];
-    bool live[kUnroll];
+    U val[kSteps];
+    size_t to[kSteps];
+    float g[kSteps];
+    bool live[kSteps];
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
+    for (int u = 0; u < kSteps; ++u) {
       live[u] = ent < n;
       if (live[u]) {
-        v[u] = src[static_cast<size_t>(s_src[ent]) * cpr + off];
+        val[u] = src[static_cast<size_t>(s_src[ent]) * cpr + off];
         to[u] = static_cast<size_t>(s_dst[ent]) * cpr + off;
         if constexpr (DT >= 0) g[u] = s_gate[ent];
       }
@@ -209,29 +315,28 @@ __global__ __launch_bounds__(kBlock) void dispatch_kernel(DispatchArgs a) {
       }
     }
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
+    for (int u = 0; u < kSteps; ++u) {
       if (live[u]) {
         if constexpr (DT >= 0) {
           constexpr int NE = BYTES / elem_bytes(DT);
           float x[NE];
-          unpack<DT, BYTES>(v[u], x);
+          unpack<DT, BYTES>(val[u], x);
 #pragma unroll
           for (int i = 0; i < NE; ++i) x[i] = x[i] * g[u];
           pack_store<DT, NE>(dst + to[u], x);
         } else {
-          dst[to[u]] = v[u];
+          dst[to[u]] = val[u];
         }
       }
     }
   }
 
-  // ---- 3. zero-fill this block's share of the padding rows ---------------------
+  // ---- 4. zero-fill this wavefront's share of the padding rows ---------------------
   if (a.counts != nullptr) {
     const long Z = s_zstart[E];
-    const long z0 = Z * blockIdx.x / gridDim.x;
-    const long z1 = Z * (blockIdx.x + 1) / gridDim.x;
-    const int wave = tid >> 6, lane = tid & (kWave - 1);
-    for (long z = z0 + wave; z < z1; z += kBlock / kWave) {
+    const long z0 = Z * wave / n_waves;
+    const long z1 = Z * (wave + 1) / n_waves;
+    for (long z = z0; z < z1; ++z) {
       int lo = 0, hi = E;  // largest e with s_zstart[e] <= z
       while (hi - lo > 1) {
         const int mid = (lo + hi) >> 1;
@@ -258,8 +363,9 @@ struct CombineArgs {
   const int* loads;
   int T, E, P, mpl;
   int cpr;      // input units per row
-  int rows_pb;  // tokens per block
-  int ep_shift; // log2 of E rounded up to a power of two (E <= 64 only)
+  int rows_pw;  // tokens per wavefront
+  int lds_pw;   // ints of LDS per wavefront
+  StepMap map;
   int is_residual, gate_dtype;
 };
 
@@ -268,88 +374,89 @@ __global__ __launch_bounds__(kBlock) void combine_kernel(CombineArgs a) {
   using U = typename Unit<BYTES>::type;
   constexpr int NE = BYTES / elem_bytes(IN_DT);
   constexpr int OUT_BYTES = NE * elem_bytes(OUT_DT);
+  constexpr int kAcc = 4;  // (token, unit) pairs accumulated concurrently per lane
   extern __shared__ int smem[];
   const int E = a.E;
-  int* s_loads = smem;
-  int* s_start = smem + E;
-  int* s_cnt = smem + 2 * E;         // valid routes per token
-  int* s_row = s_cnt + a.rows_pb;    // [rows_pb][E] source rows, ascending path order
-  float* s_gate = reinterpret_cast<float*>(s_row + a.rows_pb * E);
-
-  const int tid = threadIdx.x;
-  load_and_scan_paths(a.loads, s_loads, s_start, E, a.mpl);
-  __syncthreads();
-
-  // ---- 1. per token: ordered list of valid (source row, gate) ------------------
-  // lanes = paths, __ballot + popcount compacts the valid ones in ascending order
-  const int t0 = blockIdx.x * a.rows_pb;
-  const int nt = min(a.rows_pb, a.T - t0);
-  const int wave = tid >> 6, lane = tid & (kWave - 1);
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave_in_block = threadIdx.x >> 6;
+  const long wave = static_cast<long>(blockIdx.x) * (blockDim.x >> 6) + wave_in_block;
+  int* s_loads = smem + wave_in_block * a.lds_pw;
+  int* s_start = s_loads + E;
+  int* s_cnt = s_start + E;          // valid routes per token
+  int* s_row = s_cnt + a.rows_pw;    // [rows_pw][E] source rows, ascending path order
+  float* s_gate = reinterpret_cast<float*>(s_row + a.rows_pw * E);
   const unsigned long long lt = (1ull << lane) - 1ull;
-  if (E <= kWave) {
-    const int ep = 1 << a.ep_shift;  // lanes per token
-    const int tpw = kWave >> a.ep_shift;
-    const int sub = lane >> a.ep_shift, e = lane & (ep - 1);
-    const unsigned long long seg =
-        ep == kWave ? ~0ull : (((1ull << ep) - 1ull) << (sub * ep));
-    for (int base = wave * tpw; base < nt; base += (kBlock / kWave) * tpw) {
-      const int tl = base + sub;
-      bool ok = false;
-      int row = 0;
-      size_t gi = 0;
-      if (tl < nt && e < E) {
-        gi = static_cast<size_t>(t0 + tl) * E + e;
-        const int seat = a.idx[gi];
-        row = s_start[e] + seat - 1;
-        ok = seat >= 1 && seat <= s_loads[e] && row < a.P;
+  const unsigned long long seg = a.map.segment(lane);
+
+  const long t0 = wave * a.rows_pw;
+  const int nt = static_cast<int>(max(0l, min(static_cast<long>(a.rows_pw), a.T - t0)));
+  if (nt == 0) return;
+  const int* __restrict__ idx0 = a.idx + t0 * E;
+  const int n_steps = a.map.steps(nt);
+
+  int v[kSteps];
+#pragma unroll
+  for (int j = 0; j < kSteps; ++j) {
+    int row, e;
+    a.map.locate(j, lane, row, e);
+    v[j] = (j < n_steps && row < nt && e < E) ? idx0[row * E + e] : 0;
+  }
+  wave_path_tables(a.loads, s_loads, s_start, E, a.mpl, lane);
+  wave_sync();
+
+  // ---- per token: valid (source row, gate) in ascending path order ---------------
+  // lanes = paths; __ballot + popcount compacts the valid ones without reordering
+  for (int s0 = 0; s0 < n_steps; s0 += kSteps) {
+    if (s0 > 0) {
+#pragma unroll
+      for (int j = 0; j < kSteps; ++j) {
+        int row, e;
+        a.map.locate(s0 + j, lane, row, e);
+        v[j] = (s0 + j < n_steps && row < nt && e < E) ? idx0[row * E + e] : 0;
       }
-      const unsigned long long m = __ballot(ok) & seg;
-      if (ok) {
-        const int pos = __popcll(m & lt);
-        s_row[tl * E + pos] = row;
-        s_gate[tl * E + pos] = a.gates ? load_gate(a.gates, a.gate_dtype, gi) : 1.0f;
-      }
-      if (e == 0 && tl < nt) s_cnt[tl] = __popcll(m);
     }
-  } else {
-    for (int tl = wave; tl < nt; tl += kBlock / kWave) {
-      int base = 0;
-      for (int e0 = 0; e0 < E; e0 += kWave) {
-        const int e = e0 + lane;
+#pragma unroll
+    for (int j = 0; j < kSteps; ++j) {
+      if (s0 + j < n_steps) {  // wave-uniform
+        int row, e;
+        a.map.locate(s0 + j, lane, row, e);
         bool ok = false;
-        int row = 0;
-        size_t gi = 0;
-        if (e < E) {
-          gi = static_cast<size_t>(t0 + tl) * E + e;
-          const int seat = a.idx[gi];
-          row = s_start[e] + seat - 1;
-          ok = seat >= 1 && seat <= s_loads[e] && row < a.P;
+        int src_row = 0;
+        if (row < nt && e < E) {
+          src_row = s_start[e] + v[j] - 1;
+          ok = v[j] >= 1 && v[j] <= s_loads[e] && src_row < a.P;
         }
-        const unsigned long long m = __ballot(ok);
-        if (ok) {
-          const int pos = base + __popcll(m & lt);
-          s_row[tl * E + pos] = row;
-          s_gate[tl * E + pos] = a.gates ? load_gate(a.gates, a.gate_dtype, gi) : 1.0f;
+        const unsigned long long m = __ballot(ok) & seg;
+        if (row < nt) {
+          // a row wider than one step continues where its previous step stopped
+          const int base = (E > kWave && e >= kWave) ? s_cnt[row] : 0;
+          if (ok) {
+            const int pos = base + __popcll(m & lt);
+            s_row[row * E + pos] = src_row;
+            s_gate[row * E + pos] =
+                a.gates ? load_gate(a.gates, a.gate_dtype, static_cast<size_t>(t0 + row) * E + e)
+                        : 1.0f;
+          }
+          wave_sync();
+          if ((e & (kWave - 1)) == 0 || (E <= kWave && e == 0)) s_cnt[row] = base + __popcll(m);
         }
-        base += __popcll(m);
       }
-      if (lane == 0) s_cnt[tl] = base;
     }
   }
-  __syncthreads();
+  wave_sync();
 
-  // ---- 2. gather + fp32 accumulate, flat loop over (token, unit) pairs -----------
+  // ---- gather + fp32 accumulate, flat loop over (token, unit) pairs -----------------
   const int cpr = a.cpr;
   const U* __restrict__ src = static_cast<const U*>(a.src);
   char* __restrict__ dst = static_cast<char*>(a.dst);
-  int tl = tid / cpr, off = tid - tl * cpr;
-  const int d_tl = kBlock / cpr, d_off = kBlock - d_tl * cpr;
+  int tl = lane / cpr, off = lane - tl * cpr;
+  const int d_tl = kWave / cpr, d_off = kWave - d_tl * cpr;
   while (tl < nt) {
-    float acc[kUnroll][NE];
-    int n[kUnroll], tok[kUnroll], o[kUnroll];
+    float acc[kAcc][NE];
+    int n[kAcc], tok[kAcc], o[kAcc];
     int nmax = 0;
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
+    for (int u = 0; u < kAcc; ++u) {
       tok[u] = tl;
       o[u] = off;
       n[u] = tl < nt ? s_cnt[tl] : -1;
@@ -364,30 +471,537 @@ __global__ __launch_bounds__(kBlock) void combine_kernel(CombineArgs a) {
       }
     }
     for (int k = 0; k < nmax; ++k) {
-      U v[kUnroll];
-      float g[kUnroll];
+      U val[kAcc];
+      float g[kAcc];
 #pragma unroll
-      for (int u = 0; u < kUnroll; ++u)
+      for (int u = 0; u < kAcc; ++u)
         if (k < n[u]) {
-          v[u] = src[static_cast<size_t>(s_row[tok[u] * E + k]) * cpr + o[u]];
+          val[u] = src[static_cast<size_t>(s_row[tok[u] * E + k]) * cpr + o[u]];
           g[u] = s_gate[tok[u] * E + k];
         }
 #pragma unroll
-      for (int u = 0; u < kUnroll; ++u)
+      for (int u = 0; u < kAcc; ++u)
         if (k < n[u]) {
           float x[NE];
-          unpack<IN_DT, BYTES>(v[u], x);
+          unpack<IN_DT, BYTES>(val[u], x);
           // one rounding for the product, one for the sum (no fused multiply-add)
 #pragma unroll
           for (int i = 0; i < NE; ++i) acc[u][i] = acc[u][i] + x[i] * g[u];
         }
     }
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
+    for (int u = 0; u < kAcc; ++u) {
       // n < 0: past the end; n == 0: token without a valid route
       if (n[u] > 0 || (n[u] == 0 && !a.is_residual)) {
         const size_t at = (static_cast<size_t>(t0 + tok[u]) * cpr + o[u]) * OUT_BYTES;
         pack_store<OUT_DT, NE>(dst + at, acc[u]);
+      }
+    }
+  }
+}
+
+// ------------------------------------------------ fast path: E <= 64 paths
+// With at most 64 paths one wave-wide load covers whole rows of the index
+// matrix and everything stays in registers: lane e holds loads[e] and the start
+// offset of path e (DPP prefix scan), __ballot marks the valid (row, path)
+// pairs, and the wavefront walks the set bits, broadcasting destination/source
+// row and gate with v_readlane while all 64 lanes move the row.  No LDS, no
+// barrier; `kInFlight` 16-byte accesses per lane are issued before the first
+// store.
+constexpr int kInFlight = 8;
+
+struct SmallTables {
+  int load_e, start_e;  // of the path this lane looks at (e = lane % ep)
+  int my_load, my_start;  // of path `lane`
+};
+
+__device__ __forceinline__ SmallTables small_tables(const int* __restrict__ loads, int E, int mpl,
+                                                    int ep_shift, int lane) {
+  SmallTables t;
+  t.my_load = lane < E ? loads[lane] : 0;
+  const int incl = wave_inclusive_scan(t.my_load);
+  t.my_start = mpl != 0 ? lane * mpl : incl - t.my_load;
+  if (ep_shift == 6) {
+    t.load_e = t.my_load;
+    t.start_e = t.my_start;
+  } else {
+    const int e = lane & ((1 << ep_shift) - 1);
+    t.load_e = __shfl(t.my_load, e, kWave);
+    t.start_e = __shfl(t.my_start, e, kWave);
+  }
+  return t;
+}
+
+// UPR = 16-byte units each lane moves per row and pass (rows of up to 64*UPR
+// units take one pass); kInFlight/UPR rows are in flight together.
+template <int BYTES, int DT, int UPR>
+__global__ __launch_bounds__(kBlock) void dispatch_small_kernel(DispatchArgs a) {
+  using U = typename Unit<BYTES>::type;
+  constexpr int G = kInFlight / UPR;
+  const int E = a.E;
+  const int lane = threadIdx.x & (kWave - 1);
+  const long wave = static_cast<long>(blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  const long n_waves = static_cast<long>(gridDim.x) * (blockDim.x >> 6);
+  const int ep_shift = a.map.ep_shift;
+  const int rps = kWave >> ep_shift;  // rows per step
+  const int e = lane & ((1 << ep_shift) - 1);
+  const int sub = lane >> ep_shift;
+
+  const long r0 = wave * a.rows_pw;
+  const int nr = static_cast<int>(max(0l, min(static_cast<long>(a.rows_pw), a.T - r0)));
+  const int n_steps = (nr + rps - 1) >> (6 - ep_shift);
+  const int* __restrict__ idx0 = a.idx + r0 * E;
+  const int cpr = a.cpr;
+  const U* __restrict__ src = static_cast<const U*>(a.src);
+  U* __restrict__ dst = static_cast<U*>(a.dst);
+
+  int v_next = (n_steps > 0 && sub < nr && e < E) ? idx0[sub * E + e] : 0;
+  const SmallTables tab = small_tables(a.loads, E, a.mpl, ep_shift, lane);
+
+  for (int step = 0; step < n_steps; ++step) {
+    const int v = v_next;
+    const int row = step * rps + sub;
+    {  // prefetch the next step's index words before the rows of this one move
+      const int nrow = row + rps;
+      v_next = (step + 1 < n_steps && nrow < nr && e < E) ? idx0[nrow * E + e] : 0;
+    }
+    bool ok = false;
+    int dst_row = 0, src_row = 0;
+    float gate = 1.0f;
+    if (row < nr && e < E) {
+      const long r = r0 + row;
+      int tok;
+      if (!a.is_tag_index) {  // v = seat of token r on path e
+        ok = v >= 1 && v <= tab.load_e;
+        dst_row = tab.start_e + v - 1;
+        tok = static_cast<int>(r);
+      } else {  // v = 1-based token held by slot r of path e
+        ok = r < tab.load_e && v >= 1 && v <= a.T;
+        dst_row = tab.start_e + static_cast<int>(r);
+        tok = v - 1;
+        if (ok)  // stop rule of the reference, see dispatch_kernel
+          for (long k = r - 512; k >= 0; k -= 512)
+            if (a.idx[k * E + e] == 0) {
+              ok = false;
+              break;
+            }
+      }
+      ok = ok && dst_row >= 0 && dst_row < a.P;
+      if (ok) {
+        src_row = a.is_1d ? tok : tok * E + e;
+        if constexpr (DT >= 0) gate = load_gate(a.gates, DT, static_cast<size_t>(tok) * E + e);
+        if (a.new_tags != nullptr) a.new_tags[dst_row] = a.old_tags ? a.old_tags[tok] : tok + 1;
+      }
+    }
+    unsigned long long m = __ballot(ok);
+    while (m != 0) {  // wave-uniform: up to G rows per trip
+      int d[G], sr[G];
+      float g[G];
+      int nb = 0;
+#pragma unroll
+      for (int i = 0; i < G; ++i) {
+        d[i] = 0; sr[i] = 0; g[i] = 1.0f;
+        if (m != 0) {
+          const int b = __builtin_ctzll(m);
+          m &= m - 1;
+          d[i] = read_lane(dst_row, b);
+          sr[i] = read_lane(src_row, b);
+          if constexpr (DT >= 0) g[i] = read_lane(gate, b);
+          nb = i + 1;
+        }
+      }
+      for (int off0 = 0; off0 < cpr; off0 += kWave * UPR) {
+        U val[G][UPR];
+#pragma unroll
+        for (int i = 0; i < G; ++i)
+#pragma unroll
+          for (int u = 0; u < UPR; ++u) {
+            const int off = off0 + u * kWave + lane;
+            if (i < nb && off < cpr) val[i][u] = src[static_cast<size_t>(sr[i]) * cpr + off];
+          }
+#pragma unroll
+        for (int i = 0; i < G; ++i)
+#pragma unroll
+          for (int u = 0; u < UPR; ++u) {
+            const int off = off0 + u * kWave + lane;
+            if (i < nb && off < cpr) {
+              U* to = dst + static_cast<size_t>(d[i]) * cpr + off;
+              if constexpr (DT >= 0) {
+                constexpr int NE = BYTES / elem_bytes(DT);
+                float x[NE];
+                unpack<DT, BYTES>(val[i][u], x);
+#pragma unroll
+                for (int q = 0; q < NE; ++q) x[q] = x[q] * g[i];
+                pack_store<DT, NE>(to, x);
+              } else {
+                *to = val[i][u];
+              }
+            }
+          }
+      }
+    }
+  }
+
+  // ---- zero-fill this wavefront's share of the padding rows ------------------------
+  if (a.counts != nullptr) {
+    int z = 0;
+    if (lane < E) {
+      const int alloc = a.mpl != 0 ? a.mpl : tab.my_load;
+      const int filled = max(0, min(min(a.counts[lane], tab.my_load), alloc));
+      z = max(0, alloc - filled);
+    }
+    const int z_incl = wave_inclusive_scan(z);
+    const long Z = read_lane(z_incl, kWave - 1);
+    const long z0 = Z * wave / n_waves;
+    const long z1 = Z * (wave + 1) / n_waves;
+    for (long zi = z0; zi < z1; ++zi) {
+      // path of padding row zi: first lane whose inclusive count exceeds zi
+      const int pe = __builtin_ctzll(__ballot(z_incl > zi));
+      const int pad = read_lane(z, pe);
+      const int alloc = a.mpl != 0 ? a.mpl : read_lane(tab.my_load, pe);
+      const long row = static_cast<long>(read_lane(tab.my_start, pe)) + (alloc - pad) +
+                       (zi - (read_lane(z_incl, pe) - pad));
+      if (row < a.P) {
+        for (int o = lane; o < cpr; o += kWave) dst[static_cast<size_t>(row) * cpr + o] = zero_unit<BYTES>();
+        if (a.new_tags != nullptr && lane == 0) a.new_tags[row] = 0;
+      }
+    }
+  }
+}
+
+template <int BYTES, int IN_DT, int OUT_DT, int UPR>
+__global__ __launch_bounds__(kBlock) void combine_small_kernel(CombineArgs a) {
+  using U = typename Unit<BYTES>::type;
+  constexpr int NE = BYTES / elem_bytes(IN_DT);
+  constexpr int OUT_BYTES = NE * elem_bytes(OUT_DT);
+  constexpr int G = 4 / UPR;  // tokens accumulated together (UPR <= 4)
+  const int E = a.E;
+  const int lane = threadIdx.x & (kWave - 1);
+  const long wave = static_cast<long>(blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  const int ep_shift = a.map.ep_shift;
+  const int ep = 1 << ep_shift;
+  const int rps = kWave >> ep_shift;  // tokens per step
+  const int e = lane & (ep - 1);
+  const int sub = lane >> ep_shift;
+  const unsigned long long seg0 = ep == kWave ? ~0ull : ((1ull << ep) - 1ull);
+
+  const long t0 = wave * a.rows_pw;
+  const int nt = static_cast<int>(max(0l, min(static_cast<long>(a.rows_pw), a.T - t0)));
+  if (nt == 0) return;
+  const int n_steps = (nt + rps - 1) >> (6 - ep_shift);
+  const int* __restrict__ idx0 = a.idx + t0 * E;
+  const int cpr = a.cpr;
+  const U* __restrict__ src = static_cast<const U*>(a.src);
+  char* __restrict__ dst = static_cast<char*>(a.dst);
+
+  int v_next = (sub < nt && e < E) ? idx0[sub * E + e] : 0;
+  const SmallTables tab = small_tables(a.loads, E, a.mpl, ep_shift, lane);
+
+  for (int step = 0; step < n_steps; ++step) {
+    const int v = v_next;
+    const int row = step * rps + sub;
+    {
+      const int nrow = row + rps;
+      v_next = (step + 1 < n_steps && nrow < nt && e < E) ? idx0[nrow * E + e] : 0;
+    }
+    bool ok = false;
+    int src_row = 0;
+    float gate = 1.0f;
+    if (row < nt && e < E) {
+      src_row = tab.start_e + v - 1;
+      ok = v >= 1 && v <= tab.load_e && src_row < a.P;
+      if (ok && a.gates != nullptr)
+        gate = load_gate(a.gates, a.gate_dtype, static_cast<size_t>(t0 + row) * E + e);
+    }
+    // bit (i*ep + e) set <=> token i of this step has a valid route on path e;
+    // walking a token's bits from the lowest keeps the ascending path order
+    const unsigned long long m = __ballot(ok);
+    const int tokens = min(rps, nt - step * rps);
+    for (int tg = 0; tg < tokens; tg += G) {
+      unsigned long long rem0[G];
+      int kmax = 0;
+#pragma unroll
+      for (int i = 0; i < G; ++i) {
+        rem0[i] = (tg + i < tokens) ? ((m >> ((tg + i) * ep)) & seg0) << ((tg + i) * ep) : 0ull;
+        kmax = max(kmax, static_cast<int>(__popcll(rem0[i])));
+      }
+      for (int off0 = 0; off0 < cpr; off0 += kWave * UPR) {
+        float acc[G][UPR][NE];
+#pragma unroll
+        for (int i = 0; i < G; ++i)
+#pragma unroll
+          for (int u = 0; u < UPR; ++u)
+#pragma unroll
+            for (int q = 0; q < NE; ++q) acc[i][u][q] = 0.0f;
+        unsigned long long rem[G];
+#pragma unroll
+        for (int i = 0; i < G; ++i) rem[i] = rem0[i];
+        for (int k = 0; k < kmax; ++k) {
+          U val[G][UPR];
+          float g[G];
+          bool live[G];
+#pragma unroll
+          for (int i = 0; i < G; ++i) {
+            live[i] = rem[i] != 0;
+            g[i] = 1.0f;
+            if (live[i]) {
+              const int b = __builtin_ctzll(rem[i]);
+              rem[i] &= rem[i] - 1;
+              const int sr = read_lane(src_row, b);
+              g[i] = read_lane(gate, b);
+#pragma unroll
+              for (int u = 0; u < UPR; ++u) {
+                const int off = off0 + u * kWave + lane;
+                if (off < cpr) val[i][u] = src[static_cast<size_t>(sr) * cpr + off];
+              }
+            }
+          }
+#pragma unroll
+          for (int i = 0; i < G; ++i)
+            if (live[i]) {
+#pragma unroll
+              for (int u = 0; u < UPR; ++u) {
+                const int off = off0 + u * kWave + lane;
+                if (off < cpr) {
+                  float x[NE];
+                  unpack<IN_DT, BYTES>(val[i][u], x);
+                  // one rounding for the product, one for the sum (no fused multiply-add)
+#pragma unroll
+                  for (int q = 0; q < NE; ++q) acc[i][u][q] = acc[i][u][q] + x[q] * g[i];
+                }
+              }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < G; ++i) {
+          const bool routed = rem0[i] != 0;
+          if (tg + i < tokens && (routed || !a.is_residual)) {
+            const long t = t0 + step * rps + tg + i;
+#pragma unroll
+            for (int u = 0; u < UPR; ++u) {
+              const int off = off0 + u * kWave + lane;
+              if (off < cpr)
+                pack_store<OUT_DT, NE>(dst + (static_cast<size_t>(t) * cpr + off) * OUT_BYTES,
+                                       acc[i][u]);
+            }
+          }
+        }
+      }
+    }
+  }
+}
+
+// --------------------------------- lean kernels for the fused MoE fabrics
+// Seat indices, 1-d routing, no tag generation, E <= 64, 16-byte units: the
+// shape every fused_dispatch / fused_combine call has.  Same scheme as the
+// fast path above with everything optional compiled out.  A row is moved by a
+// group of LPR = 2^LS lanes (64 for rows of >= 64 units, fewer for short rows, so
+// that a wavefront moves 64/LPR rows at a time); each group walks the set bits
+// of its own token's slice of the ballot mask and fetches the destination row
+// from the lane that computed it with ds_bpermute.
+template <int DT, int LS, int UPR>
+__global__ __launch_bounds__(kBlock, 8) void dispatch_lean_kernel(DispatchArgs a) {
+  using U = u32x4;
+  constexpr int LPR = 1 << LS;
+  constexpr int GROUPS = kWave >> LS;
+  const int E = a.E;
+  const int lane = threadIdx.x & (kWave - 1);
+  const long wave = static_cast<long>(blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  const int ep_shift = a.map.ep_shift;
+  const int ep = 1 << ep_shift;
+  const int rps = kWave >> ep_shift;
+  const int e = lane & (ep - 1);
+  const int sub = lane >> ep_shift;
+  const int gidx = lane >> LS, glane = lane & (LPR - 1);
+  const unsigned long long seg0 = ep == kWave ? ~0ull : ((1ull << ep) - 1ull);
+
+  const long r0 = wave * a.rows_pw;
+  const int nr = static_cast<int>(max(0l, min(static_cast<long>(a.rows_pw), a.T - r0)));
+  const int n_steps = (nr + rps - 1) >> (6 - ep_shift);
+  const int* __restrict__ idx0 = a.idx + r0 * E;
+  const int cpr = a.cpr;
+  const U* __restrict__ src = static_cast<const U*>(a.src);
+  U* __restrict__ dst = static_cast<U*>(a.dst);
+
+  int v_next = (n_steps > 0 && sub < nr && e < E) ? idx0[sub * E + e] : 0;
+  const int my_count = (a.counts != nullptr && lane < E) ? a.counts[lane] : 0;
+  const SmallTables tab = small_tables(a.loads, E, a.mpl, ep_shift, lane);
+
+// In seat mode the source row of a token is the token itself, so its units are
+  // fetched before the index words have even arrived and are reused for every
+  // path the token is routed to (a top-k token is read once and stored k times).
+  auto load_units = [&](int i, int tokens, int step, int off0, U (&val)[UPR]) {
+    const size_t from = static_cast<size_t>(r0 + step * rps + i) * cpr;
+#pragma unroll
+    for (int u = 0; u < UPR; ++u) {
+      const int off = off0 + u * LPR + glane;
+      if (i < tokens && off < cpr) val[u] = src[from + off];
+    }
+  };
+
+  for (int step = 0; step < n_steps; ++step) {
+    const int tokens = min(rps, nr - step * rps);
+    U val[UPR];
+    load_units(gidx, tokens, step, 0, val);
+    const int v = v_next;
+    const int row = step * rps + sub;
+    {
+      const int nrow = row + rps;
+      v_next = (step + 1 < n_steps && nrow < nr && e < E) ? idx0[nrow * E + e] : 0;
+    }
+    const int dst_row = tab.start_e + v - 1;
+    const bool ok = row < nr && e < E && v >= 1 && v <= tab.load_e && dst_row < a.P;
+    float gate = 1.0f;
+    if constexpr (DT >= 0) {
+      if (ok) gate = load_gate(a.gates, DT, static_cast<size_t>(r0 + row) * E + e);
+    }
+    const unsigned long long m = __ballot(ok);
+    for (int tb = 0; tb < tokens; tb += GROUPS) {
+      const int i = tb + gidx;  // token of this lane group
+      const unsigned long long mine = i < tokens ? (m >> (i * ep)) & seg0 : 0ull;
+      for (int off0 = 0; off0 < cpr; off0 += LPR * UPR) {
+        if (tb != 0 || off0 != 0) load_units(i, tokens, step, off0, val);
+        unsigned long long rem = mine;
+        while (__ballot(rem != 0) != 0) {
+          const bool has = rem != 0;
+          const int b = i * ep + __builtin_ctzll(rem | (1ull << 63));
+          rem &= rem - 1;
+          const int d = __builtin_amdgcn_ds_bpermute(b << 2, dst_row);
+          float g = 1.0f;
+          if constexpr (DT >= 0)
+            g = __int_as_float(__builtin_amdgcn_ds_bpermute(b << 2, __float_as_int(gate)));
+#pragma unroll
+          for (int u = 0; u < UPR; ++u) {
+            const int off = off0 + u * LPR + glane;
+            if (has && off < cpr) {
+              U* to = dst + static_cast<size_t>(d) * cpr + off;
+              if constexpr (DT >= 0) {
+                constexpr int NE = 16 / elem_bytes(DT);
+                float x[NE];
+                unpack<DT, 16>(val[u], x);
+#pragma unroll
+                for (int q = 0; q < NE; ++q) x[q] = x[q] * g;
+                pack_store<DT, NE>(to, x);
+              } else {
+                *to = val[u];
+              }
+            }
+          }
+        }
+      }
+    }
+  }
+
+  if (a.counts != nullptr) {  // zero-fill this wavefront's share of the padding rows
+    const long n_waves = static_cast<long>(gridDim.x) * (blockDim.x >> 6);
+    int z = 0;
+    if (lane < E) {
+      const int alloc = a.mpl != 0 ? a.mpl : tab.my_load;
+      const int filled = max(0, min(min(my_count, tab.my_load), alloc));
+      z = max(0, alloc - filled);
+    }
+    const int z_incl = wave_inclusive_scan(z);
+    const long Z = read_lane(z_incl, kWave - 1);
+    const long z0 = Z * wave / n_waves;
+    const long z1 = Z * (wave + 1) / n_waves;
+    for (long zi = z0; zi < z1; ++zi) {
+      const int pe = __builtin_ctzll(__ballot(z_incl > zi));
+      const int pad = read_lane(z, pe);
+      const int alloc = a.mpl != 0 ? a.mpl : read_lane(tab.my_load, pe);
+      const long row = static_cast<long>(read_lane(tab.my_start, pe)) + (alloc - pad) +
+                       (zi - (read_lane(z_incl, pe) - pad));
+      if (row < a.P)
+        for (int o = lane; o < cpr; o += kWave) dst[static_cast<size_t>(row) * cpr + o] = zero_unit<16>();
+    }
+  }
+}
+
+template <int IN_DT, int OUT_DT, int LS, int UPR>
+__global__ __launch_bounds__(kBlock) void combine_lean_kernel(CombineArgs a) {
+  using U = u32x4;
+  constexpr int NE = 16 / elem_bytes(IN_DT);
+  constexpr int OUT_BYTES = NE * elem_bytes(OUT_DT);
+  constexpr int LPR = 1 << LS;
+  constexpr int GROUPS = kWave >> LS;
+  const int E = a.E;
+  const int lane = threadIdx.x & (kWave - 1);
+  const long wave = static_cast<long>(blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  const int ep_shift = a.map.ep_shift;
+  const int ep = 1 << ep_shift;
+  const int rps = kWave >> ep_shift;
+  const int e = lane & (ep - 1);
+  const int sub = lane >> ep_shift;
+  const int gidx = lane >> LS, glane = lane & (LPR - 1);
+  const unsigned long long seg0 = ep == kWave ? ~0ull : ((1ull << ep) - 1ull);
+
+  const long t0 = wave * a.rows_pw;
+  const int nt = static_cast<int>(max(0l, min(static_cast<long>(a.rows_pw), a.T - t0)));
+  if (nt == 0) return;
+  const int n_steps = (nt + rps - 1) >> (6 - ep_shift);
+  const int* __restrict__ idx0 = a.idx + t0 * E;
+  const int cpr = a.cpr;
+  const U* __restrict__ src = static_cast<const U*>(a.src);
+  char* __restrict__ dst = static_cast<char*>(a.dst);
+
+  int v_next = (sub < nt && e < E) ? idx0[sub * E + e] : 0;
+  const SmallTables tab = small_tables(a.loads, E, a.mpl, ep_shift, lane);
+
+  for (int step = 0; step < n_steps; ++step) {
+    const int v = v_next;
+    const int row = step * rps + sub;
+    {
+      const int nrow = row + rps;
+      v_next = (step + 1 < n_steps && nrow < nt && e < E) ? idx0[nrow * E + e] : 0;
+    }
+    const int src_row = tab.start_e + v - 1;
+    const bool ok = row < nt && e < E && v >= 1 && v <= tab.load_e && src_row < a.P;
+    float gate = 1.0f;
+    if (ok && a.gates != nullptr)
+      gate = load_gate(a.gates, a.gate_dtype, static_cast<size_t>(t0 + row) * E + e);
+    const unsigned long long m = __ballot(ok);
+    const int tokens = min(rps, nt - step * rps);
+    for (int tb = 0; tb < tokens; tb += GROUPS) {
+      const int i = tb + gidx;
+      const unsigned long long mine = i < tokens ? (m >> (i * ep)) & seg0 : 0ull;
+      const size_t to = static_cast<size_t>(t0 + step * rps + i) * cpr;
+      for (int off0 = 0; off0 < cpr; off0 += LPR * UPR) {
+        float acc[UPR][NE];
+#pragma unroll
+        for (int u = 0; u < UPR; ++u)
+#pragma unroll
+          for (int q = 0; q < NE; ++q) acc[u][q] = 0.0f;
+        unsigned long long rem = mine;
+        while (__ballot(rem != 0) != 0) {  // ascending path order: lowest set bit first
+          const bool has = rem != 0;
+          const int b = i * ep + __builtin_ctzll(rem | (1ull << 63));
+          rem &= rem - 1;
+          const int sr = __builtin_amdgcn_ds_bpermute(b << 2, src_row);
+          const float g = __int_as_float(__builtin_amdgcn_ds_bpermute(b << 2, __float_as_int(gate)));
+          U val[UPR];
+#pragma unroll
+          for (int u = 0; u < UPR; ++u) {
+            const int off = off0 + u * LPR + glane;
+            if (has && off < cpr) val[u] = src[static_cast<size_t>(sr) * cpr + off];
+          }
+#pragma unroll
+          for (int u = 0; u < UPR; ++u) {
+            const int off = off0 + u * LPR + glane;
+            if (has && off < cpr) {
+              float x[NE];
+              unpack<IN_DT, 16>(val[u], x);
+              // one rounding for the product, one for the sum (no fused multiply-add)
+#pragma unroll
+              for (int q = 0; q < NE; ++q) acc[u][q] = acc[u][q] + x[q] * g;
+            }
+          }
+        }
+        if (i < tokens && (mine != 0 || !a.is_residual)) {
+#pragma unroll
+          for (int u = 0; u < UPR; ++u) {
+            const int off = off0 + u * LPR + glane;
+            if (off < cpr) pack_store<OUT_DT, NE>(dst + (to + off) * OUT_BYTES, acc[u]);
+          }
+        }
       }
     }
   }
@@ -408,14 +1022,108 @@ int env_int(const char* name, int fallback) {
   return v ? atoi(v) : fallback;
 }
 
+StepMap make_step_map(int E) {
+  StepMap m{};
+  m.E = E;
+  m.chunks = E <= kWave ? 1 : (E + kWave - 1) / kWave;
+  int shift = 0;
+  while ((1 << shift) < std::min(E, kWave)) ++shift;
+  m.ep_shift = shift;
+  return m;
+}
+
+// Rows of the index matrix per wavefront: enough units that each lane has a
+// handful of 16-byte accesses in flight, few enough index words that one batch
+// of kSteps loads covers them.
+int rows_per_wave(const char* env, int cpr, int E, long T) {
+  int rows = env_int(env, 0);
+  if (rows <= 0) {
+    rows = std::max(1, 384 / std::max(cpr, 1));
+    while (rows > 1 && (T + rows - 1) / rows < 4096) rows >>= 1;  // keep every SIMD busy
+  }
+  const StepMap m = make_step_map(E);
+  if (E <= kWave) {  // register path: whole steps of 64 >> ep_shift rows
+    const int rps = kWave >> m.ep_shift;
+    return std::max(rps, rows / rps * rps);
+  }
+  rows = std::min(rows, std::max(1, kSteps / m.chunks));
+  rows = std::min(rows, std::max(1, 2048 / E));  // bounds the per-wave list in LDS
+  return std::max(1, rows);
+}
+
+struct LaunchShape {
+  int waves_pb, grid;
+  size_t lds;
+};
+
+// Packs as many wavefronts into a block as the LDS budget allows (at most 4).
+bool launch_shape(long T, int rows_pw, int lds_pw_ints, LaunchShape* out) {
+  const size_t per_wave = static_cast<size_t>(lds_pw_ints) * 4;
+  if (per_wave > 60 * 1024) return false;
+  int waves = std::max(1, std::min(kBlock / kWave, env_int("BRT_WAVES_PB", kBlock / kWave)));
+  while (waves > 1 && per_wave * waves > 60 * 1024) waves >>= 1;
+  const long n_waves = std::max(1l, (T + rows_pw - 1) / rows_pw);
+  out->waves_pb = waves;
+  out->grid = static_cast<int>((n_waves + waves - 1) / waves);
+  out->lds = per_wave * waves;
+  return true;
+}
+
+// Lanes per row (log2) and units per lane for the lean kernels.
+#define BRT_LEAN_SHAPES(LAUNCH)                        \
+  if (a.cpr > 2 * kWave) { LAUNCH(6, 4) }              \
+  else if (a.cpr > kWave) { LAUNCH(6, 2) }             \
+  else if (a.cpr > 32) { LAUNCH(6, 1) }                \
+  else if (a.cpr > 16) { LAUNCH(5, 1) }                \
+  else if (a.cpr > 8) { LAUNCH(4, 1) }                 \
+  else { LAUNCH(3, 1) }
+
 template <int BYTES, int DT>
-void launch_dispatch(const DispatchArgs& a, int grid, size_t lds, hipStream_t st) {
-  hipLaunchKernelGGL((dispatch_kernel<BYTES, DT>), dim3(grid), dim3(kBlock), lds, st, a);
+void launch_dispatch(const DispatchArgs& a, const LaunchShape& sh, hipStream_t st) {
+  const dim3 grid(sh.grid), block(sh.waves_pb * kWave);
+  if constexpr (BYTES == 16) {
+    if (a.E <= kWave && a.is_1d && !a.is_tag_index && a.new_tags == nullptr &&
+        env_int("BRT_NO_LEAN", 0) == 0) {
+#define BRT_LAUNCH(LS, UPR) \
+  hipLaunchKernelGGL((dispatch_lean_kernel<DT, LS, UPR>), grid, block, 0, st, a);
+      BRT_LEAN_SHAPES(BRT_LAUNCH)
+#undef BRT_LAUNCH
+      return;
+    }
+  }
+  if (a.E > kWave) {
+    hipLaunchKernelGGL((dispatch_kernel<BYTES, DT>), grid, block, sh.lds, st, a);
+  } else if (BYTES == 16 && a.cpr <= kWave) {
+    hipLaunchKernelGGL((dispatch_small_kernel<BYTES, DT, 1>), grid, block, 0, st, a);
+  } else if (BYTES == 16 && a.cpr <= 2 * kWave) {
+    hipLaunchKernelGGL((dispatch_small_kernel<BYTES, DT, 2>), grid, block, 0, st, a);
+  } else {
+    hipLaunchKernelGGL((dispatch_small_kernel<BYTES, DT, 4>), grid, block, 0, st, a);
+  }
 }
 
 template <int BYTES, int IN_DT, int OUT_DT>
-void launch_combine(const CombineArgs& a, int grid, size_t lds, hipStream_t st) {
-  hipLaunchKernelGGL((combine_kernel<BYTES, IN_DT, OUT_DT>), dim3(grid), dim3(kBlock), lds, st, a);
+void launch_combine(const CombineArgs& a, const LaunchShape& sh, hipStream_t st) {
+  const dim3 grid(sh.grid), block(sh.waves_pb * kWave);
+  if constexpr (BYTES == 16) {
+    if (a.E <= kWave && env_int("BRT_NO_LEAN", 0) == 0) {
+#define BRT_LAUNCH(LS, UPR) \
+  hipLaunchKernelGGL((combine_lean_kernel<IN_DT, OUT_DT, LS, UPR>), grid, block, 0, st, a);
+      if (env_int("BRT_COMBINE_UPR1", 0) && a.cpr > kWave) { BRT_LAUNCH(6, 1) return; }
+      BRT_LEAN_SHAPES(BRT_LAUNCH)
+#undef BRT_LAUNCH
+      return;
+    }
+  }
+  if (a.E > kWave) {
+    hipLaunchKernelGGL((combine_kernel<BYTES, IN_DT, OUT_DT>), grid, block, sh.lds, st, a);
+  } else if (BYTES == 16 && a.cpr <= kWave) {
+    hipLaunchKernelGGL((combine_small_kernel<BYTES, IN_DT, OUT_DT, 1>), grid, block, 0, st, a);
+  } else if (BYTES == 16 && a.cpr <= 2 * kWave) {
+    hipLaunchKernelGGL((combine_small_kernel<BYTES, IN_DT, OUT_DT, 2>), grid, block, 0, st, a);
+  } else {
+    hipLaunchKernelGGL((combine_small_kernel<BYTES, IN_DT, OUT_DT, 4>), grid, block, 0, st, a);
+  }
 }
 
 }  // namespace
@@ -452,29 +1160,20 @@ extern "C" int brt_hip_dispatch(const void* src, void* dst, const void* gates,
   a.T = T; a.E = E; a.P = P; a.mpl = max_path_load;
   a.cpr = static_cast<int>(row_bytes / bytes);
   a.is_1d = is_1d_routing; a.is_tag_index = is_tag_index;
-  // rows of the index matrix per block: enough row bytes to keep 256 threads busy,
-  // few enough that the grid covers the chip several times
-  int rows = env_int("BRT_DISPATCH_ROWS", 0);
-  if (rows <= 0) {
-    rows = static_cast<int>(std::max<size_t>(1, 16384 / std::max<size_t>(row_bytes, 1)));
-    rows = std::min(rows, 64);
-    while (rows > 1 && (T + rows - 1) / rows < 1024) rows >>= 1;
-  }
-  rows = std::max(1, std::min(rows, std::max(1, 4096 / E)));
-  a.rows_pb = rows;
-  a.list_cap = rows * E;
-  const size_t lds = (static_cast<size_t>(3) * E + 1 + 3 * static_cast<size_t>(a.list_cap)) * 4;
-  if (lds > 120 * 1024) return fail(BRT_E_UNSUPPORTED, "E=%d needs too much LDS", E);
-  const int grid = std::max(1, (T + rows - 1) / rows);
+  a.map = make_step_map(E);
+  a.rows_pw = rows_per_wave("BRT_DISPATCH_ROWS", a.cpr, E, T);
+  a.lds_pw = 3 * E + 1 + 3 * a.rows_pw * E;
+  LaunchShape sh;
+  if (!launch_shape(T, a.rows_pw, a.lds_pw, &sh))
+    return fail(BRT_E_UNSUPPORTED, "E=%d needs too much LDS", E);
   hipStream_t st = as_stream(stream);
 
 #define BRT_DISPATCH_CASE(B)                                               \
   case B:                                                                  \
-    if (gates == nullptr) launch_dispatch<B, -1>(a, grid, lds, st);         \
-    else if (dtype == BRT_F32) {                                           \
-      if constexpr (B >= 4) launch_dispatch<(B >= 4 ? B : 4), BRT_F32>(a, grid, lds, st); \
-    } else if (dtype == BRT_F16) launch_dispatch<B, BRT_F16>(a, grid, lds, st); \
-    else launch_dispatch<B, BRT_BF16>(a, grid, lds, st);                   \
+    if (gates == nullptr) launch_dispatch<B, -1>(a, sh, st);                \
+    else if (dtype == BRT_F32) launch_dispatch<(B >= 4 ? B : 4), BRT_F32>(a, sh, st); \
+    else if (dtype == BRT_F16) launch_dispatch<B, BRT_F16>(a, sh, st);     \
+    else launch_dispatch<B, BRT_BF16>(a, sh, st);                          \
     break;
   switch (bytes) {
     BRT_DISPATCH_CASE(16)
@@ -510,31 +1209,22 @@ extern "C" int brt_hip_combine(const void* src, void* dst, const void* gates,
   a.T = T; a.E = E; a.P = P; a.mpl = max_path_load;
   a.cpr = static_cast<int>(row_bytes / bytes);
   a.is_residual = is_residual; a.gate_dtype = gate_dtype;
-  int shift = 0;
-  while ((1 << shift) < std::min(E, 64)) ++shift;
-  a.ep_shift = shift;
-  int rows = env_int("BRT_COMBINE_ROWS", 0);
-  if (rows <= 0) {
-    rows = static_cast<int>(std::max<size_t>(1, 16384 / std::max<size_t>(row_bytes, 1)));
-    rows = std::min(rows, 64);
-    while (rows > 1 && (T + rows - 1) / rows < 1024) rows >>= 1;
-  }
-  rows = std::max(1, std::min(rows, std::max(1, 4096 / E)));
-  a.rows_pb = rows;
-  const size_t lds = (static_cast<size_t>(2) * E + rows + 2 * static_cast<size_t>(rows) * E) * 4;
-  if (lds > 120 * 1024) return fail(BRT_E_UNSUPPORTED, "E=%d needs too much LDS", E);
-  const int grid = (T + rows - 1) / rows;
+  a.map = make_step_map(E);
+  a.rows_pw = rows_per_wave("BRT_COMBINE_ROWS", a.cpr, E, T);
+  a.lds_pw = 2 * E + a.rows_pw + 2 * a.rows_pw * E;
+  LaunchShape sh;
+  if (!launch_shape(T, a.rows_pw, a.lds_pw, &sh))
+    return fail(BRT_E_UNSUPPORTED, "E=%d needs too much LDS", E);
   hipStream_t st = as_stream(stream);
 
-#define BRT_COMBINE_HALF(B, DT)                                              \
-  if (out_dtype == BRT_F32) launch_combine<B, DT, BRT_F32>(a, grid, lds, st); \
-  else launch_combine<B, DT, DT>(a, grid, lds, st);
-#define BRT_COMBINE_CASE(B)                                                  \
-  case B:                                                                    \
-    if (in_dtype == BRT_F32) {                                               \
-      if constexpr (B >= 4) launch_combine<(B >= 4 ? B : 4), BRT_F32, BRT_F32>(a, grid, lds, st); \
-    } else if (in_dtype == BRT_F16) { BRT_COMBINE_HALF(B, BRT_F16) }         \
-    else { BRT_COMBINE_HALF(B, BRT_BF16) }                                   \
+#define BRT_COMBINE_HALF(B, DT)                                        \
+  if (out_dtype == BRT_F32) launch_combine<B, DT, BRT_F32>(a, sh, st); \
+  else launch_combine<B, DT, DT>(a, sh, st);
+#define BRT_COMBINE_CASE(B)                                            \
+  case B:                                                              \
+    if (in_dtype == BRT_F32) launch_combine<(B >= 4 ? B : 4), BRT_F32, BRT_F32>(a, sh, st); \
+    else if (in_dtype == BRT_F16) { BRT_COMBINE_HALF(B, BRT_F16) }     \
+    else { BRT_COMBINE_HALF(B, BRT_BF16) }                             \
     break;
   switch (bytes) {
     BRT_COMBINE_CASE(16)

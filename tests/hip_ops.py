@@ -126,9 +126,11 @@ def dispatch(x_bits, idx, loads, gates_bits=None, counts=None, tag_generating=Fa
     if tag_generating:
         d_new = torch.full((P,), 0 if prezero else -9, dtype=torch.int32, device="cuda")
     d_old = None if tags is None else dev(np.asarray(tags, dtype=np.int32))
+    # device inputs stay referenced until the kernel has run
+    d_gates, d_idx, d_loads = dev(gates_bits), dev(idx), dev(loads)
+    d_counts = None if counts is None else dev(np.asarray(counts, dtype=np.int32))
     _lib.check(_lib.lib().brt_hip_dispatch(
-        ptr(d_x), ptr(d_out), ptr(dev(gates_bits)), ptr(dev(idx)), ptr(dev(loads)),
-        ptr(None if counts is None else dev(np.asarray(counts, dtype=np.int32))),
+        ptr(d_x), ptr(d_out), ptr(d_gates), ptr(d_idx), ptr(d_loads), ptr(d_counts),
         ptr(d_old), ptr(d_new), T, cell, E, P, max_path_load, int(is_1d), int(is_tag_index),
         DT[dtype], stream()))
     torch.cuda.synchronize()
@@ -151,9 +153,9 @@ def combine(y_bits, idx, loads, gates_bits=None, residual_bits=None, max_path_lo
         d_out = torch.full((T, cell), float("nan"), device="cuda")
     else:
         d_out = torch.full((T, cell), 0x55, dtype=torch.int16, device="cuda")
+    d_gates, d_idx, d_loads = dev(gates_bits), dev(idx), dev(np.asarray(loads, dtype=np.int32))
     _lib.check(_lib.lib().brt_hip_combine(
-        ptr(d_y), ptr(d_out), ptr(dev(gates_bits)), ptr(dev(idx)),
-        ptr(dev(np.asarray(loads, dtype=np.int32))), T, cell, E, P, max_path_load,
+        ptr(d_y), ptr(d_out), ptr(d_gates), ptr(d_idx), ptr(d_loads), T, cell, E, P, max_path_load,
         int(residual_bits is not None), DT[in_dtype], DT[out_dtype], DT[gate_dtype], stream()))
     torch.cuda.synchronize()
     return host(d_out, True)
