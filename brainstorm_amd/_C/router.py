@@ -54,12 +54,12 @@ _workspaces = {}
 
 
 def _scan_workspace(device: torch.device, T: int, E: int) -> torch.Tensor:
-    """Zero-initialised scan workspace, one per (device, stream), grown on demand."""
+    """Scratch memory of the index scan, one per (device, stream), grown on demand."""
     need = _lib.lib().brt_hip_scan_workspace_bytes(T, E)
     key = (device.index, _stream())
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < need:
-        ws = torch.zeros(max(need, 1 << 16), dtype=torch.uint8, device=device)
+        ws = torch.empty(max(need, 1 << 16), dtype=torch.uint8, device=device)
         _workspaces[key] = ws
     return ws
 

@@ -4,25 +4,34 @@
 // (generate_indices_and_loads :212-257, throttle_hotmask :59-130,
 // convert_*_indices :259-302); how it is computed does not.  The reference runs
 // one 1024-thread block per path and walks the mask column (stride E) in serial
-// 1024-row chunks.  Here the [T,E] mask is cut into row tiles that are read
-// ONCE with coalesced 128-bit loads, scanned per column inside LDS, and chained
-// across tiles with a single-pass decoupled look-back over per-(tile, column)
-// records, so the whole op is one launch that moves 4*T*E bytes in and 4*T*E
-// bytes out.
+// 1024-row chunks behind 20 block barriers each.
 //
-// Scan workspace layout (64-bit words):
-//   [0, kMaxStrips)      ticket of strip s: (epoch << 32) | next tile id
-//   [kMaxStrips]         sticky error flag (look-back spin bound exceeded)
-//   [kHeaderWords, ...)  records: rec[strip][tile][col] = (tag << 32) | value,
-//                        tag = (epoch << 2) | status, status 1 = tile aggregate,
-//                        2 = inclusive prefix up to and including the tile
-// A strip is a group of up to 256 adjacent columns; E <= 256 is one strip whose
-// tiles are contiguous in memory.  Tile ids are handed out by the ticket in
-// launch order, so a tile only ever waits for tiles that are already running.
-// The block that draws the last tile id re-arms the ticket with epoch+1; stale
-// records of earlier launches never match the current epoch, so the workspace
-// is zeroed once and then reused without clearing.
+// Here lanes are paths: a wavefront reads whole rows of the [T,E] mask with
+// coalesced loads (for E < 64 one load covers 64/ep rows, ep = E rounded up to a
+// power of two; for E > 64 the columns are walked in chunks of 64) and keeps the
+// per-path running sums in registers, so the seat of a row is one add and one
+// multiply per lane.  The rows are cut into bands, one per 4-wavefront
+// workgroup:
+//
+//   pass 1  band_count_kernel  per band and path: sum of the mask values
+//                              -> partial[band][path]
+//   pass 2  band_apply_kernel  offset of a band = sum of the partials of the
+//                              bands above it (a few KiB, cache resident; the
+//                              four wavefronts split that sum and exchange it,
+//                              together with their own column sums, through LDS
+//                              behind the kernel's only barrier), then the rows
+//                              are walked again and seats / throttled bits / tag
+//                              slots are written; the last band also emits
+//                              loads, counts and the throttle prefix.
+//
+// Two launches, no spinning and no state between calls: on this multi-die part
+// a device-scope flag takes about as long to become visible to the other dies
+// as a kernel boundary costs, so a single-pass chained scan buys nothing at MoE
+// sizes (a few MiB) and adds a way to hang.  Up to 16 rows per wavefront stay in
+// registers between the two walks of pass 2; longer bands re-read their rows
+// (from cache).  The indices are written exactly once.
 #include <algorithm>
+#include <cstdlib>
 
 #include "common.hpp"
 
@@ -30,44 +39,44 @@ namespace brt {
 namespace {
 
 constexpr int kBlock = 256;
-constexpr int kStripCols = 256;
-constexpr int kTileIntsMax = 8192;  // 32 KiB of LDS per tile
-constexpr int kTileIntsMin = 2048;
-constexpr int kMaxStrips = 64;
-constexpr int kHeaderWords = 128;  // 1 KiB
-constexpr int kWindowMax = 16;     // look-back records fetched per thread and round
-constexpr int kSpinLimit = 1 << 20;
+constexpr int kWavesPB = kBlock / kWave;
+constexpr int kBatch = 16;         // row loads in flight per lane
+constexpr int kPartialBatch = 32;  // loads of earlier bands' sums in flight per lane
+constexpr int kMaxBands = 512;
 
 enum { kSeat = 0, kTag = 1, kThrottle = 2 };
 
-typedef int v4i __attribute__((ext_vector_type(4)));  // one 128-bit access
-
 struct ScanGeometry {
-  int strips;     // column strips
-  int strip_cols; // columns per strip (last strip may hold fewer)
-  int tile_rows;  // rows per tile (multiple of 4)
-  int tiles;      // tiles per strip
-  int chunk_rows; // rows scanned by one thread
+  int ep_shift;  // log2 of the lanes one row occupies (E <= 64), 6 otherwise
+  int rows_pw;   // rows per wavefront (multiple of the rows one load covers)
+  int bands;     // workgroups
 };
+
+int env_int(const char* name, int fallback) {
+  const char* v = getenv(name);
+  return v ? atoi(v) : fallback;
+}
 
 ScanGeometry scan_geometry(int T, int E) {
   ScanGeometry g;
-  g.strip_cols = std::min(E, kStripCols);
-  g.strips = (E + kStripCols - 1) / kStripCols;
-  // Large tiles keep the look-back short (each tile publishes strip_cols
-  // records); small problems get smaller tiles so that more CUs take part.
-  long total = static_cast<long>(T) * g.strip_cols;
-  int tile_ints = kTileIntsMax;
-  while (tile_ints > kTileIntsMin && total / tile_ints < 96) tile_ints >>= 1;
-  int rows = std::max(4, (tile_ints / g.strip_cols) & ~3);
-  g.tile_rows = rows;
-  g.tiles = std::max(1, (T + rows - 1) / rows);
-  const int slots = kBlock / g.strip_cols;  // row chunks scanned in parallel
-  int chunk = (rows + slots - 1) / slots;
-  // For narrow strips several row chunks share a wavefront; an odd chunk length
-  // spreads their LDS addresses over the banks.
-  if (g.strip_cols < 32 && (chunk & 1) == 0) chunk += 1;
-  g.chunk_rows = chunk;
+  int shift = 0;
+  while ((1 << shift) < std::min(E, kWave)) ++shift;
+  g.ep_shift = shift;
+  const int rps = kWave >> shift;  // rows per load instruction
+  // Enough bands that a wavefront's rows fit one batch of loads, at least 128 (so
+  // that many CUs take part) and never more than kMaxBands, which bounds the sum
+  // over earlier bands every band has to form.
+  const long one_batch = static_cast<long>(kWavesPB) * kBatch * rps;
+  const int fit = static_cast<int>(std::min<long>(kMaxBands, (T + one_batch - 1) / one_batch));
+  const int want = env_int("BRT_SCAN_BANDS", std::max(128, fit));
+  long rows_pb = (static_cast<long>(T) + want - 1) / want;
+  rows_pb = std::max<long>(rows_pb, (static_cast<long>(T) + kMaxBands - 1) / kMaxBands);
+  long rows_pw = (rows_pb + kWavesPB - 1) / kWavesPB;
+  rows_pw = (rows_pw + rps - 1) / rps * rps;
+  rows_pw = std::max<long>(rows_pw, rps);
+  g.rows_pw = static_cast<int>(rows_pw);
+  const long per_band = rows_pw * kWavesPB;
+  g.bands = static_cast<int>(std::max(1l, (static_cast<long>(T) + per_band - 1) / per_band));
   return g;
 }
 
@@ -77,22 +86,14 @@ struct ScanArgs {
   int* loads;
   int* counts;
   const int* caps;
-  int* prefix;            // throttle only, updated in place
-  const int* threshold;   // throttle only
-  unsigned long long* ws;
+  int* prefix;           // throttle only, updated in place
+  const int* threshold;  // throttle only
+  int* partial;          // [bands][E] per-band column sums
+  int* prefix_in;        // throttle only: copy of prefix taken by pass 1 ([E])
   int T, E, C;
   int capacity_padding, path_wise_padding;
-  int tile_rows, tiles, strip_cols, chunk_rows;
-  int first_window;  // records per thread in the first look-back round
-  int vec_ok;        // mask/out 16-byte aligned -> 128-bit tile copies
+  int ep_shift, rows_pw, bands;
 };
-
-__device__ __forceinline__ unsigned long long ld_record(unsigned long long* p) {
-  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ void st_record(unsigned long long* p, unsigned long long v) {
-  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
 
 __device__ __forceinline__ int finalize_load(int real, const int* caps, int C, int cap_pad,
                                              int path_pad, int col) {
@@ -104,231 +105,186 @@ __device__ __forceinline__ int finalize_load(int real, const int* caps, int C, i
   return caps[C - 1];
 }
 
+// Sum over the lanes that hold the same path (lanes e, e+ep, e+2ep, ...); every
+// lane ends up with the total.
+__device__ __forceinline__ int sum_over_rows_in_wave(int v, int ep_shift) {
+  for (int d = 1 << ep_shift; d < kWave; d <<= 1) v += __shfl_xor(v, d, kWave);
+  return v;
+}
+
+// Second walk over one batch of row words held in registers: turns the mask words
+// into seats / throttled bits / tag slots.  Rows of one load are ordered by lane
+// group; all cross-lane traffic of the batch is issued first and does not depend
+// on the running sum (incl = sum over the groups up to and including this
+// lane's, tot = sum over all groups).
 template <int MODE>
-__global__ __launch_bounds__(kBlock) void scan_kernel(ScanArgs a) {
-  __shared__ __attribute__((aligned(16))) int s_tile[kTileIntsMax];
-  __shared__ int s_cnt[kBlock];     // per (row chunk, column) local sums
-  __shared__ int s_agg[kStripCols]; // tile aggregate per column
-  __shared__ int s_acc[kStripCols]; // exclusive prefix of earlier tiles per column
-  __shared__ int s_hi[kStripCols];  // nearest earlier tile not yet consumed
-  __shared__ int s_done[kStripCols];
-  __shared__ int s_psum[kBlock];
-  __shared__ int s_pflag[kBlock];
-  __shared__ int s_pre[kStripCols]; // throttle: incoming prefix
-  __shared__ int s_thr[kStripCols]; // throttle: threshold
-  __shared__ unsigned long long s_ticket;
-
-  const int tid = threadIdx.x;
-  const int strip = blockIdx.y;
-  const int col0 = strip * kStripCols;
-  const int cw = min(kStripCols, a.E - col0);  // columns of this strip
-  const int E = a.E;
-
-  if (tid == 0) {
-    s_ticket = __hip_atomic_fetch_add(a.ws + strip, 1ull, __ATOMIC_RELAXED,
-                                      __HIP_MEMORY_SCOPE_AGENT);
-  }
-  if (MODE == kThrottle && tid < cw) {
-    s_pre[tid] = a.prefix[col0 + tid];
-    s_thr[tid] = a.threshold[col0 + tid];
-  }
-  __syncthreads();
-  const unsigned long long ticket = s_ticket;
-  const int tile = static_cast<int>(ticket & 0xffffffffull);
-  const unsigned epoch = static_cast<unsigned>(ticket >> 32);
-  if (tile >= a.tiles) return;  // workspace was not prepared; never happens in normal use
-  if (tid == 0 && tile == a.tiles - 1) {
-    // every other block of this strip has drawn its ticket already
-    st_record(a.ws + strip, static_cast<unsigned long long>(epoch + 1u) << 32);
-  }
-  const unsigned tag_agg = ((epoch & 0x3fffffffu) << 2) | 1u;
-  const unsigned tag_pre = ((epoch & 0x3fffffffu) << 2) | 2u;
-  unsigned long long* rec =
-      a.ws + kHeaderWords + static_cast<size_t>(strip) * a.tiles * a.strip_cols;
-
-  const int row0 = tile * a.tile_rows;
-  const int rows = min(a.tile_rows, a.T - row0);
-  const int n = rows * cw;
-  const bool contiguous = (cw == E);
-
-  // ---- 1. tile -> LDS ---------------------------------------------------------
-  if (contiguous && a.vec_ok) {
-    const v4i* src4 = reinterpret_cast<const v4i*>(a.mask + static_cast<size_t>(row0) * E);
-    v4i* lds4 = reinterpret_cast<v4i*>(s_tile);
-    const int nvec = n >> 2;
-    constexpr int kIter = kTileIntsMax / (kBlock * 4);
-    v4i r[kIter];
+__device__ __forceinline__ void walk_batch(const int (&m)[kBatch], int i0, int n_ins, int& carry,
+                                           int thr, long row_w, int rps, int ep, int sub, int e,
+                                           int lane, int col, bool col_ok, const ScanArgs& a) {
+  int incl[kBatch], tot[kBatch];
 #pragma unroll
-    for (int k = 0; k < kIter; ++k) {
-      const int i = tid + k * kBlock;
-      if (i < nvec) r[k] = __builtin_nontemporal_load(src4 + i);
-    }
-#pragma unroll
-    for (int k = 0; k < kIter; ++k) {
-      const int i = tid + k * kBlock;
-      if (i < nvec) lds4[i] = r[k];
-    }
-    for (int i = (nvec << 2) + tid; i < n; i += kBlock)
-      s_tile[i] = a.mask[static_cast<size_t>(row0) * E + i];
-  } else {
-    for (int i = tid; i < n; i += kBlock) {
-      const int r = i / cw, c = i - r * cw;
-      s_tile[i] = a.mask[static_cast<size_t>(row0 + r) * E + col0 + c];
-    }
-  }
-  __syncthreads();
-
-  // ---- 2. per-column scan inside the tile --------------------------------------
-  // thread = (row chunk s, column c); consecutive lanes touch consecutive LDS words
-  const int s = tid / cw, c = tid - s * cw;
-  const int r_begin = s * a.chunk_rows;
-  const int r_end = min(rows, r_begin + a.chunk_rows);
-  const bool scanning = r_begin < rows && s * cw + cw <= kBlock;
-  int local = 0;
-  if (scanning)
-    for (int r = r_begin; r < r_end; ++r) local += s_tile[r * cw + c];
-  s_cnt[tid] = scanning ? local : 0;
-  __syncthreads();
-  int offset = 0;  // sum of the chunks above this one in the same column
-  if (scanning)
-    for (int k = 0; k < s; ++k) offset += s_cnt[k * cw + c];
-  if (tid < cw) {
-    int total = 0;
-    const int slots = kBlock / cw;
-    for (int k = 0; k < slots; ++k) total += s_cnt[k * cw + tid];
-    s_agg[tid] = total;
-    s_acc[tid] = 0;
-    s_hi[tid] = tile - 1;
-    s_done[tid] = (tile == 0);
-    // publish: tile 0 knows its inclusive prefix already
-    st_record(rec + static_cast<size_t>(tile) * a.strip_cols + tid,
-              (static_cast<unsigned long long>(tile == 0 ? tag_pre : tag_agg) << 32) |
-                  static_cast<unsigned>(total));
-  }
-  __syncthreads();
-
-  // ---- 3. decoupled look-back over earlier tiles ---------------------------------
-  if (tile > 0) {
-    const int W = kBlock / cw;  // threads cooperating on one column
-    const int w = s;
-    for (int round = 0;; ++round) {
-      const int U = round == 0 ? a.first_window : kWindowMax;
-      if (w < W && !s_done[c]) {
-        const int near = s_hi[c] - w * U;  // this thread covers tiles near, near-1, ...
-        unsigned long long r[kWindowMax];
-#pragma unroll
-        for (int u = 0; u < kWindowMax; ++u) {
-          const int j = near - u;
-          if (u < U && j >= 0) r[u] = ld_record(rec + static_cast<size_t>(j) * a.strip_cols + c);
-        }
-        int sum = 0, flag = 0;  // flag: 0 all aggregates, 1 reached a prefix, 2 not ready
-#pragma unroll
-        for (int u = 0; u < kWindowMax; ++u) {
-          const int j = near - u;
-          if (u < U && flag == 0) {
-            if (j < 0) {
-              flag = 1;  // ran past tile 0: nothing more to add
-            } else {
-              const unsigned tag = static_cast<unsigned>(r[u] >> 32);
-              const int val = static_cast<int>(r[u] & 0xffffffffull);
-              if (tag == tag_agg) {
-                sum += val;
-              } else if (tag == tag_pre) {
-                sum += val;
-                flag = 1;
-              } else {
-                flag = 2;
-              }
-            }
-          }
-        }
-        s_psum[tid] = sum;
-        s_pflag[tid] = flag;
+  for (int u = 0; u < kBatch; ++u) {
+    incl[u] = m[u];
+    tot[u] = m[u];
+    if (rps > 1 && i0 + u < n_ins) {  // wave-uniform
+      int x = m[u];
+      for (int d = ep; d < kWave; d <<= 1) {
+        const int t = __shfl_up(x, d, kWave);
+        if (lane >= d) x += t;
       }
-      __syncthreads();
-      if (tid < cw && !s_done[tid]) {
-        int total = 0, state = 0;
-        for (int k = 0; k < W; ++k) {
-          const int f = s_pflag[k * cw + tid];
-          if (f == 2) {
-            state = 2;
-            break;
-          }
-          total += s_psum[k * cw + tid];
-          if (f == 1) {
-            state = 1;
-            break;
-          }
-        }
-        if (state != 2) {  // state 2: a record was not published yet, poll again
-          s_acc[tid] += total;
-          if (state == 1)
-            s_done[tid] = 1;
-          else
-            s_hi[tid] -= W * U;
-        }
-      }
-      const int pending = __syncthreads_count(tid < cw && !s_done[tid]);
-      if (pending == 0) break;
-      if (round >= kSpinLimit) {  // give up instead of hanging; result is invalid
-        if (tid == 0) st_record(a.ws + kMaxStrips, 1ull);
-        break;
-      }
-      __builtin_amdgcn_s_sleep(1);
-    }
-    if (tid < cw) {
-      st_record(rec + static_cast<size_t>(tile) * a.strip_cols + tid,
-                (static_cast<unsigned long long>(tag_pre) << 32) |
-                    static_cast<unsigned>(s_acc[tid] + s_agg[tid]));
+      incl[u] = x;
+      tot[u] = __shfl(x, (rps - 1) * ep + e, kWave);
     }
   }
-
-  // ---- 4. rewrite the tile in LDS (or scatter tags) --------------------------------
-  if (scanning) {
-    int run = s_acc[c] + offset;
-    if (MODE == kThrottle) run += s_pre[c];
-    const int thr = MODE == kThrottle ? s_thr[c] : 0;
-    for (int r = r_begin; r < r_end; ++r) {
-      const int m = s_tile[r * cw + c];
-      run += m;
+#pragma unroll
+  for (int u = 0; u < kBatch; ++u) {
+    const int run = carry + incl[u];
+    carry += tot[u];
+    const long r = row_w + static_cast<long>(i0 + u) * rps + sub;
+    if (i0 + u < n_ins && col_ok && r < a.T) {
       if (MODE == kSeat) {
-        s_tile[r * cw + c] = run * m;
+        a.out[r * a.E + col] = run * m[u];  // location * mask, location.cu:177-178
       } else if (MODE == kThrottle) {
-        s_tile[r * cw + c] = (m == 1 && run <= thr) ? 1 : 0;
+        a.out[r * a.E + col] = (m[u] == 1 && run <= thr) ? 1 : 0;
       } else {
-        const int index = run * m;
+        const int index = run * m[u];
         if (index >= 1 && index <= a.T)
-          a.out[static_cast<size_t>(index - 1) * E + col0 + c] = row0 + r + 1;
+          a.out[static_cast<size_t>(index - 1) * a.E + col] = static_cast<int>(r) + 1;
       }
     }
   }
+}
 
-  // ---- 5. totals: loads / counts / throttle prefix (last tile only) ------------------
-  if (tile == a.tiles - 1 && tid < cw) {
-    const int total = s_acc[tid] + s_agg[tid];
-    if (MODE == kThrottle) {
-      a.prefix[col0 + tid] = min(s_pre[tid] + total, s_thr[tid]);
-    } else {
-      a.loads[col0 + tid] =
-          finalize_load(total, a.caps, a.C, a.capacity_padding, a.path_wise_padding, col0 + tid);
-      if (a.counts) a.counts[col0 + tid] = total;
+// Loads one batch of row words (zero beyond the band / the matrix).
+__device__ __forceinline__ void load_batch(int (&v)[kBatch], int i0, int n_ins, long row_w, int rps,
+                                           int sub, int col, bool col_ok, const ScanArgs& a) {
+#pragma unroll
+  for (int u = 0; u < kBatch; ++u) {
+    const long r = row_w + static_cast<long>(i0 + u) * rps + sub;
+    v[u] = (i0 + u < n_ins && col_ok && r < a.T) ? a.mask[r * a.E + col] : 0;
+  }
+}
+
+// pass 1: column sums of one band
+__global__ __launch_bounds__(kBlock) void band_count_kernel(ScanArgs a) {
+  __shared__ int s_sum[kWavesPB][kWave];
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
+  const int E = a.E;
+  const int ep = 1 << a.ep_shift, rps = kWave >> a.ep_shift;
+  const int e = lane & (ep - 1), sub = lane >> a.ep_shift;
+  const long row_w = (static_cast<long>(blockIdx.x) * kWavesPB + wave) * a.rows_pw;
+  const int n_ins = a.rows_pw / rps;
+  for (int c0 = 0; c0 < E; c0 += kWave) {
+    const int col = c0 + e;
+    const bool col_ok = col < E;
+    int sum = 0;
+    for (int i0 = 0; i0 < n_ins; i0 += kBatch) {
+      int v[kBatch];
+#pragma unroll
+      for (int u = 0; u < kBatch; ++u) {
+        const long r = row_w + static_cast<long>(i0 + u) * rps + sub;
+        v[u] = (i0 + u < n_ins && col_ok && r < a.T) ? a.mask[r * E + col] : 0;
+      }
+#pragma unroll
+      for (int u = 0; u < kBatch; ++u) sum += v[u];
+    }
+    sum = sum_over_rows_in_wave(sum, a.ep_shift);
+    if (c0 > 0) __syncthreads();
+    if (sub == 0) s_sum[wave][e] = sum;
+    __syncthreads();
+    if (tid < kWave && c0 + tid < E) {
+      int total = 0;
+#pragma unroll
+      for (int k = 0; k < kWavesPB; ++k) total += s_sum[k][tid];
+      a.partial[static_cast<size_t>(blockIdx.x) * E + c0 + tid] = total;
+      // pass 2 overwrites prefix[] while other bands may not have started yet
+      if (a.prefix != nullptr && blockIdx.x == 0) a.prefix_in[c0 + tid] = a.prefix[c0 + tid];
     }
   }
-  if (MODE == kTag) return;
-  __syncthreads();
+}
 
-  // ---- 6. LDS -> out -------------------------------------------------------------------
-  if (contiguous && a.vec_ok) {
-    v4i* dst4 = reinterpret_cast<v4i*>(a.out + static_cast<size_t>(row0) * E);
-    const v4i* lds4 = reinterpret_cast<const v4i*>(s_tile);
-    const int nvec = n >> 2;
-    for (int i = tid; i < nvec; i += kBlock) dst4[i] = lds4[i];
-    for (int i = (nvec << 2) + tid; i < n; i += kBlock)
-      a.out[static_cast<size_t>(row0) * E + i] = s_tile[i];
-  } else {
-    for (int i = tid; i < n; i += kBlock) {
-      const int r = i / cw, cc = i - r * cw;
-      a.out[static_cast<size_t>(row0 + r) * E + col0 + cc] = s_tile[i];
+// pass 2: offsets from the bands above, running sums in registers, results out
+template <int MODE>
+__global__ __launch_bounds__(kBlock) void band_apply_kernel(ScanArgs a) {
+  __shared__ int s_above[kWavesPB][kWave];  // each wave's share of the sum over earlier bands
+  __shared__ int s_own[kWavesPB][kWave];    // column sums of each wave's own rows
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
+  const int E = a.E, band = blockIdx.x;
+  const int ep = 1 << a.ep_shift, rps = kWave >> a.ep_shift;
+  const int e = lane & (ep - 1), sub = lane >> a.ep_shift;
+  const long row_w = (static_cast<long>(band) * kWavesPB + wave) * a.rows_pw;
+  const int n_ins = a.rows_pw / rps;
+
+  for (int c0 = 0; c0 < E; c0 += kWave) {
+    const int col = c0 + e;
+    const bool col_ok = col < E;
+    // ---- own rows: the first batch stays in registers ---------------------------------
+    int m0[kBatch];
+    load_batch(m0, 0, n_ins, row_w, rps, sub, col, col_ok, a);
+    // ---- this wave's share of the offset: bands wave, wave+4, ... above this one ----
+    int above = 0;
+    for (int j0 = wave + sub * kWavesPB; j0 < band; j0 += kWavesPB * rps * kPartialBatch) {
+      int v[kPartialBatch];
+#pragma unroll
+      for (int u = 0; u < kPartialBatch; ++u) {
+        const int j = j0 + u * kWavesPB * rps;
+        v[u] = (j < band && col_ok) ? a.partial[static_cast<size_t>(j) * E + col] : 0;
+      }
+#pragma unroll
+      for (int u = 0; u < kPartialBatch; ++u) above += v[u];
+    }
+    int own = 0;
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) own += m0[u];
+    for (int i0 = kBatch; i0 < n_ins; i0 += kBatch) {
+      int v[kBatch];
+      load_batch(v, i0, n_ins, row_w, rps, sub, col, col_ok, a);
+#pragma unroll
+      for (int u = 0; u < kBatch; ++u) own += v[u];
+    }
+    above = sum_over_rows_in_wave(above, a.ep_shift);
+    own = sum_over_rows_in_wave(own, a.ep_shift);
+    if (c0 > 0) __syncthreads();
+    if (sub == 0) {
+      s_above[wave][e] = above;
+      s_own[wave][e] = own;
+    }
+    __syncthreads();
+    int carry = 0, band_total = 0;
+#pragma unroll
+    for (int k = 0; k < kWavesPB; ++k) {
+      carry += s_above[k][e];
+      band_total += s_own[k][e];
+      if (k < wave) carry += s_own[k][e];
+    }
+    band_total += carry;
+#pragma unroll
+    for (int k = 0; k < kWavesPB; ++k)
+      if (k < wave) band_total -= s_own[k][e];  // = offset + all four waves
+    int thr = 0, pre_in = 0;
+    if (MODE == kThrottle && col_ok) {
+      pre_in = (a.bands > 1 ? a.prefix_in : a.prefix)[col];
+      thr = a.threshold[col];
+      carry += pre_in;
+    }
+
+    // ---- walk the rows again: running sum per path, one result per element ----------
+    walk_batch<MODE>(m0, 0, n_ins, carry, thr, row_w, rps, ep, sub, e, lane, col, col_ok, a);
+    for (int i0 = kBatch; i0 < n_ins; i0 += kBatch) {
+      int v[kBatch];
+      load_batch(v, i0, n_ins, row_w, rps, sub, col, col_ok, a);
+      walk_batch<MODE>(v, i0, n_ins, carry, thr, row_w, rps, ep, sub, e, lane, col, col_ok, a);
+    }
+
+    // ---- totals: loads / counts / throttle prefix (last band only) ---------------------
+    if (band == a.bands - 1 && wave == 0 && sub == 0 && col_ok) {
+      if (MODE == kThrottle) {
+        a.prefix[col] = min(band_total + pre_in, thr);
+      } else {
+        a.loads[col] =
+            finalize_load(band_total, a.caps, a.C, a.capacity_padding, a.path_wise_padding, col);
+        if (a.counts) a.counts[col] = band_total;
+      }
     }
   }
 }
@@ -376,33 +332,27 @@ __global__ __launch_bounds__(256) void tag_to_seat_kernel(const int* __restrict_
 
 int launch_scan(int mode, ScanArgs& a, void* workspace, size_t workspace_bytes, void* stream) {
   const ScanGeometry g = scan_geometry(a.T, a.E);
-  if (g.strips > kMaxStrips) return fail(BRT_E_UNSUPPORTED, "E=%d exceeds %d paths", a.E,
-                                         kMaxStrips * kStripCols);
   const size_t need = brt_hip_scan_workspace_bytes(a.T, a.E);
   if (workspace == nullptr || workspace_bytes < need)
     return fail(BRT_E_WORKSPACE, "scan workspace too small: %zu < %zu bytes", workspace_bytes,
                 need);
-  if (!aligned(workspace, 8)) return fail(BRT_E_INVALID, "scan workspace must be 8-byte aligned");
-  a.ws = static_cast<unsigned long long*>(workspace);
-  a.tile_rows = g.tile_rows;
-  a.tiles = g.tiles;
-  a.strip_cols = g.strip_cols;
-  a.chunk_rows = g.chunk_rows;
-  // When every tile is resident at once, nobody has an inclusive prefix yet on
-  // the first poll, so fetch a wide window straight away; in a long stream of
-  // tiles the nearest predecessors have usually finished and a narrow first
-  // window saves record traffic.
-  a.first_window = g.tiles <= 1024 ? kWindowMax : 2;
-  a.vec_ok = aligned(a.mask, 16) && aligned(a.out, 16);
-  const dim3 grid(g.tiles, g.strips);
+  if (!aligned(workspace, 4)) return fail(BRT_E_INVALID, "scan workspace must be 4-byte aligned");
+  a.partial = static_cast<int*>(workspace);
+  a.prefix_in = a.partial + static_cast<size_t>(g.bands) * a.E;
+  a.ep_shift = g.ep_shift;
+  a.rows_pw = g.rows_pw;
+  a.bands = g.bands;
+  const dim3 grid(g.bands);
   hipStream_t st = as_stream(stream);
+  if (g.bands > 1)  // a single band has nothing above it
+    hipLaunchKernelGGL(band_count_kernel, grid, dim3(kBlock), 0, st, a);
   if (mode == kSeat)
-    hipLaunchKernelGGL(scan_kernel<kSeat>, grid, dim3(kBlock), 0, st, a);
+    hipLaunchKernelGGL(band_apply_kernel<kSeat>, grid, dim3(kBlock), 0, st, a);
   else if (mode == kTag)
-    hipLaunchKernelGGL(scan_kernel<kTag>, grid, dim3(kBlock), 0, st, a);
+    hipLaunchKernelGGL(band_apply_kernel<kTag>, grid, dim3(kBlock), 0, st, a);
   else
-    hipLaunchKernelGGL(scan_kernel<kThrottle>, grid, dim3(kBlock), 0, st, a);
-  return check_launch("scan_kernel");
+    hipLaunchKernelGGL(band_apply_kernel<kThrottle>, grid, dim3(kBlock), 0, st, a);
+  return check_launch("band_apply_kernel");
 }
 
 }  // namespace
@@ -411,10 +361,9 @@ int launch_scan(int mode, ScanArgs& a, void* workspace, size_t workspace_bytes, 
 using namespace brt;
 
 extern "C" size_t brt_hip_scan_workspace_bytes(int T, int E) {
-  if (T <= 0 || E <= 0) return kHeaderWords * 8;
+  if (T <= 0 || E <= 0) return 0;
   const ScanGeometry g = scan_geometry(T, E);
-  return (static_cast<size_t>(kHeaderWords) +
-          static_cast<size_t>(g.strips) * g.tiles * g.strip_cols) * 8;
+  return (static_cast<size_t>(g.bands) + 1) * E * sizeof(int);
 }
 
 extern "C" int brt_hip_generate_indices_and_loads(const int32_t* mask, int32_t* indices,

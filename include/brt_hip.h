@@ -45,10 +45,10 @@ const char* brt_hip_last_error(void);
 const char* brt_hip_version(void);
 
 /*
- * Bytes of scan workspace needed by brt_hip_generate_indices_and_loads /
- * brt_hip_throttle_hotmask for a [T,E] mask.  The workspace must be
- * zero-filled ONCE after allocation; the kernels leave it reusable (records
- * are stamped with a launch epoch kept inside the workspace).  One workspace
+ * Bytes of scratch memory brt_hip_generate_indices_and_loads /
+ * brt_hip_throttle_hotmask need for a [T,E] mask (per-band column sums handed
+ * from their first to their second kernel).  The content needs no
+ * initialisation and carries nothing from one call to the next; one workspace
  * must not be used by two calls that can run concurrently (two streams).
  */
 size_t brt_hip_scan_workspace_bytes(int T, int E);

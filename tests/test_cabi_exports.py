@@ -26,10 +26,10 @@ def test_library_exports_every_declared_symbol():
 
 def test_workspace_size_is_monotonic_and_small():
     f = _lib.lib().brt_hip_scan_workspace_bytes
-    assert f(0, 8) == f(0, 64) == 1024
-    assert f(8192, 64) >= 1024 + 64 * 8 * 8
+    assert f(0, 8) == f(0, 64) == 0
+    assert f(8192, 64) >= 2 * 64 * 4
     assert f(100352, 8) < 1 << 20
-    assert f(1 << 20, 64) < 64 << 20
+    assert f(1 << 20, 64) < 1 << 20
 
 
 def test_argument_errors_do_not_need_a_gpu():
