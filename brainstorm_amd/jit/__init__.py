@@ -1,0 +1,120 @@
+"""``brt.jit``: the homo-fused expert kernel as one grouped GEMM.
+
+The reference glues per-capacity TVM-tuned fp32 ``Linear`` kernels into one NVRTC
+kernel and launches it through ``brt._C.jit.homo_invoke``
+(python/brt/jit/factory.py:28-44, python/brt/jit/compiler.py:29-31,
+src/jit/compiler.cu:151-246).  Here ``make_jit_kernel(..., opt_level="homo_fuse")``
+returns a callable with the same shape
+
+    kernel(shared_inputs=[x, out], standalone_inputs=[w0, (b0,) w1, ...], capacities=loads)
+
+that runs ONE hand-written bf16 MFMA grouped GEMM over all branches; the loads
+are read on the device, need not come from a menu of compiled capacities, and no
+host copy or per-launch pointer shuffling happens.  Other fusion levels of the
+reference (horizontal / hetero fusion, the TVM kernel database) are not part of
+this build.
+"""
+from typing import Callable, List, Optional, Sequence, Union
+
+import torch
+import torch.nn as nn
+
+from brainstorm_amd import _lib
+
+__all__ = ["make_jit_kernel", "grouped_linear", "GroupedLinearKernel"]
+
+_ACT = {None: _lib.ACT_NONE, "none": _lib.ACT_NONE, "gelu": _lib.ACT_GELU, "relu": _lib.ACT_RELU}
+
+
+class _PointerTable:
+    """Device array of per-branch pointers, rebuilt only when the tensors change."""
+
+    def __init__(self):
+        self.key = None
+        self.table = None
+
+    def get(self, tensors: Sequence[torch.Tensor]) -> torch.Tensor:
+        key = tuple(t.data_ptr() for t in tensors)
+        if key != self.key:
+            self.table = torch.tensor(key, dtype=torch.int64, device=tensors[0].device)
+            self.key = key
+        return self.table
+
+
+def grouped_linear(x: torch.Tensor, out: torch.Tensor, weight_table: torch.Tensor,
+                   bias_table: Optional[torch.Tensor], loads: torch.Tensor, in_features: int,
+                   out_features: int, activation: Optional[str] = None) -> torch.Tensor:
+    """``out[s_e : s_e + loads[e]] = act(x[s_e : s_e + loads[e]] @ W_e^T + b_e)`` for every
+    branch e, ``s_e = sum(loads[:e])``, in one launch.  ``weight_table`` /
+    ``bias_table`` are int64 device tensors holding the branch pointers."""
+    if x.dtype != torch.bfloat16 or out.dtype != torch.bfloat16:
+        raise NotImplementedError("the grouped GEMM computes in bf16 (fp32 accumulation)")
+    if not (x.is_cuda and out.is_cuda and loads.is_cuda):
+        raise RuntimeError("grouped_linear needs device tensors")
+    if loads.dtype != torch.int32:
+        raise RuntimeError("capacities must be int32")
+    if not (x.is_contiguous() and out.is_contiguous()):
+        raise RuntimeError("shared inputs must be contiguous")
+    rows = x.shape[0]
+    if x.numel() != rows * in_features or out.numel() != rows * out_features:
+        raise RuntimeError("shared inputs do not match [rows, in_features] / [rows, out_features]")
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.lib().brt_hip_grouped_gemm(
+            x.data_ptr(), weight_table.data_ptr(),
+            None if bias_table is None else bias_table.data_ptr(), out.data_ptr(),
+            loads.data_ptr(), loads.numel(), rows, in_features, out_features, _ACT[activation],
+            torch.cuda.current_stream().cuda_stream))
+    return out
+
+
+class GroupedLinearKernel:
+    """Callable returned by ``make_jit_kernel(ModuleList[Linear], ..., "homo_fuse")``."""
+
+    def __init__(self, in_features: int, out_features: int, has_bias: bool,
+                 activation: Optional[str] = None):
+        self.in_features = in_features
+        self.out_features = out_features
+        self.has_bias = has_bias
+        self.activation = activation
+        self._weights = _PointerTable()
+        self._biases = _PointerTable()
+
+    def __call__(self, shared_inputs: List[torch.Tensor], standalone_inputs: Sequence[torch.Tensor],
+                 capacities: Union[torch.Tensor, Sequence[int]] = ()):
+        x, out = shared_inputs
+        standalone_inputs = list(standalone_inputs)
+        step = 2 if self.has_bias else 1
+        weights = standalone_inputs[0::step]
+        biases = standalone_inputs[1::step] if self.has_bias else None
+        if not torch.is_tensor(capacities):
+            capacities = torch.tensor(list(capacities), dtype=torch.int32, device=x.device)
+        if capacities.numel() > len(weights):
+            raise RuntimeError("more capacities than branches")
+        for w in weights[: capacities.numel()]:
+            if w.dtype != torch.bfloat16 or not w.is_contiguous():
+                raise NotImplementedError("branch weights must be contiguous bf16 [out, in]")
+        grouped_linear(
+            x, out, self._weights.get(weights),
+            self._biases.get(biases) if biases else None,
+            capacities.to(device=x.device, dtype=torch.int32), self.in_features,
+            self.out_features, self.activation)
+
+
+def make_jit_kernel(modules, sample_inputs=None, method: str = "forward", opt_level=None,
+                    objective_func: str = "fastest", rank=1, activation: Optional[str] = None
+                    ) -> Callable[..., None]:
+    """Signature of the reference (python/brt/jit/factory.py:28-44).  Only
+    ``opt_level="homo_fuse"`` over ``nn.Linear`` branches of one shape is built;
+    ``sample_inputs``, ``objective_func`` and ``rank`` (tuning knobs of the
+    reference's kernel database) are accepted and ignored.  ``activation`` (not in
+    the reference) fuses GELU / ReLU into the epilogue."""
+    if opt_level != "homo_fuse" or method != "forward":
+        raise NotImplementedError("only opt_level='homo_fuse', method='forward' is built")
+    branches = list(modules) if isinstance(modules, (nn.ModuleList, list, tuple)) else [modules]
+    if not branches or not all(isinstance(m, nn.Linear) for m in branches):
+        raise NotImplementedError("homo_fuse is built for nn.Linear branches")
+    shapes = {(m.in_features, m.out_features, m.bias is not None) for m in branches}
+    if len(shapes) != 1:
+        raise ValueError("homo_fuse needs branches of one shape")
+    (in_features, out_features, has_bias), = shapes
+    return GroupedLinearKernel(in_features, out_features, has_bias, activation)

@@ -1,0 +1,572 @@
+"""Fabrics: move cells between the flow a router receives and the per-path flows.
+
+Registry names, constructor keywords and call conventions follow
+python/brt/router/fabric/{base,generic,fused,identity,single_cell,placeholder,
+distributed}.py of the reference.  All device work goes through
+``brainstorm_amd._C.router`` (HIP kernels behind the C ABI).
+"""
+import os
+from typing import Any, Callable, Dict, List, Optional, Tuple, Union
+
+import numpy as np
+import torch
+import torch.nn as nn
+
+from brainstorm_amd._C import router as c_router
+from brainstorm_amd.router.utils import make_kwargs
+from brainstorm_amd.runtime import Registry
+from brainstorm_amd.runtime.grid_tensor import GridTensor, init_grid_tensor, to_torch_tensor
+
+_CAPTURE_MODES = ("avg", "max", "cum")
+
+
+class FabricBase(nn.Module):
+    """fabric/base.py:17-237: index-format flag plus optional flow statistics
+    (load history, routing decisions, cell shapes) for profile-guided passes."""
+
+    def __init__(self, flow_num: int, index_format: str = None, **kwargs) -> None:
+        super().__init__()
+        self.flow_num = flow_num
+        assert index_format in ("tag_index", "seat_index"), (
+            f"index_format should be tag_index or seat_index, but got {index_format}")
+        self.is_tag_index = index_format == "tag_index"
+        if os.environ.get("BRT_CAPTURE_STATS", "False").lower() == "true":
+            mode = os.environ.get("BRT_CAPTURE_MODE", "avg")
+            assert mode in _CAPTURE_MODES, f"Invalid capture mode: {mode}, valid: {_CAPTURE_MODES}"
+            self.enable_capture(mode, os.environ.get("BRT_CAPTURED_FABRIC_TYPE") or "dispatch")
+        else:
+            self.disable_capture()
+        self.reset_flow_stats()
+
+    def forward(self, *inputs: Any):
+        raise NotImplementedError("FabricBase is an abstract class for Fabric")
+
+    def check_compatibility(self, kwargs: Dict[str, Any]) -> None:
+        pass
+
+    # ---- capture switches ------------------------------------------------------------
+    def enable_capture(self, mode: str = "cum", fabric_type: str = "dispatch"):
+        self.capturing = True
+        self.capture_mode = mode
+        self.captured_fabric_type = fabric_type.split(",") if isinstance(fabric_type, str) else fabric_type
+
+    def disable_capture(self):
+        self.capturing = False
+        self.capture_mode = None
+        self.captured_fabric_type = []
+
+    def reset_flow_stats(self):
+        self.history_len = 0
+        self.cell_tag_base = 0
+        self.load_history: Optional[np.ndarray] = None
+        self.cell_decision_history: Optional[List[np.ndarray]] = None
+        self.cell_grain_history = None
+        self.cell_dtype_history = None
+        self.cell_device_history = None
+
+    def copy_flow_stats_from(self, other):
+        for name in ("history_len", "cell_tag_base", "load_history", "cell_decision_history",
+                     "cell_grain_history", "cell_device_history"):
+            setattr(self, name, getattr(other, name))
+
+    # ---- capture (forces device->host copies; keep off in timed runs) ----------------------
+    def capture_flow_stats(self, in_flows, route_indices=None, loads=None):
+        if not self.capturing:
+            return
+        kind = self.brt_abs_type
+        if "dispatch" in kind and "dispatch" in self.captured_fabric_type:
+            self._capture_correlations(route_indices, loads)
+            self._capture_cell_grains_and_options(in_flows, is_dispatch=True)
+            self._accumulate_loads(loads.cpu().numpy())
+        elif "combine" in kind and "combine" in self.captured_fabric_type:
+            if isinstance(in_flows, list) and len(in_flows) == 0:
+                return
+            self._capture_cell_grains_and_options(in_flows, is_dispatch=False)
+            if all(isinstance(f, list) for f in in_flows):
+                if not all(len(f) > 0 for f in in_flows):
+                    return
+                in_flows = in_flows[0]  # all groups are assumed to share their loads
+            self._accumulate_loads(np.array([f.size(0) for f in in_flows], dtype=np.float64))
+        else:
+            return
+        self.history_len += 1
+
+    def _accumulate_loads(self, current: np.ndarray):
+        if self.history_len == 0:
+            self.load_history = np.zeros_like(current, dtype=np.float64)
+        if self.capture_mode == "avg":
+            self.load_history = (self.load_history * self.history_len + current) / (self.history_len + 1.0)
+        elif self.capture_mode == "max":
+            self.load_history = np.maximum(self.load_history, current)
+        elif self.capture_mode == "cum":
+            self.load_history = self.load_history + current
+
+    def _capture_cell_grains_and_options(self, flows, is_dispatch=True) -> None:
+        flows = self._listing_flows(flows, is_dispatch)
+        if self.cell_grain_history is not None:
+            return
+        heads = flows if is_dispatch else [f[0] for f in flows]
+        self.cell_grain_history = [h.shape for h in heads]
+        self.cell_dtype_history = [h.dtype for h in heads]
+        self.cell_device_history = [h.device for h in heads]
+
+    def _capture_correlations(self, indices: torch.Tensor, loads: torch.Tensor):
+        tag_indices = indices
+        if not self.is_tag_index:
+            # the reference calls convert_index_format(..., True) here, which as built
+            # runs the opposite kernel (router.cc:104-107); this uses the direction meant
+            tag_indices = c_router.seat_to_tag_indices(indices, loads)
+        host_loads = loads.cpu().tolist()
+        current = []
+        for e, load in enumerate(host_loads):
+            column = tag_indices[:load, e].cpu().numpy()
+            current.append(column[column != 0] + self.cell_tag_base)
+        if self.history_len == 0:
+            self.cell_decision_history = current
+        else:
+            self.cell_decision_history = [
+                np.concatenate((old, new), axis=None)
+                for old, new in zip(self.cell_decision_history, current)]
+        for history in self.cell_decision_history:
+            if history.size > 0:
+                self.cell_tag_base = history.max()
+
+    def _listing_flows(self, flows, is_dispatch=True):
+        if is_dispatch:
+            return [flows] if isinstance(flows, torch.Tensor) else flows
+        if isinstance(flows, list):
+            return [flows] if isinstance(flows[0], torch.Tensor) else flows
+        return flows
+
+    def check_cell_consistency(self, flows, is_dispatch=True) -> bool:
+        if self.cell_grain_history is None:
+            return self.history_len == 0
+        for i, flow in enumerate(flows):
+            head = flow if is_dispatch else flow[0]
+            if (head.shape[1:] != self.cell_grain_history[i][1:]
+                    or head.dtype != self.cell_dtype_history[i]
+                    or head.device != self.cell_device_history[i]):
+                return False
+        return True
+
+
+def register_fabric(fabric_type: str) -> Callable:
+    return Registry.register_sub_cls(fabric_type, FabricBase)
+
+
+def make_fabric(fabric_type: str, kwargs: Dict[str, Any]) -> FabricBase:
+    fabric_cls = Registry.get_sub_cls(fabric_type, FabricBase)
+    if fabric_cls is None:
+        raise ValueError(f"Fabric type: {fabric_type} is not registered.")
+    return fabric_cls(**make_kwargs(kwargs))
+
+
+def switch_capture(m: nn.Module, capture=True, mode=None, fabric_type=None):
+    for child in m.children():
+        switch_capture(child, capture=capture, mode=mode, fabric_type=fabric_type)
+    if isinstance(m, FabricBase):
+        if capture:
+            m.enable_capture(mode=mode if mode is not None else m.capture_mode,
+                             fabric_type=fabric_type if fabric_type is not None else m.captured_fabric_type)
+        else:
+            m.disable_capture()
+    return m
+
+
+def reset_router_stats(m: nn.Module):
+    for child in m.children():
+        reset_router_stats(child)
+    if isinstance(m, FabricBase):
+        m.reset_flow_stats()
+    return m
+
+
+def _per_flow(value, flow_num: int, allowed=None, kind=str) -> list:
+    """Broadcasts a scalar option to one entry per flow and validates it."""
+    values = [value] * flow_num if isinstance(value, kind) else value
+    assert isinstance(values, list) and len(values) == flow_num
+    assert all(isinstance(v, kind) and (allowed is None or v in allowed) for v in values)
+    return values
+
+
+# --------------------------------------------------------------------------- generic
+@register_fabric("dispatch")
+class DispatchFabric(FabricBase):
+    """fabric/generic.py:17-182.
+
+    Keywords: ``route_logic`` ("1d" | "2d", or a list per flow), ``transform``
+    (scale cells by the score), ``index_format`` ("tag_index" default),
+    ``supported_capacities`` (int | list[int]), ``capacity_padding``,
+    ``path_wise_padding``, ``max_path_padding``, ``max_path_load``.
+    """
+
+    def __init__(self, flow_num: int, route_logic: Union[str, List[str]] = "1d",
+                 transform: Union[bool, List[bool]] = False, **kwargs):
+        index_format = kwargs.pop("index_format", "tag_index")
+        super().__init__(flow_num=flow_num, index_format=index_format, **kwargs)
+        self.route_logics = _per_flow(route_logic, flow_num, ("1d", "2d"), str)
+        self.transforms = _per_flow(transform, flow_num, None, bool)
+        caps = kwargs.pop("supported_capacities", None)
+        self.capacity_padding = kwargs.pop("capacity_padding", False)
+        if caps is not None:
+            caps = [caps] if isinstance(caps, int) else caps
+            assert isinstance(caps, list) and all(isinstance(c, int) for c in caps)
+            self.register_buffer("supported_capacities", torch.tensor(caps, dtype=torch.int32))
+            self.path_wise_padding = kwargs.pop("path_wise_padding", False)
+        else:
+            self.register_buffer("supported_capacities", None)
+            self.path_wise_padding = False
+        self.max_path_padding = kwargs.pop("max_path_padding", False)
+        self.max_path_load = kwargs.pop("max_path_load", 0)
+
+    def forward(self, in_flow, hot_mask: torch.Tensor, runtime_capacities: torch.Tensor = None,
+                score: torch.Tensor = None):
+        caps = runtime_capacities if runtime_capacities is not None else self.supported_capacities
+        route_indices, loads = c_router.generate_indices_and_loads(
+            hot_mask, supported_capacities=caps, capacity_padding=self.capacity_padding,
+            path_wise_padding=self.path_wise_padding, is_tag_index=False)
+        in_flows = [in_flow] if self.flow_num == 1 else in_flow
+        self.capture_flow_stats(in_flows, route_indices, loads)
+        all_out_flows, score = self.dispatch(in_flows, route_indices, loads, score)
+        if self.flow_num == 1:
+            all_out_flows = all_out_flows[0]
+        return all_out_flows, score
+
+    def _dispatch_flow(self, flow_idx, flow_data, flow_tag, route_indices, loads, score):
+        # positional layout of the reference call (generic.py:127-137): the 5th
+        # argument is tag_generating, seat indices are always what is dispatched with
+        return c_router.dispatch_with_indices_and_loads(
+            flow_data, route_indices, loads, score if self.transforms[flow_idx] else None,
+            self.is_tag_index, flow_tag, self.max_path_padding, self.max_path_load,
+            self.route_logics[flow_idx] == "1d")
+
+    def dispatch(self, in_flows, route_indices, loads, score):
+        all_out_flows = []
+        path_num = route_indices.size(1)
+        for flow_idx in range(self.flow_num):
+            data, tags, load_stack, extra = to_torch_tensor(in_flows[flow_idx], retrieve_attr=True)
+            flow_tag = tags[-1]
+            tags, load_stack = tags[:-1], load_stack[:-1]
+            routed = self._dispatch_flow(flow_idx, data, flow_tag, route_indices, loads, score)
+            if self.is_tag_index:
+                routed_data, routed_tags = routed
+                datas, path_loads, path_tags = c_router.split_fused_cells_to_paths(
+                    routed_data, loads, self.max_path_padding, is_load_split=True,
+                    is_tag_split=True, tags=routed_tags)
+                all_out_flows.append([
+                    init_grid_tensor(datas[i], tags + [path_tags[i]], load_stack + [path_loads[i]], extra)
+                    for i in range(path_num)])
+            else:
+                (datas,) = c_router.split_fused_cells_to_paths(
+                    routed[0], loads, self.max_path_padding, is_load_split=False, is_tag_split=False)
+                all_out_flows.append([
+                    init_grid_tensor(datas[i], tags + [route_indices], load_stack + [loads], extra)
+                    for i in range(path_num)])
+        return all_out_flows, score
+
+
+@register_fabric("combine")
+class CombineFabric(FabricBase):
+    """fabric/generic.py:185-313.  Keywords: ``reduction``, ``transform``,
+    ``index_format``, ``max_path_padding``, ``ever_padded``."""
+
+    def __init__(self, flow_num: int, reduction="add", transform=False, **kwargs):
+        index_format = kwargs.pop("index_format", "tag_index")
+        super().__init__(flow_num=flow_num, index_format=index_format, **kwargs)
+        self.max_path_padding = kwargs.pop("max_path_padding", False)
+        self.ever_padded = kwargs.pop("ever_padded", False) or self.max_path_padding
+        self.reduction = reduction
+        self.transform = transform
+
+    def forward(self, in_flows, residual_flows=None, score: torch.Tensor = None):
+        if self.flow_num == 1:
+            in_flows = [in_flows]
+            residual_flows = [residual_flows] if residual_flows is not None else None
+        self.capture_flow_stats(in_flows)
+        out_flows = self.combine(in_flows, residual_flows, score)
+        return out_flows[0] if self.flow_num == 1 else out_flows
+
+    def combine(self, in_flows, residual_flows, score):
+        out_flows = []
+        for flow_idx in range(self.flow_num):
+            residual = residual_flows[flow_idx] if residual_flows is not None else None
+            datas, tags, loads = [], [], []
+            for flow in in_flows[flow_idx]:
+                data, tag_stack, load_stack, extra = to_torch_tensor(flow, retrieve_attr=True)
+                datas.append(data)
+                tags.append(tag_stack[-1])
+                loads.append(load_stack[-1])
+            if len(datas) == 1 and tags[0] is None:
+                # a single un-routed flow: label its cells 1..n
+                data = datas[0]
+                n = data.shape[0]
+                tag_stack[-1] = torch.arange(1, n + 1, dtype=torch.int32, device=data.device)
+                load_stack[-1] = torch.tensor([n], dtype=torch.int32, device=data.device)
+                out_flows.append(init_grid_tensor(data, tag_stack, load_stack, extra))
+                continue
+            if self.is_tag_index:
+                fused, fused_tags, route_indices = c_router.fuse_split_cells_from_paths(
+                    datas, is_tag_fuse=True, loads=loads, tags=tags)
+                fused_loads = None
+            else:
+                (fused,) = c_router.fuse_split_cells_from_paths(datas)
+                fused_loads, route_indices, fused_tags = loads[0], tags[0], None
+            result = c_router.combine_with_indices_and_loads(
+                fused, route_indices, fused_loads, score if self.transform else None, residual,
+                max_path_padding=self.max_path_padding, ever_padded=self.ever_padded,
+                is_tag_index=self.is_tag_index, tags=fused_tags)
+            if self.is_tag_index:
+                out_data, out_tag, out_load = result
+            else:
+                (out_data,), out_tag, out_load = result, None, None
+            out_flow = init_grid_tensor(out_data, tag_stack[:-1], load_stack[:-1], extra)
+            out_flows.append(out_flow.pack(out_tag, out_load))
+        return out_flows
+
+
+# ----------------------------------------------------------------------------- fused
+@register_fabric("fused_dispatch")
+class FusedDispatchFabric(DispatchFabric):
+    """fabric/fused.py:18-75: one path-major buffer per flow (seat indices); the MoE
+    path.  Output GridTensor gets ``route_indices`` / ``loads`` pushed on its stacks."""
+
+    def __init__(self, flow_num: int, route_logic="1d", transform=False, **kwargs):
+        kwargs["index_format"] = "seat_index"
+        super().__init__(flow_num, route_logic=route_logic, transform=transform, **kwargs)
+
+    def dispatch(self, in_flows, route_indices, loads, score):
+        all_out_flows = []
+        for flow_idx, flow in enumerate(in_flows):
+            data, tags, load_stack, extra = to_torch_tensor(flow, retrieve_attr=True)
+            flow_tag = tags[-1]
+            assert flow_tag is None  # fused dispatch starts from freshly annotated cells
+            (routed,) = self._dispatch_flow(flow_idx, data, flow_tag, route_indices, loads, score)
+            all_out_flows.append(init_grid_tensor(
+                routed, tags[:-1] + [route_indices], load_stack[:-1] + [loads], extra))
+        return all_out_flows, score
+
+
+@register_fabric("fused_combine")
+class FusedCombineFabric(CombineFabric):
+    """fabric/fused.py:78-123."""
+
+    def __init__(self, flow_num, reduction="add", transform=False, **kwargs) -> None:
+        kwargs["index_format"] = "seat_index"
+        super().__init__(flow_num=flow_num, reduction=reduction, transform=transform, **kwargs)
+
+    def combine(self, in_flows, residual_flows, score):
+        out_flows = []
+        for flow_idx, in_flow in enumerate(in_flows):
+            data, tags, load_stack, extra = to_torch_tensor(in_flow, retrieve_attr=True)
+            residual = residual_flows[flow_idx] if residual_flows is not None else None
+            route_indices, loads = tags.pop(), load_stack.pop()
+            (out,) = c_router.combine_with_indices_and_loads(
+                data, route_indices, loads, score if self.transform else None, residual,
+                max_path_padding=self.max_path_padding, ever_padded=self.ever_padded)
+            out_flows.append(init_grid_tensor(out, tags, load_stack, extra))
+        return out_flows
+
+
+# -------------------------------------------------------------------------- identity
+@register_fabric("identity_dispatch")
+class IndentityDispatchFabric(DispatchFabric):  # (sic) class name of the reference
+    """fabric/identity.py:12-83: every path sees the whole flow."""
+
+    def __init__(self, path_num: int, flow_num: int, route_logic="1d", transform=False, **kwargs):
+        super().__init__(flow_num=flow_num, route_logic=route_logic, transform=transform, **kwargs)
+        self.path_num = path_num
+
+    def forward(self, in_flow, hot_mask, runtime_capacities=None, score=None):
+        in_flows = [in_flow] if self.flow_num == 1 else in_flow
+        all_out_flows = self.dispatch(in_flows, None, None, score)
+        if self.flow_num == 1:
+            all_out_flows = all_out_flows[0]
+        return all_out_flows
+
+    def dispatch(self, in_flows, route_indices, loads, score):
+        all_out_flows = []
+        for flow_idx in range(self.flow_num):
+            flow = in_flows[flow_idx]
+            logic = self.route_logics[flow_idx]
+            if logic == "2d":
+                flow = flow.transpose(0, 1).contiguous()
+            out_flows = []
+            for path_id in range(self.path_num):
+                if logic == "1d":
+                    out = flow
+                    if self.transforms[flow_idx]:
+                        out = out * score[:, path_id].view((-1,) + (1,) * (flow.dim() - 1))
+                else:
+                    out = flow[path_id].contiguous()
+                out_flows.append(out)
+            all_out_flows.append(out_flows)
+        return all_out_flows, score
+
+
+@register_fabric("identity_combine")
+class IdentityCombineFabric(CombineFabric):
+    """fabric/identity.py:86-111: element-wise sum of the per-path flows."""
+
+    def __init__(self, flow_num: int, **kwargs):
+        super().__init__(flow_num=flow_num, **kwargs)
+
+    def combine(self, in_flows, residual_flows, scores):
+        out_flows = []
+        for flow_idx, flows in enumerate(in_flows):
+            shape = flows[0].shape
+            if residual_flows is not None:
+                flows.append(residual_flows[flow_idx])
+            out_flows.append(torch.cat(flows, dim=0).reshape(-1, 1, *shape[1:]).sum(dim=0))
+        return out_flows
+
+
+# ----------------------------------------------------------------------- single cell
+@register_fabric("single_cell_dispatch")
+class SingleCellDispatchFabric(DispatchFabric):
+    """fabric/single_cell.py:11-98: batch size 1, the hot mask itself is the loads;
+    works on CPU and GPU tensors (no kernel involved)."""
+
+    def __init__(self, flow_num: int, route_logic="1d", transform=False, **kwargs):
+        super().__init__(flow_num=flow_num, route_logic=route_logic, transform=transform, **kwargs)
+
+    def forward(self, in_flow, hot_mask, runtime_capacities=None, score=None):
+        in_flows = [in_flow] if self.flow_num == 1 else in_flow
+        if hot_mask.numel() == 0:
+            loads = torch.zeros([hot_mask.size(1)], dtype=hot_mask.dtype, device=hot_mask.device)
+        else:
+            loads = hot_mask.view(-1)
+        self.capture_flow_stats(in_flows, hot_mask, loads)
+        all_out_flows, score = self.dispatch(in_flows, hot_mask, loads, score)
+        if self.flow_num == 1:
+            all_out_flows = all_out_flows[0]
+        return all_out_flows, score
+
+    def dispatch(self, in_flows, route_indices, loads, score):
+        all_out_flows = []
+        host_loads = loads.cpu().tolist()
+        for flow_idx, flow in enumerate(in_flows):
+            logic = self.route_logics[flow_idx]
+            route_shape = list(flow.shape[1:])
+            if logic == "2d":
+                route_shape[0] = 1
+                flow = flow.transpose(0, 1).contiguous()
+            out_flows = []
+            for path_id, load in enumerate(host_loads):
+                if load == 0:
+                    out_flows.append(torch.zeros(0, *route_shape, dtype=flow.dtype, device=flow.device))
+                    continue
+                out = flow if logic == "1d" else flow[path_id:path_id + 1].contiguous()
+                if self.transforms[flow_idx]:
+                    out = out * score[:, path_id].view((-1,) + (1,) * len(route_shape))
+                out_flows.append(out)
+            all_out_flows.append(out_flows)
+        return all_out_flows, score
+
+
+@register_fabric("single_cell_combine")
+class SingleCellCombineFabric(CombineFabric):
+    """fabric/single_cell.py:101-131."""
+
+    def __init__(self, flow_num: int, reduction="add", transform=False, **kwargs):
+        super().__init__(flow_num=flow_num, reduction=reduction, transform=transform, **kwargs)
+        assert reduction == "add" and not transform
+
+    def combine(self, in_flows, residual_flows, score):
+        out_flows = []
+        for flow_idx, in_flow in enumerate(in_flows):
+            fused = torch.cat(in_flow, dim=0)
+            if fused.numel() > 0:
+                out_flows.append(fused.sum(dim=0, keepdim=True))
+            elif residual_flows is not None:
+                out_flows.append(residual_flows[flow_idx])
+            else:
+                out_flows.append(fused)
+        return out_flows
+
+
+# ------------------------------------------------------------------------ placeholder
+@register_fabric("placeholder_combine")
+class PlaceholderCombineFabric(CombineFabric):
+    """fabric/placeholder.py:12-58: returns empty flows of recorded shape (dead paths)."""
+
+    def __init__(self, flow_num: int, runtime_load: int, cell_grains: List[torch.Size],
+                 cell_dtypes: List[torch.dtype], cell_devices: List[torch.device], **kwargs):
+        super().__init__(flow_num=flow_num, **kwargs)
+        self.runtime_load = runtime_load
+        self.cell_grains = [[0] + list(g)[1:] for g in cell_grains[:flow_num]] + list(cell_grains[flow_num:])
+        self.cell_dtypes = cell_dtypes
+        self.cell_devices = cell_devices
+        assert len(self.cell_grains) == len(cell_dtypes) == len(cell_devices) == flow_num, (
+            "cell_grains/dtypes/devices must have the same elements as flow_num")
+
+    def forward(self, in_flow, hot_mask=None, runtime_capacities=None, score=None):
+        outs = [torch.zeros(self.cell_grains[i], dtype=self.cell_dtypes[i], device=self.cell_devices[i])
+                for i in range(self.flow_num)]
+        return outs[0] if self.flow_num == 1 else outs
+
+
+# ------------------------------------------------------------------------ distributed
+def _require_single_process():
+    import torch.distributed as dist
+
+    if dist.is_available() and dist.is_initialized() and dist.get_world_size() > 1:
+        raise NotImplementedError(
+            "the sparse all-to-all of the distributed fabrics is not part of this build; "
+            "on one GPU they are the fused fabrics (python/brt/runtime/distributed.py:177-202)")
+
+
+@register_fabric("distributed_fused_dispatch")
+class DistributedFusedDispatchFabric(FusedDispatchFabric):
+    """fabric/distributed.py:14-97 on one process: the exchange is the identity, so
+    the result is the fused dispatch with ``in_loads`` recorded next to the loads."""
+
+    def __init__(self, flow_num: int, capacity_padding=False, route_logic="1d", transform=False,
+                 task_locality: bool = False, **kwargs):
+        self.task_locality = task_locality
+        super().__init__(flow_num=flow_num, capacity_padding=capacity_padding,
+                         route_logic=route_logic, transform=transform, **kwargs)
+
+    def dispatch(self, in_flows, route_indices, loads, score):
+        _require_single_process()
+        all_out_flows = []
+        for flow_idx in range(self.flow_num):
+            data, tags, load_stack, extra = to_torch_tensor(in_flows[flow_idx], retrieve_attr=True)
+            (routed,) = c_router.dispatch_with_indices_and_loads(
+                data, route_indices, loads, score if self.transforms[flow_idx] else None,
+                False, None, self.max_path_padding, self.max_path_load,
+                self.route_logics[flow_idx] == "1d")
+            if self.task_locality:  # world of one: path i holds task i
+                host_loads = loads.cpu().tolist()
+                score = torch.repeat_interleave(
+                    torch.arange(len(host_loads), device=routed.device),
+                    torch.tensor(host_loads, device=routed.device))
+                all_out_flows.append(routed)
+                continue
+            out_flow = init_grid_tensor(routed, tags, load_stack, extra)
+            out_flow.pack(route_indices, loads, in_loads=loads)
+            all_out_flows.append(out_flow)
+        return all_out_flows, score
+
+
+@register_fabric("distributed_fused_combine")
+class DistributedFusedCombineFabric(FusedCombineFabric):
+    """fabric/distributed.py:100-158 on one process."""
+
+    def __init__(self, flow_num, reduction="add", transform=False, task_locality: bool = False,
+                 **kwargs) -> None:
+        self.task_locality = task_locality
+        super().__init__(flow_num=flow_num, reduction=reduction, transform=transform, **kwargs)
+
+    def combine(self, in_flows, residual_flows, score):
+        _require_single_process()
+        out_flows = []
+        for idx, in_flow in enumerate(in_flows):
+            in_flow, route_indices, _in_loads, attrs = in_flow.unpack("in_loads")
+            out_loads = attrs["in_loads"]
+            data, tags, load_stack, extra = to_torch_tensor(in_flow, retrieve_attr=True)
+            residual = residual_flows[idx] if residual_flows is not None else None
+            (out,) = c_router.combine_with_indices_and_loads(
+                data, route_indices, out_loads, score if self.transform else None, residual,
+                max_path_padding=self.max_path_padding, ever_padded=self.ever_padded)
+            out_flows.append(init_grid_tensor(out, tags, load_stack, extra))
+        return out_flows

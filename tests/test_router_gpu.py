@@ -1,0 +1,256 @@
+"""Router-level behaviour on the GPU through the reference's Python API
+(scenarios of test/python/router_test.py:16-407 re-expressed), plus the
+``brt._C.router`` shim against the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+import torch.nn as nn
+
+import oracle
+from routing_cases import softmax, to_bf16_bits, topk_mask
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def brt_mod():
+    import brt
+    import brt._C.router as c_router
+    from brt.router import GatherRouter, ScatterRouter
+
+    return brt, c_router, ScatterRouter, GatherRouter
+
+
+class BranchRoute(nn.Module):
+    """threshold-0.5 gate, two identity experts (router_test.py:16-56)."""
+
+    def __init__(self, brt_mod, gate, dispatch_score=False, single_cell=False,
+                 supported_capacities=None, capacity_padding=False, path_wise_padding=False):
+        super().__init__()
+        brt, _, ScatterRouter, GatherRouter = brt_mod
+        self.gate = gate
+        self.annotator = brt.Annotator([0])
+        self.scatter_router = ScatterRouter(
+            dispatch_score=dispatch_score, protocol_type="threshold",
+            fabric_type="single_cell_dispatch" if single_cell else "dispatch",
+            protocol_kwargs={"threshold": 0.5},
+            fabric_kwargs={"supported_capacities": supported_capacities,
+                           "capacity_padding": capacity_padding,
+                           "path_wise_padding": path_wise_padding})
+        self.gather_router = GatherRouter(
+            fabric_type="single_cell_combine" if single_cell else "combine",
+            fabric_kwargs={"ever_padded": capacity_padding})
+
+    def forward(self, x):
+        x = self.annotator(x)
+        routed = self.scatter_router(x, self.gate(x))
+        return routed[0], routed[1], self.gather_router([routed[0], routed[1]])
+
+
+class WeightedBranchRoute(BranchRoute):
+    def __init__(self, brt_mod, gate, single_cell=False):
+        super().__init__(brt_mod, gate, dispatch_score=True, single_cell=single_cell)
+
+    def forward(self, x):
+        x = self.annotator(x)
+        score = self.annotator(self.gate(x))
+        dims = x.dim()
+        routed, routed_score = self.scatter_router(x, score)
+        shape = lambda s: s.view(-1, *([1] * (dims - 1)))  # noqa: E731
+        pre = self.gather_router([routed[0] * shape(routed_score[0]), routed[1] * shape(routed_score[1])])
+        post = self.gather_router([routed[0], routed[1]]) * shape(
+            self.gather_router([routed_score[0], routed_score[1]]))
+        return pre, post
+
+
+def half_gate(dst, which_half):
+    def gate(inputs):
+        gates = torch.zeros(inputs.shape[0], 2, dtype=torch.float, device=inputs.device)
+        n = inputs.shape[0]
+        rows = slice(n // 2, None) if which_half == "upper" else slice(0, n // 2) if which_half == "lower" else slice(None)
+        gates[rows, dst] = 1
+        return gates
+    return gate
+
+
+def samples(first):
+    return [torch.arange(0, first * 10, dtype=torch.float32).view(first, 10).cuda(),
+            torch.arange(0, first * 20, dtype=torch.float32).view(first, 2, 10).cuda(),
+            torch.arange(0, first * 40, dtype=torch.float32).view(first, 2, 10, 2).cuda()]
+
+
+@pytest.mark.parametrize("dst", [0, 1])
+@pytest.mark.parametrize("which_half", [None, "upper", "lower"])
+def test_generic_route(brt_mod, dst, which_half):
+    for x in samples(8):
+        model = BranchRoute(brt_mod, half_gate(dst, which_half)).eval().cuda()
+        n = x.size(0)
+        want = x if which_half is None else x[n // 2:] if which_half == "upper" else x[: n // 2]
+        for _ in range(3):
+            res = model(x)
+            assert torch.equal(res[dst].data, want)
+            assert res[1 - dst].numel() == 0
+            assert torch.equal(res[2].data, want)
+        weighted = WeightedBranchRoute(brt_mod, half_gate(dst, which_half)).eval().cuda()
+        pre, post = weighted(x)
+        assert torch.allclose(pre.data, post.data)
+
+
+def test_single_cell_route_cpu_then_gpu(brt_mod):
+    for x in samples(1):
+        for dst in (0, 1, [0, 1]):
+            def gate(inp, dst=dst):
+                g = torch.zeros(1, 2, dtype=torch.float, device=inp.device)
+                for d in (dst if isinstance(dst, list) else [dst]):
+                    g[:, d] = 1
+                return g
+            model = BranchRoute(brt_mod, gate, single_cell=True).eval()
+            for inp in (x.cpu(), x):
+                if inp.is_cuda:
+                    model.cuda()
+                res = model(inp)
+                if isinstance(dst, list):
+                    assert all(torch.equal(res[d], inp) for d in dst)
+                    assert torch.equal(res[2], inp * 2)
+                else:
+                    assert torch.equal(res[dst], inp) and res[1 - dst].numel() == 0
+                    assert torch.equal(res[2], inp)
+
+
+@pytest.mark.parametrize("dst", [0, 1])
+@pytest.mark.parametrize("which_half", [None, "upper", "lower"])
+@pytest.mark.parametrize("padding", ["clip", "pad", "path_wise"])
+def test_padded_route(brt_mod, dst, which_half, padding):
+    caps = [10, 12]
+    for x in samples(8):
+        model = BranchRoute(brt_mod, half_gate(dst, which_half), supported_capacities=caps,
+                            capacity_padding=padding != "clip",
+                            path_wise_padding=padding == "path_wise").eval().cuda()
+        n = x.size(0)
+        want = x if which_half is None else x[n // 2:] if which_half == "upper" else x[: n // 2]
+        real = want.size(0)
+        rows = real if padding == "clip" else caps[dst] if padding == "path_wise" else 10
+        res = model(x)
+        assert res[dst].size(0) == rows
+        assert torch.equal(res[dst].data[:real], want)
+        assert not res[dst].data[real:].any()  # padding rows are exactly zero
+        if padding == "path_wise":
+            # the kernel pads EVERY path to its capacity, also the empty one
+            # (src/router/location.cu:227-230)
+            assert res[1 - dst].size(0) == caps[1 - dst] and not res[1 - dst].data.any()
+        else:
+            assert res[1 - dst].numel() == 0
+        assert torch.equal(res[2].data, want)
+
+
+def test_fused_moe_path_matches_oracle(brt_mod):
+    """Annotator -> ScatterRouter(fused_dispatch) -> experts -> GatherRouter(fused_combine)
+    with residual, as in benchmark/switch_moe/switch_transformer.py:352-385."""
+    brt, c_router, ScatterRouter, GatherRouter = brt_mod
+    T, E, d, cap = 2048, 16, 256, 160
+    mask, logits = topk_mask(T, E, 1, seed=5)
+    x = torch.from_numpy(to_bf16_bits(np.random.default_rng(5).standard_normal((T, d))).view(np.int16)
+                         ).cuda().view(torch.bfloat16)
+    scatter = ScatterRouter(protocol_type="switch_top1", fabric_type="fused_dispatch",
+                            fabric_kwargs={"supported_capacities": [cap], "capacity_padding": True}).cuda()
+    gather = GatherRouter(fabric_type="fused_combine").cuda()
+    cells = brt.Annotator([0])(x)
+    routed = scatter(cells, torch.from_numpy(mask).cuda())
+    assert isinstance(routed, brt.GridTensor) and routed.stack_size == 1
+    idx, loads = routed.tag, routed.load
+    o_idx, o_loads = oracle.generate_indices_and_loads(mask, [cap], True)
+    assert np.array_equal(idx.cpu().numpy(), o_idx) and np.array_equal(loads.cpu().numpy(), o_loads)
+    xb = x.view(torch.int16).cpu().numpy().view(np.uint16)
+    o_y, _ = oracle.dispatch(xb, o_idx, o_loads, dtype="bf16")
+    assert np.array_equal(brt.to_torch_tensor(routed).view(torch.int16).cpu().numpy().view(np.uint16), o_y)
+    expert_out = routed * 2  # stacks travel through the expert
+    residual = x.clone()
+    out = gather(expert_out, residual)
+    assert out.data_ptr() == residual.data_ptr() and out.stack_size == 0
+    o_out = oracle.combine(brt.to_torch_tensor(expert_out).view(torch.int16).cpu().numpy().view(np.uint16),
+                           o_idx, o_loads, out_data=xb, in_dtype="bf16")
+    assert np.array_equal(out.view(torch.int16).cpu().numpy().view(np.uint16), o_out)
+
+
+def test_shim_signatures_and_errors(brt_mod):
+    _, c_router, _, _ = brt_mod
+    mask, logits = topk_mask(300, 4, 2, seed=9)
+    d_mask = torch.from_numpy(mask).cuda()
+    with pytest.raises(RuntimeError):
+        c_router.generate_indices_and_loads(torch.from_numpy(mask))  # CPU tensor
+    with pytest.raises(RuntimeError):
+        c_router.generate_indices_and_loads(d_mask, None, True)  # padding without capacities
+    idx, loads = c_router.generate_indices_and_loads(d_mask)
+    x = torch.randn(300, 6, device="cuda")
+    with pytest.raises(NotImplementedError):
+        c_router.dispatch_with_indices_and_loads(x.double(), idx, loads)
+    # positional call of the fabrics: (in, idx, loads, gates, tag_generating, tags, pad, load, is_1d)
+    out, tags = c_router.dispatch_with_indices_and_loads(x, idx, loads, None, True, None, False, 0, True)
+    o_out, o_tags = oracle.dispatch(x.cpu().numpy(), mask.cumsum(0) * mask, mask.sum(0), tag_generating=True)
+    assert np.array_equal(out.cpu().numpy(), o_out) and np.array_equal(tags.cpu().numpy(), o_tags)
+    # loads on the host are accepted (router.cc:181-187); the pre-zeroed path is taken
+    out2, = c_router.dispatch_with_indices_and_loads(x, idx, loads.cpu())
+    assert torch.equal(out, out2)
+    # empty input (router.cc:150-168) and the legacy alias
+    e, = c_router.dispatch_with_indices_and_loads(x[:0], idx[:0], loads)
+    assert e.shape == (0, 6)
+    i0, l0 = c_router.generate_indices_and_loads(d_mask[:0])
+    assert i0.shape == (0, 4) and l0.tolist() == [0, 0, 0, 0]
+    assert c_router.combine_with_src_indices is c_router.combine_with_indices_and_loads
+    back, = c_router.combine_with_src_indices(out, idx, loads)
+    assert torch.equal(back, 2 * x)
+    # T == 1 shortcut of the binding (router.cc:402-412): no routing applied
+    one, = c_router.combine_with_indices_and_loads(out[:1], idx[:1], loads)
+    assert one.data_ptr() == out[:1].data_ptr()
+    # 2-d routing of the score tensor: [T,E] -> [P,1]
+    s = torch.from_numpy(softmax(logits)).cuda()
+    routed_s, = c_router.dispatch_with_indices_and_loads(s, idx, loads, is_1d_routing=False)
+    assert routed_s.shape == (int(loads.sum()), 1)
+    assert np.array_equal(routed_s.cpu().numpy(),
+                          oracle.dispatch(s.cpu().numpy(), idx.cpu().numpy(), loads.cpu().numpy(),
+                                          is_1d_routing=False)[0])
+    # split / fuse and the tag-index combine (sample/cpp/dispatch.ipynb cells 1-2)
+    datas, split_loads, split_tags = c_router.split_fused_cells_to_paths(
+        out, loads, is_load_split=True, is_tag_split=True, tags=tags)
+    assert [t.size(0) for t in datas] == loads.tolist()
+    fused, new_tags, seats = c_router.fuse_split_cells_from_paths(datas, is_tag_fuse=True, tags=split_tags)
+    final, final_tags, n = c_router.combine_with_indices_and_loads(
+        fused, seats, None, tags=new_tags, is_tag_index=True)
+    assert torch.allclose(final, 2 * x) and n.item() == 300
+    # convert_index_format keeps the as-built flag meaning; the named helpers are explicit
+    tag_idx, _ = c_router.generate_indices_and_loads(d_mask, is_tag_index=True)
+    assert torch.equal(c_router.seat_to_tag_indices(idx, loads), tag_idx)
+    assert torch.equal(c_router.convert_index_format(tag_idx, loads, True), idx)
+    assert torch.equal(c_router.convert_index_format(idx, loads, False), tag_idx)
+
+
+def test_throttle_and_swin_scatter(brt_mod):
+    brt, c_router, _, _ = brt_mod
+    from brt.router import SwinMoEScatterRouter
+
+    T, E, d = 4096, 8, 96
+    rng = np.random.default_rng(11)
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    score = torch.from_numpy(softmax(logits)).cuda()
+    x = torch.from_numpy(rng.standard_normal((T, d)).astype(np.float16)).cuda()
+    router = SwinMoEScatterRouter(
+        protocol_kwargs={"top_k": 1, "capacity_factor": 1.0},
+        fabric_type="fused_dispatch",
+        fabric_kwargs={"capacity_padding": True, "max_path_padding": True}).cuda()
+    routed, new_score = router(brt.Annotator([0])(x), score, None, None)
+    cap = 512
+    assert router.fabric.max_path_load == cap and routed.shape == (E * cap, d)
+    mask = np.zeros((T, E), dtype=np.int32)
+    mask[np.arange(T), softmax(logits).argmax(1)] = 1
+    thr, _ = oracle.throttle_hotmask(mask, np.zeros(E, np.int32), np.full(E, cap, np.int32))
+    o_idx, o_loads = oracle.generate_indices_and_loads(thr, [cap] * E, True)
+    assert np.array_equal(routed.tag.cpu().numpy(), o_idx)
+    assert np.array_equal(routed.load.cpu().numpy(), o_loads)
+    o_y, _ = oracle.dispatch(x.cpu().numpy().view(np.uint16), o_idx, o_loads, max_path_padding=True,
+                             max_path_load=cap, dtype="f16")
+    assert np.array_equal(brt.to_torch_tensor(routed).cpu().numpy().view(np.uint16), o_y)
+    from brt.router import GatherRouter
+    out = GatherRouter(fabric_type="fused_combine", fabric_kwargs={"max_path_padding": True})(routed)
+    kept = thr.any(1)
+    assert torch.equal(out[torch.from_numpy(kept).cuda()], x[torch.from_numpy(kept).cuda()])
+    assert not out[torch.from_numpy(~kept).cuda()].any()
