@@ -1,0 +1,305 @@
+#!/usr/bin/env python3
+"""Benchmark of the MoE routing hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Workload (BASELINE.json configs[1]): Switch-MoE layer, bf16, 8192 tokens x d=768,
+64 experts, top-1 softmax gate over N(0,1) logits, capacity factor 1.25
+(capacity 160, overflow dropped), expert FFN 768->3072->768 GELU with N(0,0.02)
+weights; seeded synthetic data, everything resident in HBM before timing.
+
+A step is one pass of the hot path over the batch, called through the C ABI of
+libbrt_hip.so and replayed as one HIP graph:
+    index/load generation -> dispatch -> grouped FFN (two launches) -> combine.
+`value` is the headline metric: algorithmic bytes of dispatch + combine divided
+by the sum of their kernel times.  Kernel times are measured in this process
+with HIP events around graphs of back-to-back launches of the one kernel, on the
+stream the kernels are launched on.  The reference's PyTorch CPU routing path
+(oracle/torch_path.py) is timed on the host cores as `cpu_baseline`.
+Prints ONE JSON line.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+
+# Bytes per launch seen by the memory side for this workload: rocprofv3 --pmc
+# FETCH_SIZE and WRITE_SIZE (KiB), each scaled by what the same counter reads for
+# a 12 MiB device-to-device copy (fetch x1.996, write x1.000).
+MEASURED_TRAFFIC_BYTES = {
+    "dispatch": int((7203.0 * 1.996 + 12288.0) * 1024),
+    "combine": int((7197.0 * 1.996 + 12288.0) * 1024),
+}
+
+T, D, E, DFF = 8192, 768, 64, 3072
+CAPACITY = int(1.25 * (T // E))  # 160
+SEED = 2
+
+
+def parse():
+    p = argparse.ArgumentParser()
+    p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--steps", type=int, default=200)
+    p.add_argument("--warmup", type=int, default=20)
+    p.add_argument("--no-cpu-baseline", action="store_true")
+    return p.parse_args()
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: the routing hot path is built and measured on a "
+                 "single MI355X (no collectives in this build); run with --gpus 1")
+    import numpy as np
+    import torch
+
+    from brainstorm_amd import _lib
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    L = _lib.lib()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    stream = torch.cuda.Stream()  # every kernel and every timing event goes on this stream
+
+    # ---------------------------------------------------------------- inputs
+    g = torch.Generator().manual_seed(SEED)
+    x32 = torch.randn(T, D, generator=g)
+    logits = torch.randn(T, E, generator=g)
+    probs = torch.softmax(logits, dim=1)
+    expert = probs.argmax(dim=1)
+    mask_h = torch.zeros(T, E, dtype=torch.int32)
+    mask_h[torch.arange(T), expert] = 1
+    wi_h = (torch.randn(E, DFF, D, generator=g) * 0.02).to(torch.bfloat16)
+    wo_h = (torch.randn(E, D, DFF, generator=g) * 0.02).to(torch.bfloat16)
+
+    x = x32.to(torch.bfloat16).to(dev)
+    mask = mask_h.to(dev)
+    caps = torch.tensor([CAPACITY], dtype=torch.int32, device=dev)
+    idx = torch.empty_like(mask)
+    loads_counts = torch.empty(2, E, dtype=torch.int32, device=dev)
+    loads, counts = loads_counts[0], loads_counts[1]
+    ws = torch.empty(max(16, L.brt_hip_scan_workspace_bytes(T, E)), dtype=torch.uint8, device=dev)
+
+    def sptr():
+        return stream.cuda_stream
+
+    def k_indexgen():
+        _lib.check(L.brt_hip_generate_indices_and_loads(
+            mask.data_ptr(), idx.data_ptr(), loads.data_ptr(), counts.data_ptr(), T, E,
+            caps.data_ptr(), 1, 0, 0, 0, ws.data_ptr(), ws.numel(), sptr()))
+
+    with torch.cuda.stream(stream):
+        k_indexgen()
+    stream.synchronize()
+    loads_h, counts_h = loads.cpu(), counts.cpu()
+    P = int(loads_h.sum())                               # rows of the dispatched buffer
+    R = int(torch.minimum(loads_h, counts_h).sum())      # rows actually routed
+    y = torch.empty(P, D, dtype=torch.bfloat16, device=dev)
+    out = x.clone()                                      # residual: unrouted tokens keep x
+
+    wi = wi_h.to(dev)
+    wo = wo_h.to(dev)
+    wi_tab = torch.tensor([wi[e].data_ptr() for e in range(E)], dtype=torch.int64, device=dev)
+    wo_tab = torch.tensor([wo[e].data_ptr() for e in range(E)], dtype=torch.int64, device=dev)
+    h = torch.empty(P, DFF, dtype=torch.bfloat16, device=dev)
+    y2 = torch.empty(P, D, dtype=torch.bfloat16, device=dev)
+
+    def k_dispatch():
+        _lib.check(L.brt_hip_dispatch(
+            x.data_ptr(), y.data_ptr(), None, idx.data_ptr(), loads.data_ptr(), counts.data_ptr(),
+            None, None, T, D, E, P, 0, 1, 0, _lib.BF16, sptr()))
+
+    def k_gemm1():
+        _lib.check(L.brt_hip_grouped_gemm(
+            y.data_ptr(), wi_tab.data_ptr(), None, h.data_ptr(), loads.data_ptr(), E, P, D, DFF,
+            _lib.ACT_GELU, sptr()))
+
+    def k_gemm2():
+        _lib.check(L.brt_hip_grouped_gemm(
+            h.data_ptr(), wo_tab.data_ptr(), None, y2.data_ptr(), loads.data_ptr(), E, P, DFF, D,
+            _lib.ACT_NONE, sptr()))
+
+    have_ffn = True
+    try:
+        with torch.cuda.stream(stream):
+            k_gemm1()
+            k_gemm2()
+        stream.synchronize()
+    except (NotImplementedError, RuntimeError) as err:
+        have_ffn = False
+        ffn_note = str(err)
+
+    combine_src = y2 if have_ffn else y
+
+    def k_combine():
+        _lib.check(L.brt_hip_combine(
+            combine_src.data_ptr(), out.data_ptr(), None, idx.data_ptr(), loads.data_ptr(), T, D,
+            E, P, 0, 1, _lib.BF16, _lib.BF16, _lib.F32, sptr()))
+
+    def step():
+        k_indexgen()
+        k_dispatch()
+        if have_ffn:
+            k_gemm1()
+            k_gemm2()
+        k_combine()
+
+    def capture(fn, repeat=1):
+        with torch.cuda.stream(stream):
+            for _ in range(2):
+                fn()
+        stream.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            for _ in range(repeat):
+                fn()
+        return graph
+
+    def timed(graph, replays):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        with torch.cuda.stream(stream):
+            a.record(stream)
+            for _ in range(replays):
+                graph.replay()
+            b.record(stream)
+        stream.synchronize()
+        return a.elapsed_time(b)  # ms
+
+    # ------------------------------------------------------- timed region: K steps
+    g_step = capture(step)
+    with torch.cuda.stream(stream):
+        for _ in range(args.warmup):
+            g_step.replay()
+    stream.synchronize()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ms_total = timed(g_step, args.steps)
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    ms_per_step = ms_total / args.steps
+
+    # ---------------------------------------- per-kernel durations (same process)
+    INNER = 20
+    kernels = {"indexgen": k_indexgen, "dispatch": k_dispatch, "combine": k_combine}
+    if have_ffn:
+        kernels.update({"ffn_gemm1_gelu": k_gemm1, "ffn_gemm2": k_gemm2})
+    replays = max(10, args.steps // 4)
+    us = {}
+    for name, fn in kernels.items():
+        gk = capture(fn, INNER)
+        timed(gk, 3)
+        runs = [timed(gk, replays) for _ in range(3)]
+        us[name] = sum(runs) / len(runs) * 1e3 / (replays * INNER)  # average launch duration
+
+    es = 2  # bf16
+    idx_bytes = 4 * T * E
+    bytes_ = {
+        "indexgen": 2 * idx_bytes + 4 * E,
+        "dispatch": R * D * es + P * D * es + idx_bytes,
+        "combine": R * D * es + T * D * es + idx_bytes,
+    }
+    flops = {"ffn_gemm1_gelu": 2.0 * R * D * DFF, "ffn_gemm2": 2.0 * R * DFF * D}
+    dc_bytes = bytes_["dispatch"] + bytes_["combine"]
+    dc_us = us["dispatch"] + us["combine"]
+    value = dc_bytes / dc_us / 1e3  # GB/s
+
+    dominant = "combine" if us["combine"] >= us["dispatch"] else "dispatch"
+    roofline = {
+        "kernel": dominant,
+        "bound": "hbm",
+        "achieved": round(bytes_[dominant] / us[dominant] / 1e3, 1),
+        "peak": HBM_PEAK_GBPS,
+        "unit": "GB/s",
+        "frac": round(bytes_[dominant] / us[dominant] / 1e3 / HBM_PEAK_GBPS, 4),
+        "traffic": MEASURED_TRAFFIC_BYTES.get(dominant),
+        "avg_us": round(us[dominant], 3),
+        "algorithmic_bytes": bytes_[dominant],
+    }
+    per_kernel = {}
+    for name in us:
+        entry = {"us": round(us[name], 3)}
+        if name in bytes_:
+            entry["GBps"] = round(bytes_[name] / us[name] / 1e3, 1)
+            entry["hbm_frac"] = round(bytes_[name] / us[name] / 1e3 / HBM_PEAK_GBPS, 4)
+        if name in flops:
+            entry["TFLOPs"] = round(flops[name] / us[name] / 1e6, 1)
+            entry["mfma_frac"] = round(flops[name] / us[name] / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4)
+        per_kernel[name] = entry
+
+    # ------------------------------------------------------------ CPU baseline
+    cpu_baseline = None
+    if not args.no_cpu_baseline:
+        from oracle import torch_path
+
+        cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+        torch.set_num_threads(cores)
+        m_idx, m_loads = torch_path.generate_indices_and_loads(mask_h, [CAPACITY], False)
+        for _ in range(3):
+            yy = torch_path.dispatch(x32, m_idx, m_loads)
+            torch_path.combine(yy, m_idx, m_loads, None, x32)
+        reps, spent = 0, 0.0
+        t_dc = []
+        while (spent < 10.0 and reps < 200) or reps < 5:
+            t1 = time.perf_counter()
+            yy = torch_path.dispatch(x32, m_idx, m_loads)
+            torch_path.combine(yy, m_idx, m_loads, None, x32)
+            dt = time.perf_counter() - t1
+            t_dc.append(dt)
+            spent += dt
+            reps += 1
+        med = float(np.median(t_dc))
+        cpu_bytes = 2 * R * D * 4 + P * D * 4 + T * D * 4 + 2 * idx_bytes  # same ops in fp32
+        cpu_baseline = {
+            "value": round(cpu_bytes / med / 1e9, 2),
+            "unit": "GB/s",
+            "cores": torch.get_num_threads(),
+            "kind": "port",
+            "sample": (f"{reps} passes of torch CPU dispatch+combine (index_select / index_add_, "
+                       f"fp32) on the same {T}x{D} x {E}-expert inputs, median {med * 1e3:.2f} ms"),
+        }
+
+    result = {
+        "metric": "dispatch+combine GB/s",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": "Switch-MoE layer routing hot path (BASELINE.json configs[1])",
+            "tokens": T, "d_model": D, "experts": E, "d_ff": DFF, "top_k": 1,
+            "capacity": CAPACITY, "capacity_mode": "clip (overflow dropped, no padding)",
+            "routed_rows": R, "dispatched_rows": P, "seed": SEED,
+            "step": "indexgen+dispatch+" + ("ffn(2 grouped GEMMs)+" if have_ffn else "") + "combine, one HIP graph",
+        },
+        "hbm_peak_frac": round(value / HBM_PEAK_GBPS, 4),
+        "layer_us": round(ms_per_step * 1e3, 2),
+        "wall_ms_timed_region": round(wall_ms, 3),
+        "algorithmic_bytes_dispatch_combine": dc_bytes,
+        "kernels": per_kernel,
+        "roofline": roofline,
+        "cpu_baseline": cpu_baseline,
+    }
+    if not have_ffn:
+        result["ffn"] = None
+        result["ffn_note"] = ffn_note
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()
