@@ -9,22 +9,29 @@
 // here the tile -> (expert, row block) map is computed on the device from
 // `loads`, so any non-negative loads work and nothing is copied to the host.
 //
-// Tiling (CDNA4, wave64): a 256-thread workgroup owns a BM x BN output tile and
-// walks K in steps of 64.  Both operands are K-contiguous in memory, which is the
-// MFMA operand layout (each lane feeds 8 consecutive k of one row/column), so
-// tiles go global -> registers -> LDS as 16-byte chunks without any transpose and
-// come back out of LDS as ds_read_b128 fragments.  LDS rows are padded by 16 bytes
-// so that 8 consecutive rows hit 8 distinct bank groups.  Two LDS stages: the next
-// K-step is in flight in registers while the current one feeds
-// v_mfma_f32_32x32x16_bf16 (fp32 accumulate); one barrier per K-step.  The
-// epilogue (bias, GELU/ReLU, round to bf16) goes through LDS so that the stores
-// are full 16-byte, row-contiguous accesses.
+// Tiling (CDNA4, wave64).  The expert FFN is a skinny GEMM (at most a few hundred
+// rows per expert) whose cost is streaming the weights, so the tile is chosen to
+// read them once: a workgroup owns BM = 32*MT rows (160 covers a whole capacity-
+// padded Switch expert) by BN = 32*WAVES columns, every wavefront owning all BM
+// rows of its own 32 columns.  Both operands are K-contiguous in memory, which is
+// the MFMA operand layout (a lane feeds 8 consecutive k of one row), so tiles
+// travel global -> registers -> LDS as 16-byte chunks without any transpose and
+// come back as ds_read_b128 fragments; chunk c of row r lives in slot c ^ (r & 7)
+// so that the 8 rows a read touches per cycle fall into distinct bank groups
+// without padding.  The loop is bound by memory latency, not by MFMA issue, so it
+// keeps two K-steps in flight in registers on top of the two LDS stages (one
+// barrier per K-step of 64).  v_mfma_f32_32x32x16_bf16 is issued with the weight
+// fragment as its first operand: the accumulator then holds the transposed tile,
+// i.e. four consecutive output columns of one row per lane, which makes the
+// epilogue (bias, GELU/ReLU, round to bf16) an 8-byte LDS write per group and the
+// final stores full 16-byte, row-contiguous accesses.
 //
-// Workgroups are renumbered so that consecutive logical tiles run on the same
-// XCD (hardware deals workgroups round-robin over the 8 XCDs): the BN-wide column
-// tiles of one row block then share that XCD's L2 copy of the activation rows.
+// Workgroups are renumbered so that the column tiles of one row block run on the
+// same XCD (hardware deals workgroups round-robin over the 8 XCDs) and share that
+// XCD's L2 copy of the activation rows, while row blocks alternate between XCDs.
 #include <algorithm>
 #include <cstdlib>
+#include <type_traits>
 
 #include "common.hpp"
 
@@ -32,13 +39,19 @@ namespace brt {
 namespace {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+// Pointers read from the per-expert table are generic to the compiler, which would
+// make every weight load a flat load counted on the LDS counter as well; the
+// explicit global address space keeps weight loads off the LDS wait path.
+typedef const __bf16 __attribute__((address_space(1)))* global_bf16;
+typedef const u32x4 __attribute__((address_space(1)))* global_u32x4;
+typedef const bf16x4 __attribute__((address_space(1)))* global_bf16x4;
 
-constexpr int kThreads = 256;
-constexpr int kBK = 64;                    // k elements per stage
-constexpr int kChunks = kBK / 8;           // 16-byte chunks per tile row
-constexpr int kRowBytes = kBK * 2 + 16;    // padded LDS row
+constexpr int kBK = 64;               // k elements per stage
+constexpr int kChunks = kBK / 8;      // 16-byte chunks per tile row
+constexpr int kRowBytes = kBK * 2;    // LDS row (swizzled, unpadded)
 constexpr int kXcds = 8;
 
 struct GemmArgs {
@@ -49,32 +62,71 @@ struct GemmArgs {
   const int* loads;
   int E, P, K, N;
   int tiles_n, tiles_m_max;
-  int act;
 };
 
-__device__ __forceinline__ float apply_act(float v, int act) {
-  if (act == BRT_ACT_GELU) return 0.5f * v * (1.0f + erff(v * 0.70710678118654752f));
-  if (act == BRT_ACT_RELU) return fmaxf(v, 0.0f);
+// erf to 1.5e-7 absolute (Abramowitz & Stegun 7.1.26), branch free.
+__device__ __forceinline__ float fast_erf(float x) {
+  const float ax = fabsf(x);
+  const float t = __frcp_rn(__builtin_fmaf(0.3275911f, ax, 1.0f));
+  float p = 1.061405429f;
+  p = __builtin_fmaf(p, t, -1.453152027f);
+  p = __builtin_fmaf(p, t, 1.421413741f);
+  p = __builtin_fmaf(p, t, -0.284496736f);
+  p = __builtin_fmaf(p, t, 0.254829592f);
+  const float r = 1.0f - p * t * __expf(-ax * ax);
+  return copysignf(r, x);
+}
+
+template <int ACT>
+__device__ __forceinline__ float apply_act(float v) {
+  if (ACT == BRT_ACT_GELU) return 0.5f * v * (1.0f + fast_erf(v * 0.70710678118654752f));
+  if (ACT == BRT_ACT_RELU) return fmaxf(v, 0.0f);
   return v;
 }
 
-template <int BM, int BN>
-__global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmArgs a) {
-  constexpr int WM = BM / 2, WN = BN / 2;  // 2 x 2 wavefronts
-  constexpr int TM = WM / 32, TN = WN / 32;
-  constexpr int A_BYTES = BM * kRowBytes, B_BYTES = BN * kRowBytes;
-  constexpr int STAGE = A_BYTES + B_BYTES;
-  constexpr int A_LOADS = BM * kChunks / kThreads, B_LOADS = BN * kChunks / kThreads;
+#ifdef BRT_GEMM_TRACE
+constexpr int kTraceSlots = 64, kTraceBlocks = 4096;
+__device__ unsigned long long g_trace[kTraceBlocks * kTraceSlots];
+#define TRACE(slot)                                                                   \
+  do {                                                                                \
+    if (threadIdx.x == 0 && blockIdx.x < kTraceBlocks && (slot) < kTraceSlots)        \
+      g_trace[blockIdx.x * kTraceSlots + (slot)] = wall_clock64();                    \
+  } while (0)
+#else
+#define TRACE(slot)
+#endif
+
+template <int N>
+struct Staged {
+  u32x4 v[N];
+};
+
+template <int MT, int NT, int WAVES, int ACT>
+__global__ __launch_bounds__(WAVES * 64) void grouped_gemm_kernel(GemmArgs a) {
+  constexpr int THREADS = WAVES * 64;
+  constexpr int BM = MT * 32, WN = NT * 32, BN = WAVES * WN;
+  constexpr int TILE_ROWS = BM + BN;  // activation rows first, then weight rows
+  constexpr int STAGE = TILE_ROWS * kRowBytes;
+  constexpr int ROWS_PER_PASS = THREADS / kChunks;  // rows one load instruction of the block covers
+  constexpr int A_LOADS = (BM + ROWS_PER_PASS - 1) / ROWS_PER_PASS;
+  constexpr int B_LOADS = BN / ROWS_PER_PASS;
+  constexpr bool A_EXACT = BM % ROWS_PER_PASS == 0;
+  static_assert(BN % ROWS_PER_PASS == 0 && ROWS_PER_PASS % 8 == 0, "tile shape");
   constexpr int OUT_ROW = BN * 2 + 16;
   extern __shared__ __attribute__((aligned(16))) char smem[];
   __shared__ int s_tile[3];  // expert, first row, valid rows
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  TRACE(0);
 
   // ---- which tile: XCD-aware renumbering, then expert lookup from the loads ----------
-  const int per_xcd = gridDim.x / kXcds;
-  const int logical = (blockIdx.x % kXcds) * per_xcd + blockIdx.x / kXcds;
-  const int mt = logical / a.tiles_n, nt = logical - mt * a.tiles_n;
+  // hardware deals workgroups round-robin over the XCDs: workgroup b runs on XCD b % 8.
+  // Row blocks are dealt round-robin too (row block m on XCD m % 8, so the row blocks
+  // that really exist -- only the device knows how many -- spread evenly), and the
+  // column tiles of one row block are consecutive workgroups of that XCD.
+  const int xcd = blockIdx.x % kXcds, idx = blockIdx.x / kXcds;
+  const int mt = (idx / a.tiles_n) * kXcds + xcd, nt = idx % a.tiles_n;
   if (mt >= a.tiles_m_max) return;
   if (tid < kWave) {
     int carry_t = 0, carry_m = 0;
@@ -102,135 +154,257 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmArgs a) {
     if (!found && lane == 0) s_tile[0] = -1;
   }
   __syncthreads();
-  const int e = s_tile[0];
+  const int e = __builtin_amdgcn_readfirstlane(s_tile[0]);
   if (e < 0) return;  // beyond the last tile
-  const int row0 = s_tile[1], rows = s_tile[2];
+  const int row0 = __builtin_amdgcn_readfirstlane(s_tile[1]);
+  const int rows = __builtin_amdgcn_readfirstlane(s_tile[2]);
+  const int row_tiles = (rows + 31) >> 5;
   const int n0 = nt * BN;
   const int K = a.K;
 
-  const __bf16* __restrict__ xa = a.x + static_cast<size_t>(row0) * K;
-  const __bf16* __restrict__ wb = a.w[e] + static_cast<size_t>(n0) * K;
-
-  // global -> register staging: thread t owns chunk (t % 8) of rows t/8 + 32 i
+  // ---- global -> register staging ------------------------------------------------
+  // Thread t owns 16-byte chunk t%8 of rows t/8 + i*ROWS_PER_PASS of the activation
+  // tile and of the weight tile.  Rows past the expert's last row or past N are
+  // clamped to a valid row (their products land in output rows/columns that are
+  // never stored, and all MT row tiles are always multiplied: the inner loop stays
+  // one branch-free block); only a K tail that is not a multiple of 64 needs real
+  // zeros.
   const int lc = tid % kChunks, lr = tid / kChunks;
-  u32x4 ra[A_LOADS], rb[B_LOADS];
-  auto fetch = [&](int k0) {
-    const bool k_ok = k0 + lc * 8 < K;
+  // Buffer loads: a wave-uniform resource (base, byte extent) per operand, a 32-bit
+  // per-lane byte offset and the K offset as the scalar offset, so the loop carries no
+  // 64-bit address arithmetic; reads past the extent return zero instead of faulting.
+  const char* xa = reinterpret_cast<const char*>(a.x + static_cast<size_t>(row0) * K);
+  const char* wb = reinterpret_cast<const char*>(a.w[e] + static_cast<size_t>(n0) * K);
+  const size_t xa_bytes = static_cast<size_t>(a.P - row0) * K * 2;
+  const size_t wb_bytes = static_cast<size_t>(a.N - n0) * K * 2;
+  const __amdgpu_buffer_rsrc_t res_a = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<char*>(xa), 0, static_cast<int>(std::min<size_t>(xa_bytes, 0x7fffffff)), 0x00020000);
+  const __amdgpu_buffer_rsrc_t res_b = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<char*>(wb), 0, static_cast<int>(std::min<size_t>(wb_bytes, 0x7fffffff)), 0x00020000);
+  // when ROWS_PER_PASS does not divide BM only the lower wavefronts take the last pass
+  const bool a_last = A_EXACT || lr + (A_LOADS - 1) * ROWS_PER_PASS < BM;
+  uint32_t off_a[A_LOADS], off_b[B_LOADS];
 #pragma unroll
-    for (int i = 0; i < A_LOADS; ++i) {
-      const int r = lr + i * (kThreads / kChunks);
-      u32x4 z = {};
-      ra[i] = (k_ok && r < rows)
-                  ? *reinterpret_cast<const u32x4*>(xa + static_cast<size_t>(r) * K + k0 + lc * 8)
-                  : z;
-    }
+  for (int i = 0; i < A_LOADS; ++i)
+    off_a[i] = (static_cast<uint32_t>(min(min(lr + i * ROWS_PER_PASS, BM - 1), rows - 1)) * K + lc * 8) * 2;
 #pragma unroll
-    for (int i = 0; i < B_LOADS; ++i) {
-      const int r = lr + i * (kThreads / kChunks);
-      u32x4 z = {};
-      rb[i] = (k_ok && n0 + r < a.N)
-                  ? *reinterpret_cast<const u32x4*>(wb + static_cast<size_t>(r) * K + k0 + lc * 8)
-                  : z;
-    }
-  };
-  auto stash = [&](int stage) {
-    char* sa = smem + stage * STAGE;
-    char* sb = sa + A_BYTES;
-#pragma unroll
-    for (int i = 0; i < A_LOADS; ++i) {
-      const int r = lr + i * (kThreads / kChunks);
-      *reinterpret_cast<u32x4*>(sa + r * kRowBytes + lc * 16) = ra[i];
-    }
-#pragma unroll
-    for (int i = 0; i < B_LOADS; ++i) {
-      const int r = lr + i * (kThreads / kChunks);
-      *reinterpret_cast<u32x4*>(sb + r * kRowBytes + lc * 16) = rb[i];
-    }
-  };
+  for (int i = 0; i < B_LOADS; ++i)
+    off_b[i] = (static_cast<uint32_t>(min(lr + i * ROWS_PER_PASS, a.N - n0 - 1)) * K + lc * 8) * 2;
+  // LDS slot of chunk c of row r is c ^ (r & 7); ROWS_PER_PASS is a multiple of 8, so
+  // the swizzle is the same for every pass of this thread
+  const int slot = lr * kRowBytes + ((lc ^ (lr & 7)) << 4);
+  const bool k_tail = (K % kBK) != 0;
 
-  f32x16 acc[TM][TN];
+  using Yes = std::integral_constant<bool, true>;
+  using No = std::integral_constant<bool, false>;
+  constexpr int LOADS = A_LOADS + B_LOADS;
+  constexpr int kSteps = kBK / 16;
+  // Loads and LDS writes are issued in kSteps slices so that they can be spread over
+  // the k-steps of the multiply; slice p covers loads [p*LOADS/kSteps, (p+1)*LOADS/kSteps).
+  auto fetch_slice = [&](Staged<LOADS>& s, int k0, int p) {
 #pragma unroll
-  for (int i = 0; i < TM; ++i)
-#pragma unroll
-    for (int j = 0; j < TN; ++j) acc[i][j] = f32x16{};
-
-  const int wm = wave >> 1, wn = wave & 1;
-  const int frag_row = lane & 31, frag_k = lane >> 5;  // MFMA operand: row / k-half of this lane
-
-  fetch(0);
-  stash(0);
-  __syncthreads();
-  const int k_tiles = (K + kBK - 1) / kBK;
-  for (int kt = 0; kt < k_tiles; ++kt) {
-    if (kt + 1 < k_tiles) fetch((kt + 1) * kBK);
-    const char* sa = smem + (kt & 1) * STAGE;
-    const char* sb = sa + A_BYTES;
-#pragma unroll
-    for (int ks = 0; ks < kBK / 16; ++ks) {
-      bf16x8 fa[TM], fb[TN];
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-        fa[i] = *reinterpret_cast<const bf16x8*>(
-            sa + (wm * WM + i * 32 + frag_row) * kRowBytes + (ks * 2 + frag_k) * 16);
-#pragma unroll
-      for (int j = 0; j < TN; ++j)
-        fb[j] = *reinterpret_cast<const bf16x8*>(
-            sb + (wn * WN + j * 32 + frag_row) * kRowBytes + (ks * 2 + frag_k) * 16);
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
-    }
-    if (kt + 1 < k_tiles) stash((kt + 1) & 1);
-    __syncthreads();
-  }
-
-  // ---- epilogue: bias + activation, bf16, through LDS, 16-byte row stores ---------------
-  // accumulator r of a 32x32 tile: row 8*(r/4) + 4*(lane/32) + r%4, column lane%32
-  const __bf16* bias = a.bias != nullptr ? a.bias[e] : nullptr;
-#pragma unroll
-  for (int i = 0; i < TM; ++i)
-#pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      const int col = wn * WN + j * 32 + (lane & 31);
-      const float b = (bias != nullptr && n0 + col < a.N) ? static_cast<float>(bias[n0 + col]) : 0.0f;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int row = wm * WM + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
-        const float v = apply_act(acc[i][j][r] + b, a.act);
-        *reinterpret_cast<__bf16*>(smem + row * OUT_ROW + col * 2) = static_cast<__bf16>(v);
+    for (int i = 0; i < LOADS; ++i) {
+      if (i < p * LOADS / kSteps || i >= (p + 1) * LOADS / kSteps) continue;
+      if (i < A_LOADS) {
+        if (i + 1 < A_LOADS || a_last)
+          s.v[i] = __builtin_amdgcn_raw_buffer_load_b128(res_a, off_a[i < A_LOADS ? i : 0], k0 * 2, 0);
+      } else {
+        s.v[i] = __builtin_amdgcn_raw_buffer_load_b128(res_b, off_b[i >= A_LOADS ? i - A_LOADS : 0],
+                                                       k0 * 2, 0);
       }
     }
+  };
+  // the K tail (only ever in the last tile) is zeroed here, when the data is in registers
+  auto stash_slice = [&](const Staged<LOADS>& s, int stage, int k0, int p, auto may_be_last) {
+    char* base = smem + stage * STAGE + slot;
+    const bool k_ok = !decltype(may_be_last)::value || !k_tail || k0 + lc * 8 < K;
+    const u32x4 z = {};
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i) {
+      if (i < p * LOADS / kSteps || i >= (p + 1) * LOADS / kSteps) continue;
+      const u32x4 v = k_ok ? s.v[i] : z;
+      if (i < A_LOADS) {
+        if (i + 1 < A_LOADS || a_last)
+          *reinterpret_cast<u32x4*>(base + i * ROWS_PER_PASS * kRowBytes) = v;
+      } else {
+        *reinterpret_cast<u32x4*>(base + (BM + (i - A_LOADS) * ROWS_PER_PASS) * kRowBytes) = v;
+      }
+    }
+  };
+
+  f32x16 acc[MT][NT];
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+#pragma unroll
+    for (int j = 0; j < NT; ++j) acc[i][j] = f32x16{};
+
+  // MFMA operand: this lane feeds row (lane % 32), k-half (lane / 32) of a 32 x 16 block
+  const int frag_row = lane & 31, frag_k = lane >> 5;
+
+  // One K-step of 64: multiply the tile in LDS stage `stage`; meanwhile write the tile
+  // that has arrived in `arrived` (K offset k_arrived) to the other stage and start
+  // loading the tile after that (K offset k_fetch) into `incoming`.  With one wavefront
+  // per SIMD nothing hides a stalled instruction stream, so every 16-wide k-step is
+  // issued as MFMA, memory op, MFMA, memory op, ...: the global loads, the fragment
+  // reads of the next k-step and the LDS writes each ride behind an MFMA that keeps the
+  // matrix pipe busy while they issue.
+  auto step = [&](int stage, Staged<LOADS>& incoming, const Staged<LOADS>& arrived, int k_fetch,
+                  int k_arrived, auto do_fetch, auto do_stash, auto last_tile) {
+    constexpr bool kFetch = decltype(do_fetch)::value, kStash = decltype(do_stash)::value;
+    const char* sa = smem + stage * STAGE + frag_row * kRowBytes;
+    const char* sb = sa + (BM + wave * WN) * kRowBytes;
+    bf16x8 fw[2][NT], fx[2][MT];
+    auto read_frags = [&](int ks, int buf) {
+      const int phys = ((ks * 2 + frag_k) ^ (frag_row & 7)) << 4;
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+        fw[buf][j] = *reinterpret_cast<const bf16x8*>(sb + j * 32 * kRowBytes + phys);
+#pragma unroll
+      for (int i = 0; i < MT; ++i)
+        fx[buf][i] = *reinterpret_cast<const bf16x8*>(sa + i * 32 * kRowBytes + phys);
+    };
+    read_frags(0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int ks = 0; ks < kSteps; ++ks) {
+#ifndef DBG_NO_FETCH
+      if constexpr (kFetch) fetch_slice(incoming, k_fetch, ks);
+#endif
+      if (ks + 1 < kSteps) read_frags(ks + 1, (ks + 1) & 1);
+#pragma unroll
+      for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int j = 0; j < NT; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fw[ks & 1][j], fx[ks & 1][i],
+                                                              acc[i][j], 0, 0, 0);
+#ifndef DBG_NO_STASH
+      if constexpr (kStash) stash_slice(arrived, stage ^ 1, k_arrived, ks, last_tile);
+#endif
+      // issue order of this k-step: one MFMA, then at most one op of each memory kind
+      constexpr int kSlice = (LOADS + kSteps - 1) / kSteps;
+      constexpr int kReads = MT + NT;
+#pragma unroll
+      for (int m = 0; m < MT * NT; ++m) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                     // MFMA
+        if (m < kReads) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);      // LDS read
+        if (kFetch && m < kSlice) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // global load
+        if (kStash && m >= MT * NT - kSlice) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);  // LDS write
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
+  // ---- K loop: tile kt in LDS stage kt&1, tile kt+1 in one register set (written to LDS
+  // during step kt), tile kt+2 being loaded into the other ------------------------------
+  const int k_tiles = (K + kBK - 1) / kBK;
+  Staged<LOADS> s0, s1;
+  TRACE(1);
+#pragma unroll
+  for (int p = 0; p < kSteps; ++p) fetch_slice(s0, 0, p);
+  if (k_tiles > 1) {
+#pragma unroll
+    for (int p = 0; p < kSteps; ++p) fetch_slice(s1, kBK, p);
+  }
+#pragma unroll
+  for (int p = 0; p < kSteps; ++p) stash_slice(s0, 0, 0, p, Yes{});
   __syncthreads();
+  TRACE(2);
+  int kt = 0;
+  for (; kt + 3 < k_tiles; kt += 2) {
+    step(0, s0, s1, (kt + 2) * kBK, (kt + 1) * kBK, Yes{}, Yes{}, No{});
+    TRACE(4 + 3 * kt);
+    __syncthreads();
+    TRACE(6 + 3 * kt);
+    step(1, s1, s0, (kt + 3) * kBK, (kt + 2) * kBK, Yes{}, Yes{}, No{});
+    TRACE(7 + 3 * kt);
+    __syncthreads();
+    TRACE(9 + 3 * kt);
+  }
+  const int left = k_tiles - kt;  // 1, 2 or 3 tiles; kt is even, so the next tile is in stage 0
+  if (left == 3) {
+    step(0, s0, s1, (kt + 2) * kBK, (kt + 1) * kBK, Yes{}, Yes{}, No{});
+    __syncthreads();
+    step(1, s1, s0, 0, (kt + 2) * kBK, No{}, Yes{}, Yes{});
+    __syncthreads();
+    step(0, s0, s1, 0, 0, No{}, No{}, No{});
+  } else if (left == 2) {
+    step(0, s0, s1, 0, (kt + 1) * kBK, No{}, Yes{}, Yes{});
+    __syncthreads();
+    step(1, s1, s0, 0, 0, No{}, No{}, No{});
+  } else {
+    step(0, s0, s1, 0, 0, No{}, No{}, No{});
+  }
+  __syncthreads();
+
+  // ---- epilogue: bias + activation, bf16, through LDS, 16-byte row stores ---------------
+  // transposed accumulator: element r of tile (i, j) is output row 32 i + lane%32, column
+  // (of this wavefront's 32 j .. 32 j + 31) 8*(r/4) + 4*(lane/32) + r%4
+  const global_bf16 bias = a.bias != nullptr ? (global_bf16)(a.bias[e]) : (global_bf16)nullptr;
+#pragma unroll
+  for (int j = 0; j < NT; ++j) {
+    float bv[4][4];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int col = n0 + wave * WN + j * 32 + 8 * g + 4 * frag_k;
+      bf16x4 b4 = {};
+      if (a.bias != nullptr && col < a.N) b4 = *(global_bf16x4)(bias + col);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) bv[g][q] = static_cast<float>(b4[q]);
+    }
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+      if (i < row_tiles) {
+        char* dst = smem + (i * 32 + frag_row) * OUT_ROW + (wave * WN + j * 32 + 4 * frag_k) * 2;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          bf16x4 o;
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+            o[q] = static_cast<__bf16>(apply_act<ACT>(acc[i][j][4 * g + q] + bv[g][q]));
+          *reinterpret_cast<bf16x4*>(dst + 16 * g) = o;
+        }
+      }
+    }
+  }
+  __syncthreads();
+  TRACE(62);
   constexpr int OUT_CHUNKS = BN / 8;
   __bf16* __restrict__ oc = a.out + static_cast<size_t>(row0) * a.N + n0;
-  for (int q = tid; q < BM * OUT_CHUNKS; q += kThreads) {
+  for (int q = tid; q < rows * OUT_CHUNKS; q += THREADS) {
     const int r = q / OUT_CHUNKS, c = q - r * OUT_CHUNKS;
-    if (r < rows && n0 + c * 8 < a.N)
+    if (n0 + c * 8 < a.N)
       *reinterpret_cast<u32x4*>(oc + static_cast<size_t>(r) * a.N + c * 8) =
           *reinterpret_cast<const u32x4*>(smem + r * OUT_ROW + c * 16);
   }
+  TRACE(63);
 }
 
-template <int BM, int BN>
-int launch(GemmArgs& a, hipStream_t st) {
+template <int MT, int NT, int WAVES, int ACT>
+int launch_act(GemmArgs& a, hipStream_t st) {
+  constexpr int BM = MT * 32, BN = WAVES * NT * 32;
   constexpr int STAGE = (BM + BN) * kRowBytes;
   constexpr int OUT_BYTES = BM * (BN * 2 + 16);
   const size_t lds = std::max(2 * STAGE, OUT_BYTES);
   a.tiles_n = (a.N + BN - 1) / BN;
-  a.tiles_m_max = (a.P + BM - 1) / BM + a.E;  // sum over experts of ceil(M_e/BM) never exceeds this
-  long grid = static_cast<long>(a.tiles_m_max) * a.tiles_n;
-  grid = (grid + kXcds - 1) / kXcds * kXcds;
+  // sum over experts of ceil(M_e/BM) never exceeds P/BM + E; rounded up to whole XCD rounds
+  a.tiles_m_max = ((a.P + BM - 1) / BM + a.E + kXcds - 1) / kXcds * kXcds;
+  const long grid = static_cast<long>(a.tiles_m_max) * a.tiles_n;
   static bool configured = false;
   if (!configured) {
-    hipFuncSetAttribute(reinterpret_cast<const void*>(&grouped_gemm_kernel<BM, BN>),
+    hipFuncSetAttribute(reinterpret_cast<const void*>(&grouped_gemm_kernel<MT, NT, WAVES, ACT>),
                         hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
     configured = true;
   }
-  hipLaunchKernelGGL((grouped_gemm_kernel<BM, BN>), dim3(static_cast<unsigned>(grid)),
-                     dim3(kThreads), lds, st, a);
+  hipLaunchKernelGGL((grouped_gemm_kernel<MT, NT, WAVES, ACT>), dim3(static_cast<unsigned>(grid)),
+                     dim3(WAVES * 64), lds, st, a);
   return check_launch("grouped_gemm_kernel");
+}
+
+template <int MT, int NT, int WAVES>
+int launch(GemmArgs& a, int act, hipStream_t st) {
+  if (act == BRT_ACT_GELU) return launch_act<MT, NT, WAVES, BRT_ACT_GELU>(a, st);
+  if (act == BRT_ACT_RELU) return launch_act<MT, NT, WAVES, BRT_ACT_RELU>(a, st);
+  return launch_act<MT, NT, WAVES, BRT_ACT_NONE>(a, st);
 }
 
 }  // namespace
@@ -255,6 +429,20 @@ extern "C" int brt_hip_grouped_gemm(const void* x, const void* const* weights,
   a.bias = reinterpret_cast<const __bf16* const*>(biases);
   a.out = static_cast<__bf16*>(out);
   a.loads = loads;
-  a.E = E; a.P = P; a.K = K; a.N = N; a.act = act;
-  return launch<128, 128>(a, as_stream(stream));
+  a.E = E; a.P = P; a.K = K; a.N = N;
+  // Tile choice: a wavefront owns 160 x 64 outputs (7 LDS fragment reads feed 10 MFMAs;
+  // LDS read bandwidth is what bounds the inner loop).  Wide outputs use 4 wavefronts
+  // (160 x 256 per workgroup); narrow ones use 2 (160 x 128) so that the grid still
+  // has more workgroups than the chip has compute units.
+  static const int forced = std::getenv("BRT_GEMM_SHAPE") ? std::atoi(std::getenv("BRT_GEMM_SHAPE")) : 0;
+  const int shape = forced ? forced : (N >= 2048 ? 24 : 22);
+  if (shape == 24) return launch<5, 2, 4>(a, act, as_stream(stream));
+  if (shape == 22) return launch<5, 2, 2>(a, act, as_stream(stream));
+  return launch<5, 1, 4>(a, act, as_stream(stream));
 }
+
+#ifdef BRT_GEMM_TRACE
+extern "C" int brt_hip_debug_trace(void* host, size_t bytes) {
+  return hipMemcpyFromSymbol(host, HIP_SYMBOL(brt::g_trace), bytes) == hipSuccess ? 0 : -1;
+}
+#endif
