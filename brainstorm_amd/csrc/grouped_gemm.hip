@@ -84,18 +84,6 @@ __device__ __forceinline__ float apply_act(float v) {
   return v;
 }
 
-#ifdef BRT_GEMM_TRACE
-constexpr int kTraceSlots = 64, kTraceBlocks = 4096;
-__device__ unsigned long long g_trace[kTraceBlocks * kTraceSlots];
-#define TRACE(slot)                                                                   \
-  do {                                                                                \
-    if (threadIdx.x == 0 && blockIdx.x < kTraceBlocks && (slot) < kTraceSlots)        \
-      g_trace[blockIdx.x * kTraceSlots + (slot)] = wall_clock64();                    \
-  } while (0)
-#else
-#define TRACE(slot)
-#endif
-
 template <int N>
 struct Staged {
   u32x4 v[N];
@@ -118,7 +106,6 @@ __global__ __launch_bounds__(WAVES * 64) void grouped_gemm_kernel(GemmArgs a) {
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  TRACE(0);
 
   // ---- which tile: XCD-aware renumbering, then expert lookup from the loads ----------
   // hardware deals workgroups round-robin over the XCDs: workgroup b runs on XCD b % 8.
@@ -267,9 +254,7 @@ __global__ __launch_bounds__(WAVES * 64) void grouped_gemm_kernel(GemmArgs a) {
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int ks = 0; ks < kSteps; ++ks) {
-#ifndef DBG_NO_FETCH
       if constexpr (kFetch) fetch_slice(incoming, k_fetch, ks);
-#endif
       if (ks + 1 < kSteps) read_frags(ks + 1, (ks + 1) & 1);
 #pragma unroll
       for (int i = 0; i < MT; ++i)
@@ -277,9 +262,7 @@ __global__ __launch_bounds__(WAVES * 64) void grouped_gemm_kernel(GemmArgs a) {
         for (int j = 0; j < NT; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fw[ks & 1][j], fx[ks & 1][i],
                                                               acc[i][j], 0, 0, 0);
-#ifndef DBG_NO_STASH
       if constexpr (kStash) stash_slice(arrived, stage ^ 1, k_arrived, ks, last_tile);
-#endif
       // issue order of this k-step: one MFMA, then at most one op of each memory kind
       constexpr int kSlice = (LOADS + kSteps - 1) / kSteps;
       constexpr int kReads = MT + NT;
@@ -298,7 +281,6 @@ __global__ __launch_bounds__(WAVES * 64) void grouped_gemm_kernel(GemmArgs a) {
   // during step kt), tile kt+2 being loaded into the other ------------------------------
   const int k_tiles = (K + kBK - 1) / kBK;
   Staged<LOADS> s0, s1;
-  TRACE(1);
 #pragma unroll
   for (int p = 0; p < kSteps; ++p) fetch_slice(s0, 0, p);
   if (k_tiles > 1) {
@@ -308,17 +290,12 @@ __global__ __launch_bounds__(WAVES * 64) void grouped_gemm_kernel(GemmArgs a) {
 #pragma unroll
   for (int p = 0; p < kSteps; ++p) stash_slice(s0, 0, 0, p, Yes{});
   __syncthreads();
-  TRACE(2);
   int kt = 0;
   for (; kt + 3 < k_tiles; kt += 2) {
     step(0, s0, s1, (kt + 2) * kBK, (kt + 1) * kBK, Yes{}, Yes{}, No{});
-    TRACE(4 + 3 * kt);
     __syncthreads();
-    TRACE(6 + 3 * kt);
     step(1, s1, s0, (kt + 3) * kBK, (kt + 2) * kBK, Yes{}, Yes{}, No{});
-    TRACE(7 + 3 * kt);
     __syncthreads();
-    TRACE(9 + 3 * kt);
   }
   const int left = k_tiles - kt;  // 1, 2 or 3 tiles; kt is even, so the next tile is in stage 0
   if (left == 3) {
@@ -367,7 +344,6 @@ __global__ __launch_bounds__(WAVES * 64) void grouped_gemm_kernel(GemmArgs a) {
     }
   }
   __syncthreads();
-  TRACE(62);
   constexpr int OUT_CHUNKS = BN / 8;
   __bf16* __restrict__ oc = a.out + static_cast<size_t>(row0) * a.N + n0;
   for (int q = tid; q < rows * OUT_CHUNKS; q += THREADS) {
@@ -376,7 +352,6 @@ __global__ __launch_bounds__(WAVES * 64) void grouped_gemm_kernel(GemmArgs a) {
       *reinterpret_cast<u32x4*>(oc + static_cast<size_t>(r) * a.N + c * 8) =
           *reinterpret_cast<const u32x4*>(smem + r * OUT_ROW + c * 16);
   }
-  TRACE(63);
 }
 
 template <int MT, int NT, int WAVES, int ACT>
@@ -441,8 +416,3 @@ extern "C" int brt_hip_grouped_gemm(const void* x, const void* const* weights,
   return launch<5, 1, 4>(a, act, as_stream(stream));
 }
 
-#ifdef BRT_GEMM_TRACE
-extern "C" int brt_hip_debug_trace(void* host, size_t bytes) {
-  return hipMemcpyFromSymbol(host, HIP_SYMBOL(brt::g_trace), bytes) == hipSuccess ? 0 : -1;
-}
-#endif
