@@ -67,19 +67,25 @@ def _scan_workspace(device: torch.device, T: int, E: int) -> torch.Tensor:
 class _Pairing:
     """Remembers which (indices, loads) pair one index-generation call produced,
     together with the true per-path counts, so that dispatch can zero-fill the
-    padding rows itself instead of clearing the whole output first."""
+    padding rows itself instead of clearing the whole output first.  For routes
+    that send a cell to at most one path (``single_path``) it also keeps the
+    per-row tags the last dispatch wrote, which let combine run in scatter form."""
 
-    __slots__ = ("indices_ref", "indices_ptr", "indices_version", "loads_version", "counts")
+    __slots__ = ("indices_ref", "indices_ptr", "indices_version", "loads_version", "counts",
+                 "single_path", "row_tags", "row_tags_stride")
 
-    def __init__(self, indices, loads, counts):
+    def __init__(self, indices, loads, counts, single_path=False):
         self.indices_ref = weakref.ref(indices)
         self.indices_ptr = indices.data_ptr()
         self.indices_version = indices._version
         self.loads_version = loads._version
         self.counts = counts
+        self.single_path = single_path
+        self.row_tags = None        # [P] int32: 1-based cell of each dispatched row, 0 = padding
+        self.row_tags_stride = 0    # max_path_load the rows were laid out with (0 = packed)
 
 
-def _paired_counts(route_indices: torch.Tensor, loads: torch.Tensor) -> Optional[torch.Tensor]:
+def _pairing_of(route_indices: torch.Tensor, loads: torch.Tensor) -> Optional[_Pairing]:
     pairing = getattr(loads, "_brt_pairing", None)
     if (
         pairing is None
@@ -89,7 +95,12 @@ def _paired_counts(route_indices: torch.Tensor, loads: torch.Tensor) -> Optional
         or pairing.loads_version != loads._version
     ):
         return None
-    return pairing.counts
+    return pairing
+
+
+def _paired_counts(route_indices: torch.Tensor, loads: torch.Tensor) -> Optional[torch.Tensor]:
+    pairing = _pairing_of(route_indices, loads)
+    return None if pairing is None else pairing.counts
 
 
 # ------------------------------------------------------------------------- ops
@@ -122,8 +133,13 @@ def generate_indices_and_loads(
     capacity_padding: bool = False,
     path_wise_padding: bool = False,
     is_tag_index: bool = False,
+    *,
+    single_path: bool = False,
 ) -> Tuple[torch.Tensor, torch.Tensor]:
-    """router.cc:48-80."""
+    """router.cc:48-80.  ``single_path`` (keyword only, not in the reference) is the
+    caller's promise that no row of ``hot_mask`` has more than one nonzero; dispatch
+    and combine calls that receive the returned pair may then use the tag-driven
+    combine (same results, one memory round trip less)."""
     _check_on_device(hot_mask, "hot_mask")
     _check_int32(hot_mask, "hot_mask")
     T, E = hot_mask.size(0), hot_mask.size(1)
@@ -151,7 +167,7 @@ def generate_indices_and_loads(
             int(capacity_padding), int(path_wise_padding), int(is_tag_index),
             _ptr(ws), ws.numel(), _stream()))
         if not is_tag_index:
-            loads._brt_pairing = _Pairing(indices, loads, counts)
+            loads._brt_pairing = _Pairing(indices, loads, counts, bool(single_path))
     return indices, loads
 
 
@@ -234,7 +250,8 @@ def dispatch_with_indices_and_loads(
         if not is_1d_routing:
             cell //= E
 
-        counts = None if is_tag_index else _paired_counts(route_indices, loads)
+        pairing = None if is_tag_index else _pairing_of(route_indices, loads)
+        counts = None if pairing is None else pairing.counts
         _check_int32(loads, "loads")
         dev_loads = loads if loads.is_cuda else loads.to(device, non_blocking=True)
 
@@ -278,11 +295,17 @@ def dispatch_with_indices_and_loads(
                 old_tags = tags.contiguous()
             # old_tags None = arange(1, T+1) (router.cc:240-241), generated in the kernel
             new_tags = alloc((total,), dtype=route_indices.dtype, device=device)
+        hidden_tags = (pairing is not None and pairing.single_path and is_1d_routing
+                       and not tag_generating)
+        if hidden_tags and new_tags is None:
+            new_tags = torch.empty((total,), dtype=torch.int32, device=device)
 
         _lib.check(_lib.lib().brt_hip_dispatch(
             _ptr(in_data), _ptr(out), _ptr(dev_gates), _ptr(route_indices), _ptr(dev_loads),
             _ptr(counts), _ptr(old_tags), _ptr(new_tags), T, cell, E, total, mpl,
             int(is_1d_routing), int(is_tag_index), dtype, _stream()))
+        if hidden_tags:
+            pairing.row_tags, pairing.row_tags_stride = new_tags, mpl
     if tag_generating:
         return [out, new_tags]
     return [out]
@@ -418,6 +441,18 @@ def combine_with_indices_and_loads(
             residual = 0
         if result.dtype not in _DT or result.numel() != T * cell:
             raise RuntimeError("out_data does not match [cell_num, *cell_shape]")
+        # single-path routes whose rows still carry the tags of the paired dispatch:
+        # scatter form (identical rows; cells without a row keep the residual)
+        pairing = _pairing_of(route_indices, loads)
+        if (residual and dev_gates is None and pairing is not None and pairing.single_path
+                and pairing.row_tags is not None and pairing.row_tags.numel() == P
+                and pairing.row_tags_stride == mpl
+                and (cell * in_data.element_size()) % 16 == 0
+                and (result.dtype == in_data.dtype or result.dtype == torch.float32)):
+            _lib.check(_lib.lib().brt_hip_combine_by_tags(
+                _ptr(in_data), _ptr(result), _ptr(pairing.row_tags), P, cell, T,
+                _DT[in_data.dtype], _DT[result.dtype], _stream()))
+            return [result]
         _lib.check(_lib.lib().brt_hip_combine(
             _ptr(in_data), _ptr(result), _ptr(dev_gates), _ptr(route_indices), _ptr(dev_loads),
             T, cell, E, P, mpl, residual, _DT[in_data.dtype], _DT[result.dtype], gate_dtype,

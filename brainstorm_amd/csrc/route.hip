@@ -15,6 +15,8 @@
 #include <algorithm>
 #include <cstdlib>
 
+#include <type_traits>
+
 #include "common.hpp"
 
 namespace brt {
@@ -870,6 +872,10 @@ __global__ __launch_bounds__(kBlock, 8) void dispatch_lean_kernel(DispatchArgs a
           float g = 1.0f;
           if constexpr (DT >= 0)
             g = __int_as_float(__builtin_amdgcn_ds_bpermute(b << 2, __float_as_int(gate)));
+          if (a.new_tags != nullptr && has && glane == 0 && off0 == 0) {
+            const int tok = static_cast<int>(r0) + step * rps + i;
+            a.new_tags[d] = a.old_tags != nullptr ? a.old_tags[tok] : tok + 1;
+          }
 #pragma unroll
           for (int u = 0; u < UPR; ++u) {
             const int off = off0 + u * LPR + glane;
@@ -910,8 +916,10 @@ __global__ __launch_bounds__(kBlock, 8) void dispatch_lean_kernel(DispatchArgs a
       const int alloc = a.mpl != 0 ? a.mpl : read_lane(tab.my_load, pe);
       const long row = static_cast<long>(read_lane(tab.my_start, pe)) + (alloc - pad) +
                        (zi - (read_lane(z_incl, pe) - pad));
-      if (row < a.P)
+      if (row < a.P) {
         for (int o = lane; o < cpr; o += kWave) dst[static_cast<size_t>(row) * cpr + o] = zero_unit<16>();
+        if (a.new_tags != nullptr && lane == 0) a.new_tags[row] = 0;
+      }
     }
   }
 }
@@ -943,63 +951,193 @@ __global__ __launch_bounds__(kBlock) void combine_lean_kernel(CombineArgs a) {
   const U* __restrict__ src = static_cast<const U*>(a.src);
   char* __restrict__ dst = static_cast<char*>(a.dst);
 
-  int v_next = (sub < nt && e < E) ? idx0[sub * E + e] : 0;
+  auto load_idx = [&](int step) {
+    const int row = step * rps + sub;
+    return (step < n_steps && row < nt && e < E) ? idx0[row * E + e] : 0;
+  };
+  // index vectors are fetched two steps ahead of their use
+  int v_cur = load_idx(0), v_next = load_idx(1);
   const SmallTables tab = small_tables(a.loads, E, a.mpl, ep_shift, lane);
 
-  for (int step = 0; step < n_steps; ++step) {
-    const int v = v_next;
+  // per step (64 >> ep_shift tokens): source row and gate of (token sub, path e) in lane
+  // sub*ep + e, and the mask of routed (token, path) pairs
+  struct StepVec {
+    int src_row;
+    float gate;
+    unsigned long long m;
+    int tokens;
+    long t_first;
+  };
+  auto make_step = [&](int step, int v) {
+    StepVec s;
     const int row = step * rps + sub;
-    {
-      const int nrow = row + rps;
-      v_next = (step + 1 < n_steps && nrow < nt && e < E) ? idx0[nrow * E + e] : 0;
-    }
-    const int src_row = tab.start_e + v - 1;
-    const bool ok = row < nt && e < E && v >= 1 && v <= tab.load_e && src_row < a.P;
-    float gate = 1.0f;
+    s.src_row = tab.start_e + v - 1;
+    const bool ok = row < nt && e < E && v >= 1 && v <= tab.load_e && s.src_row < a.P;
+    s.gate = 1.0f;
     if (ok && a.gates != nullptr)
-      gate = load_gate(a.gates, a.gate_dtype, static_cast<size_t>(t0 + row) * E + e);
-    const unsigned long long m = __ballot(ok);
-    const int tokens = min(rps, nt - step * rps);
-    for (int tb = 0; tb < tokens; tb += GROUPS) {
-      const int i = tb + gidx;
-      const unsigned long long mine = i < tokens ? (m >> (i * ep)) & seg0 : 0ull;
-      const size_t to = static_cast<size_t>(t0 + step * rps + i) * cpr;
+      s.gate = load_gate(a.gates, a.gate_dtype, static_cast<size_t>(t0 + row) * E + e);
+    s.m = __ballot(ok);
+    s.tokens = min(rps, nt - step * rps);
+    s.t_first = t0 + step * rps;
+    return s;
+  };
+
+  // One item = GROUPS tokens (one per lane group) x one pass of LPR*UPR units.  Its first
+  // path's rows are loaded when the item is prepared and consumed one item later, so the
+  // loads of two consecutive items (tokens) are in flight together; further paths of a
+  // token (top-k > 1) are walked in ascending order when the item is consumed.
+  struct Item {
+    unsigned long long mine;
+    size_t to;
+    int i, off0, src_vec;  // i: token slot inside its step
+    float gate_vec, g;
+    bool live, has;
+    U val[UPR];
+  };
+  auto prepare = [&](const StepVec& s, int tb, int off0) {
+    Item it;
+    const int i = tb + gidx;
+    it.i = i;
+    it.live = i < s.tokens;
+    it.mine = it.live ? (s.m >> (i * ep)) & seg0 : 0ull;
+    it.has = it.mine != 0;
+    it.to = static_cast<size_t>(s.t_first + i) * cpr;
+    it.off0 = off0;
+    it.src_vec = s.src_row;
+    it.gate_vec = s.gate;
+    const int b = (i * ep + __builtin_ctzll(it.mine | (1ull << 63))) & (kWave - 1);
+    const int sr = __builtin_amdgcn_ds_bpermute(b << 2, s.src_row);
+    it.g = __int_as_float(__builtin_amdgcn_ds_bpermute(b << 2, __float_as_int(s.gate)));
+#pragma unroll
+    for (int u = 0; u < UPR; ++u) {
+      const int off = off0 + u * LPR + glane;
+      it.val[u] = U{};
+      if (it.has && off < cpr) it.val[u] = src[static_cast<size_t>(sr) * cpr + off];
+    }
+    return it;
+  };
+  auto consume = [&](const Item& it) {
+    float acc[UPR][NE];
+#pragma unroll
+    for (int u = 0; u < UPR; ++u) {
+      float x[NE];
+      unpack<IN_DT, 16>(it.val[u], x);
+      // one rounding for the product, one for the sum (no fused multiply-add); the sum
+      // starts from +0 like the sequential reference
+#pragma unroll
+      for (int q = 0; q < NE; ++q) acc[u][q] = it.has ? 0.0f + x[q] * it.g : 0.0f;
+    }
+    unsigned long long rem = it.mine & (it.mine - 1);
+    while (__ballot(rem != 0) != 0) {  // ascending path order: lowest set bit first
+      const bool has = rem != 0;
+      const int b = (it.i * ep + __builtin_ctzll(rem | (1ull << 63))) & (kWave - 1);
+      rem &= rem - 1;
+      const int sr = __builtin_amdgcn_ds_bpermute(b << 2, it.src_vec);
+      const float g = __int_as_float(__builtin_amdgcn_ds_bpermute(b << 2, __float_as_int(it.gate_vec)));
+      U val[UPR];
+#pragma unroll
+      for (int u = 0; u < UPR; ++u) {
+        const int off = it.off0 + u * LPR + glane;
+        if (has && off < cpr) val[u] = src[static_cast<size_t>(sr) * cpr + off];
+      }
+#pragma unroll
+      for (int u = 0; u < UPR; ++u) {
+        const int off = it.off0 + u * LPR + glane;
+        if (has && off < cpr) {
+          float x[NE];
+          unpack<IN_DT, 16>(val[u], x);
+#pragma unroll
+          for (int q = 0; q < NE; ++q) acc[u][q] = acc[u][q] + x[q] * g;
+        }
+      }
+    }
+    if (it.live && (it.mine != 0 || !a.is_residual)) {
+#pragma unroll
+      for (int u = 0; u < UPR; ++u) {
+        const int off = it.off0 + u * LPR + glane;
+        if (off < cpr) pack_store<OUT_DT, NE>(dst + (it.to + off) * OUT_BYTES, acc[u]);
+      }
+    }
+  };
+
+  Item pend;
+  pend.mine = 0; pend.to = 0; pend.i = 0; pend.off0 = 0; pend.src_vec = 0; pend.gate_vec = 0.0f; pend.g = 0.0f;
+  pend.live = false; pend.has = false;
+#pragma unroll
+  for (int u = 0; u < UPR; ++u) pend.val[u] = U{};
+
+  StepVec cur = make_step(0, v_cur);
+  for (int step = 0; step < n_steps; ++step) {
+    StepVec nxt = cur;
+    if (step + 1 < n_steps) {
+      nxt = make_step(step + 1, v_next);
+      v_next = load_idx(step + 2);
+    }
+    for (int tb = 0; tb < cur.tokens; tb += GROUPS) {
       for (int off0 = 0; off0 < cpr; off0 += LPR * UPR) {
-        float acc[UPR][NE];
+        const Item fresh = prepare(cur, tb, off0);
+        consume(pend);
+        pend = fresh;
+      }
+    }
+    cur = nxt;
+  }
+  consume(pend);
+}
+
+// Combine in scatter form for routes where no cell owns more than one row (top-1):
+// every source row carries the 1-based tag of the cell it came from (the new_tags
+// output of dispatch; 0 marks a padding row), so a row's data and its tag are fetched
+// together and the row is stored to dst[tag-1] -- one memory round trip less than the
+// gather form, which must read a cell's index words before it knows which row to load.
+// Cells without a row are left untouched.
+struct CombineRowsArgs {
+  const void* src;
+  void* dst;
+  const int* row_tags;
+  int T, P, cpr, rows_pw;
+};
+
+template <int IN_DT, int OUT_DT, int LS, int UPR>
+__global__ __launch_bounds__(kBlock) void combine_rows_kernel(CombineRowsArgs a) {
+  using U = u32x4;
+  constexpr int NE = 16 / elem_bytes(IN_DT);
+  constexpr int OUT_BYTES = NE * elem_bytes(OUT_DT);
+  constexpr int LPR = 1 << LS;
+  constexpr int GROUPS = kWave >> LS;
+  const int lane = threadIdx.x & (kWave - 1);
+  const long wave = static_cast<long>(blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  const int gidx = lane >> LS, glane = lane & (LPR - 1);
+  const long p0 = wave * a.rows_pw;
+  const int np = static_cast<int>(max(0l, min(static_cast<long>(a.rows_pw), a.P - p0)));
+  const int cpr = a.cpr;
+  const U* __restrict__ src = static_cast<const U*>(a.src);
+  char* __restrict__ dst = static_cast<char*>(a.dst);
+  for (int rb = 0; rb < np; rb += GROUPS) {
+    const int i = rb + gidx;
+    const bool live = i < np;
+    const int tag = live ? a.row_tags[p0 + i] : 0;
+    const size_t from = static_cast<size_t>(p0 + i) * cpr;
+    for (int off0 = 0; off0 < cpr; off0 += LPR * UPR) {
+      U val[UPR];
 #pragma unroll
-        for (int u = 0; u < UPR; ++u)
+      for (int u = 0; u < UPR; ++u) {
+        const int off = off0 + u * LPR + glane;
+        if (live && off < cpr) val[u] = src[from + off];
+      }
+      if (tag >= 1 && tag <= a.T) {
+        const size_t to = static_cast<size_t>(tag - 1) * cpr;
 #pragma unroll
-          for (int q = 0; q < NE; ++q) acc[u][q] = 0.0f;
-        unsigned long long rem = mine;
-        while (__ballot(rem != 0) != 0) {  // ascending path order: lowest set bit first
-          const bool has = rem != 0;
-          const int b = i * ep + __builtin_ctzll(rem | (1ull << 63));
-          rem &= rem - 1;
-          const int sr = __builtin_amdgcn_ds_bpermute(b << 2, src_row);
-          const float g = __int_as_float(__builtin_amdgcn_ds_bpermute(b << 2, __float_as_int(gate)));
-          U val[UPR];
-#pragma unroll
-          for (int u = 0; u < UPR; ++u) {
-            const int off = off0 + u * LPR + glane;
-            if (has && off < cpr) val[u] = src[static_cast<size_t>(sr) * cpr + off];
-          }
-#pragma unroll
-          for (int u = 0; u < UPR; ++u) {
-            const int off = off0 + u * LPR + glane;
-            if (has && off < cpr) {
+        for (int u = 0; u < UPR; ++u) {
+          const int off = off0 + u * LPR + glane;
+          if (off < cpr) {
+            if constexpr (IN_DT == OUT_DT) {
+              *reinterpret_cast<U*>(dst + (to + off) * 16) = val[u];
+            } else {
               float x[NE];
               unpack<IN_DT, 16>(val[u], x);
-              // one rounding for the product, one for the sum (no fused multiply-add)
-#pragma unroll
-              for (int q = 0; q < NE; ++q) acc[u][q] = acc[u][q] + x[q] * g;
+              pack_store<OUT_DT, NE>(dst + (to + off) * OUT_BYTES, x);
             }
-          }
-        }
-        if (i < tokens && (mine != 0 || !a.is_residual)) {
-#pragma unroll
-          for (int u = 0; u < UPR; ++u) {
-            const int off = off0 + u * LPR + glane;
-            if (off < cpr) pack_store<OUT_DT, NE>(dst + (to + off) * OUT_BYTES, acc[u]);
           }
         }
       }
@@ -1082,8 +1220,7 @@ template <int BYTES, int DT>
 void launch_dispatch(const DispatchArgs& a, const LaunchShape& sh, hipStream_t st) {
   const dim3 grid(sh.grid), block(sh.waves_pb * kWave);
   if constexpr (BYTES == 16) {
-    if (a.E <= kWave && a.is_1d && !a.is_tag_index && a.new_tags == nullptr &&
-        env_int("BRT_NO_LEAN", 0) == 0) {
+    if (a.E <= kWave && a.is_1d && !a.is_tag_index && env_int("BRT_NO_LEAN", 0) == 0) {
 #define BRT_LAUNCH(LS, UPR) \
   hipLaunchKernelGGL((dispatch_lean_kernel<DT, LS, UPR>), grid, block, 0, st, a);
       BRT_LEAN_SHAPES(BRT_LAUNCH)
@@ -1235,4 +1372,51 @@ extern "C" int brt_hip_combine(const void* src, void* dst, const void* gates,
 #undef BRT_COMBINE_CASE
 #undef BRT_COMBINE_HALF
   return check_launch("combine_kernel");
+}
+
+extern "C" int brt_hip_combine_by_tags(const void* src, void* dst, const int32_t* row_tags, int P,
+                                       int cell, int T, int in_dtype, int out_dtype, void* stream) {
+  if (T < 0 || cell < 0 || P < 0) return fail(BRT_E_INVALID, "bad shape T=%d cell=%d P=%d", T, cell, P);
+  if ((in_dtype != BRT_F32 && in_dtype != BRT_F16 && in_dtype != BRT_BF16) ||
+      (out_dtype != in_dtype && out_dtype != BRT_F32))
+    return fail(BRT_E_UNSUPPORTED, "dtype pair %d -> %d is not supported", in_dtype, out_dtype);
+  if (P == 0 || cell == 0 || T == 0) return BRT_OK;
+  if (!src || !dst || !row_tags) return fail(BRT_E_INVALID, "null argument");
+  const size_t row_bytes = static_cast<size_t>(cell) * elem_bytes(in_dtype);
+  if (row_bytes % 16 != 0 || !aligned(src, 16) || !aligned(dst, 16))
+    return fail(BRT_E_UNSUPPORTED, "rows must be whole 16-byte units (row is %zu bytes)", row_bytes);
+  CombineRowsArgs a{};
+  a.src = src; a.dst = dst; a.row_tags = row_tags; a.T = T; a.P = P;
+  a.cpr = static_cast<int>(row_bytes / 16);
+  int rows = env_int("BRT_COMBINE_ROWS", 0);
+  if (rows <= 0) {
+    rows = std::max(1, 384 / a.cpr);
+    while (rows > 1 && (P + rows - 1) / rows < 4096) rows >>= 1;
+  }
+  a.rows_pw = rows;
+  const long n_waves = (static_cast<long>(P) + rows - 1) / rows;
+  const int waves_pb = kBlock / kWave;
+  const dim3 grid(static_cast<unsigned>((n_waves + waves_pb - 1) / waves_pb)), block(kBlock);
+  hipStream_t st = as_stream(stream);
+#define BRT_ROWS_LAUNCH(IN, OUT)                                                          \
+  {                                                                                       \
+    auto launch = [&](auto ls, auto upr) {                                                \
+      hipLaunchKernelGGL((combine_rows_kernel<IN, OUT, decltype(ls)::value, decltype(upr)::value>), \
+                         grid, block, 0, st, a);                                          \
+    };                                                                                    \
+    using std::integral_constant;                                                         \
+    if (a.cpr > 2 * kWave) launch(integral_constant<int, 6>{}, integral_constant<int, 4>{});        \
+    else if (a.cpr > kWave) launch(integral_constant<int, 6>{}, integral_constant<int, 2>{});       \
+    else if (a.cpr > 32) launch(integral_constant<int, 6>{}, integral_constant<int, 1>{});          \
+    else if (a.cpr > 16) launch(integral_constant<int, 5>{}, integral_constant<int, 1>{});          \
+    else if (a.cpr > 8) launch(integral_constant<int, 4>{}, integral_constant<int, 1>{});           \
+    else launch(integral_constant<int, 3>{}, integral_constant<int, 1>{});                          \
+  }
+  if (in_dtype == BRT_F32) BRT_ROWS_LAUNCH(BRT_F32, BRT_F32)
+  else if (in_dtype == BRT_F16 && out_dtype == BRT_F16) BRT_ROWS_LAUNCH(BRT_F16, BRT_F16)
+  else if (in_dtype == BRT_F16) BRT_ROWS_LAUNCH(BRT_F16, BRT_F32)
+  else if (out_dtype == BRT_BF16) BRT_ROWS_LAUNCH(BRT_BF16, BRT_BF16)
+  else BRT_ROWS_LAUNCH(BRT_BF16, BRT_F32)
+#undef BRT_ROWS_LAUNCH
+  return check_launch("combine_rows_kernel");
 }

@@ -224,7 +224,8 @@ class DispatchFabric(FabricBase):
         caps = runtime_capacities if runtime_capacities is not None else self.supported_capacities
         route_indices, loads = c_router.generate_indices_and_loads(
             hot_mask, supported_capacities=caps, capacity_padding=self.capacity_padding,
-            path_wise_padding=self.path_wise_padding, is_tag_index=False)
+            path_wise_padding=self.path_wise_padding, is_tag_index=False,
+            single_path=getattr(hot_mask, "_brt_single_path", False))
         in_flows = [in_flow] if self.flow_num == 1 else in_flow
         self.capture_flow_stats(in_flows, route_indices, loads)
         all_out_flows, score = self.dispatch(in_flows, route_indices, loads, score)

@@ -23,10 +23,17 @@ class ProtocolBase(nn.Module):
         super().__init__()
         self.debug = os.environ.get("BRT_DEBUG", "False").lower() in ("true", "1")
 
+    #: True when the protocol never routes a cell to more than one path; the hot mask is
+    #: then marked so that the fabrics can use the tag-driven combine
+    single_path = False
+
     def forward(self, score: torch.Tensor, *args, **kwargs):
         decisions = self.make_route_decision(score, *args, **kwargs)
         if self.debug:
             self.check_decision(decisions, score)
+        if self.single_path:
+            hot_mask = decisions[0] if isinstance(decisions, (tuple, list)) else decisions
+            hot_mask._brt_single_path = True
         return decisions
 
     def make_route_decision(self, score, **kwargs):
@@ -64,6 +71,7 @@ class TopKProtocol(ProtocolBase):
     def __init__(self, top_k=1):
         super().__init__()
         self.top_k = top_k
+        self.single_path = top_k == 1
 
     def make_route_decision(self, score):
         return _one_hot_int32(torch.topk(score, self.top_k, dim=1).indices, score)
@@ -72,6 +80,8 @@ class TopKProtocol(ProtocolBase):
 @register_protocol("switch_top1")
 class SwitchTop1Protocol(ProtocolBase):
     """protocol/switch.py:13-33: the score already is the (capacity-masked) one-hot."""
+
+    single_path = True
 
     def make_route_decision(self, score):
         return score.reshape(-1, score.shape[-1]).to(torch.int32, non_blocking=True)

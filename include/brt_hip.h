@@ -146,6 +146,25 @@ int brt_hip_combine(const void* src, void* dst, const void* gates, const int32_t
                     int is_residual, int in_dtype, int out_dtype, int gate_dtype, void* stream);
 
 /*
+ * Combine for routes in which no cell owns more than one row (top-1 protocols),
+ * driven by the per-row tags that dispatch generates (new_tags above; the
+ * reference produces them with tag_generating=true, router.cc:235-250, and carries
+ * them on the tag stack of the routed tensor).  Gives exactly the rows that
+ * brt_hip_combine(..., gates=NULL, is_residual=1) gives for such a route, with
+ * one memory round trip less: a row and its tag are fetched together, nothing has
+ * to be looked up in the [T,E] index matrix first.
+ *
+ *   src       [P, cell] in in_dtype
+ *   dst       [T, cell] in out_dtype (= in_dtype, or BRT_F32); rows of cells that
+ *             own no row are left untouched
+ *   row_tags  [P]: 1-based cell of row p, 0 for a padding row; tags > T are ignored
+ *   Rows must be whole 16-byte units (BRT_E_UNSUPPORTED otherwise: use brt_hip_combine).
+ *   If two rows carry the same tag the result is unspecified (one of them wins).
+ */
+int brt_hip_combine_by_tags(const void* src, void* dst, const int32_t* row_tags, int P, int cell,
+                            int T, int in_dtype, int out_dtype, void* stream);
+
+/*
  * Replaces the homo-fused expert kernel launch jit::CUDACompiler::HomoExecute
  * (src/jit/compiler.cu:151-246, binding src/backend/torch/jit.cc:54-75) for
  * Linear branches (python/brt/jit/modules/linear.py:15-61):

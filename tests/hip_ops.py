@@ -159,3 +159,19 @@ def combine(y_bits, idx, loads, gates_bits=None, residual_bits=None, max_path_lo
         int(residual_bits is not None), DT[in_dtype], DT[out_dtype], DT[gate_dtype], stream()))
     torch.cuda.synchronize()
     return host(d_out, True)
+
+
+def combine_by_tags(y_bits, row_tags, residual_bits, in_dtype="f32", out_dtype=None):
+    out_dtype = out_dtype or in_dtype
+    y_bits = np.ascontiguousarray(y_bits)
+    P = y_bits.shape[0]
+    cell = y_bits.size // max(P, 1)
+    residual_bits = np.ascontiguousarray(residual_bits)
+    T = residual_bits.shape[0]
+    d_y = dev(y_bits.reshape(P, -1))
+    d_out = dev(residual_bits.reshape(T, -1)).clone()
+    d_tags = dev(np.asarray(row_tags, dtype=np.int32))
+    _lib.check(_lib.lib().brt_hip_combine_by_tags(
+        ptr(d_y), ptr(d_out), ptr(d_tags), P, cell, T, DT[in_dtype], DT[out_dtype], stream()))
+    torch.cuda.synchronize()
+    return host(d_out, True)

@@ -274,6 +274,56 @@ def test_combine_max_path_padding_and_odd_rows(hip):
             assert same_bits(got, want)
 
 
+# ------------------------------------------------- tag-driven combine (single-path routes)
+@pytest.mark.parametrize("T,E,cell,in_dtype,out_dtype", [
+    (1024, 16, 512, "f32", "f32"),
+    (8192, 64, 768, "bf16", "bf16"),      # the Switch layer shape
+    (8192, 64, 768, "bf16", "f32"),
+    (3000, 8, 96, "f16", "f16"),          # 192-byte rows, several rows per wavefront step
+    (777, 5, 8, "f16", "f32"),            # one 16-byte unit per row
+    (513, 64, 1100, "f32", "f32"),        # rows wider than one pass of a wavefront
+])
+@pytest.mark.parametrize("layout", ["clip", "capacity_padding", "max_path_padding"])
+def test_combine_by_tags_equals_gather_combine(hip, T, E, cell, in_dtype, out_dtype, layout):
+    mask, _ = topk_mask(T, E, 1, seed=T + cell)
+    rng = np.random.default_rng(T + cell + 3)
+    cap = max(1, int(0.9 * T / E))        # some cells are dropped
+    pad = layout == "capacity_padding"
+    idx, loads, counts = hip.generate_indices_and_loads(mask, [cap], pad, want_counts=True)
+    want_idx, want_loads = oracle.generate_indices_and_loads(mask, [cap], capacity_padding=pad)
+    assert np.array_equal(idx, want_idx) and np.array_equal(loads, want_loads)
+    mpl = int(loads.max()) + 3 if layout == "max_path_padding" else 0
+    x = as_dtype_bits(rng.standard_normal((T, cell)), in_dtype)
+    # tags come from the dispatch kernel itself, with and without the zero-fill contract
+    y, tags = hip.dispatch(x, idx, loads, counts=counts, tag_generating=True, max_path_load=mpl,
+                           dtype=in_dtype)
+    y0, tags0 = hip.dispatch(x, idx, loads, tag_generating=True, max_path_load=mpl, dtype=in_dtype)
+    want_y, want_tags = oracle.dispatch(x, idx, loads, tag_generating=True,
+                                        max_path_padding=mpl != 0, max_path_load=mpl, dtype=in_dtype)
+    assert same_bits(y, want_y) and same_bits(y0, want_y)
+    assert np.array_equal(tags, want_tags) and np.array_equal(tags0, want_tags)
+    expert_out = as_dtype_bits(rng.standard_normal(y.shape), in_dtype)
+    res = as_dtype_bits(rng.standard_normal((T, cell)), out_dtype)
+    want = oracle.combine(expert_out, idx, loads, out_data=res, max_path_padding=mpl != 0,
+                          in_dtype=in_dtype, out_dtype=out_dtype)
+    got = hip.combine_by_tags(expert_out, tags, res, in_dtype=in_dtype, out_dtype=out_dtype)
+    assert same_bits(got, want)
+    assert same_bits(got, hip.combine(expert_out, idx, loads, None, res, max_path_load=mpl,
+                                      in_dtype=in_dtype, out_dtype=out_dtype))
+
+
+def test_combine_by_tags_rejects_rows_that_are_not_16_byte_units(hip):
+    y = np.zeros((4, 3), dtype=np.float32)
+    with pytest.raises(NotImplementedError):
+        hip.combine_by_tags(y, [1, 2, 0, 3], np.zeros((3, 3), dtype=np.float32))
+    # out-of-range tags are ignored, empty inputs are fine
+    y = np.arange(32, dtype=np.float32).reshape(4, 8)
+    got = hip.combine_by_tags(y, [2, 0, 99, -5], np.full((3, 8), 7.0, dtype=np.float32))
+    want = np.full((3, 8), 7.0, dtype=np.float32)
+    want[1] = y[0]
+    assert np.array_equal(got, want)
+
+
 # ------------------------------------------------- full-size configurations
 def _route(hip, mask, caps=None, pad=False):
     idx, loads, counts = hip.generate_indices_and_loads(mask, caps, pad, want_counts=True)

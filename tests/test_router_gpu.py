@@ -163,6 +163,10 @@ def test_fused_moe_path_matches_oracle(brt_mod):
     xb = x.view(torch.int16).cpu().numpy().view(np.uint16)
     o_y, _ = oracle.dispatch(xb, o_idx, o_loads, dtype="bf16")
     assert np.array_equal(brt.to_torch_tensor(routed).view(torch.int16).cpu().numpy().view(np.uint16), o_y)
+    # a single-path protocol: dispatch left the per-row tags for the tag-driven combine
+    tags = loads._brt_pairing.row_tags
+    assert tags is not None and np.array_equal(
+        tags.cpu().numpy(), oracle.dispatch(xb, o_idx, o_loads, tag_generating=True, dtype="bf16")[1])
     expert_out = routed * 2  # stacks travel through the expert
     residual = x.clone()
     out = gather(expert_out, residual)
@@ -170,6 +174,38 @@ def test_fused_moe_path_matches_oracle(brt_mod):
     o_out = oracle.combine(brt.to_torch_tensor(expert_out).view(torch.int16).cpu().numpy().view(np.uint16),
                            o_idx, o_loads, out_data=xb, in_dtype="bf16")
     assert np.array_equal(out.view(torch.int16).cpu().numpy().view(np.uint16), o_out)
+
+
+def test_fused_moe_path_top2_keeps_the_gather_combine(brt_mod):
+    """top-2: a cell owns two rows, so no tags are kept and combine sums in path order."""
+    brt, c_router, ScatterRouter, GatherRouter = brt_mod
+    T, E, d = 1000, 8, 128
+    _, logits = topk_mask(T, E, 2, seed=15)
+    score = torch.from_numpy(softmax(logits).astype(np.float32)).cuda()
+    x = torch.from_numpy(np.random.default_rng(15).standard_normal((T, d)).astype(np.float32)).cuda()
+    scatter = ScatterRouter(protocol_type="topk", fabric_type="fused_dispatch",
+                            protocol_kwargs={"top_k": 2}).cuda()
+    gather = GatherRouter(fabric_type="fused_combine").cuda()
+    routed = scatter(brt.Annotator([0])(x), score)
+    idx, loads = routed.tag, routed.load
+    assert loads._brt_pairing.row_tags is None
+    residual = torch.zeros_like(x)
+    out = gather(routed * 1.0, residual)
+    o_mask = (idx.cpu().numpy() > 0).astype(np.int32)
+    o_idx, o_loads = oracle.generate_indices_and_loads(o_mask)
+    o_y, _ = oracle.dispatch(x.cpu().numpy(), o_idx, o_loads)
+    o_out = oracle.combine(o_y, o_idx, o_loads, out_data=np.zeros((T, d), dtype=np.float32))
+    assert np.array_equal(out.cpu().numpy(), o_out)
+    # same routers with top_k=1 take the tag-driven path and agree with the oracle too
+    scatter1 = ScatterRouter(protocol_type="topk", fabric_type="fused_dispatch").cuda()
+    routed1 = scatter1(brt.Annotator([0])(x), score)
+    assert routed1.load._brt_pairing.row_tags is not None
+    res1 = torch.full_like(x, 3.0)
+    i1, l1 = routed1.tag.cpu().numpy(), routed1.load.cpu().numpy()
+    out1 = gather(routed1 * 1.0, res1)
+    o_y1, _ = oracle.dispatch(x.cpu().numpy(), i1, l1)
+    assert np.array_equal(out1.cpu().numpy(),
+                          oracle.combine(o_y1, i1, l1, out_data=np.full((T, d), 3.0, dtype=np.float32)))
 
 
 def test_shim_signatures_and_errors(brt_mod):
