@@ -11,6 +11,10 @@ weights; seeded synthetic data, everything resident in HBM before timing.
 A step is one pass of the hot path over the batch, called through the C ABI of
 libbrt_hip.so and replayed as one HIP graph:
     index/load generation -> dispatch -> grouped FFN (two launches) -> combine.
+The route is top-1, so the step takes the path the routers take for single-path
+protocols: dispatch also writes the per-row tags and combine is the tag-driven
+scatter form (brt_hip_combine_by_tags); the index-driven gather form
+(brt_hip_combine) is timed beside it as `combine_gather`.
 `value` is the headline metric: algorithmic bytes of dispatch + combine divided
 by the sum of their kernel times.  Kernel times are measured in this process
 with HIP events around graphs of back-to-back launches of the one kernel, on the
@@ -36,7 +40,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # a 12 MiB device-to-device copy (fetch x1.996, write x1.000).
 MEASURED_TRAFFIC_BYTES = {
     "dispatch": int((7203.0 * 1.996 + 12288.0) * 1024),
-    "combine": int((7197.0 * 1.996 + 12288.0) * 1024),
+    "combine": None,
 }
 
 T, D, E, DFF = 8192, 768, 64, 3072
@@ -104,7 +108,9 @@ def main():
     P = int(loads_h.sum())                               # rows of the dispatched buffer
     R = int(torch.minimum(loads_h, counts_h).sum())      # rows actually routed
     y = torch.empty(P, D, dtype=torch.bfloat16, device=dev)
+    row_tags = torch.empty(P, dtype=torch.int32, device=dev)
     out = x.clone()                                      # residual: unrouted tokens keep x
+    out_gather = x.clone()
 
     wi = wi_h.to(dev)
     wo = wo_h.to(dev)
@@ -116,7 +122,7 @@ def main():
     def k_dispatch():
         _lib.check(L.brt_hip_dispatch(
             x.data_ptr(), y.data_ptr(), None, idx.data_ptr(), loads.data_ptr(), counts.data_ptr(),
-            None, None, T, D, E, P, 0, 1, 0, _lib.BF16, sptr()))
+            None, row_tags.data_ptr(), T, D, E, P, 0, 1, 0, _lib.BF16, sptr()))
 
     def k_gemm1():
         _lib.check(L.brt_hip_grouped_gemm(
@@ -141,9 +147,14 @@ def main():
     combine_src = y2 if have_ffn else y
 
     def k_combine():
+        _lib.check(L.brt_hip_combine_by_tags(
+            combine_src.data_ptr(), out.data_ptr(), row_tags.data_ptr(), P, D, T,
+            _lib.BF16, _lib.BF16, sptr()))
+
+    def k_combine_gather():
         _lib.check(L.brt_hip_combine(
-            combine_src.data_ptr(), out.data_ptr(), None, idx.data_ptr(), loads.data_ptr(), T, D,
-            E, P, 0, 1, _lib.BF16, _lib.BF16, _lib.F32, sptr()))
+            combine_src.data_ptr(), out_gather.data_ptr(), None, idx.data_ptr(), loads.data_ptr(),
+            T, D, E, P, 0, 1, _lib.BF16, _lib.BF16, _lib.F32, sptr()))
 
     def step():
         k_indexgen()
@@ -174,6 +185,14 @@ def main():
         stream.synchronize()
         return a.elapsed_time(b)  # ms
 
+    # both combine forms must agree bit for bit on this route before anything is timed
+    with torch.cuda.stream(stream):
+        step()
+        k_combine_gather()
+    stream.synchronize()
+    if not torch.equal(out.view(torch.int16), out_gather.view(torch.int16)):
+        sys.exit("bench.py: tag-driven and index-driven combine disagree")
+
     # ------------------------------------------------------- timed region: K steps
     g_step = capture(step)
     with torch.cuda.stream(stream):
@@ -189,7 +208,8 @@ def main():
 
     # ---------------------------------------- per-kernel durations (same process)
     INNER = 20
-    kernels = {"indexgen": k_indexgen, "dispatch": k_dispatch, "combine": k_combine}
+    kernels = {"indexgen": k_indexgen, "dispatch": k_dispatch, "combine": k_combine,
+               "combine_gather": k_combine_gather}
     if have_ffn:
         kernels.update({"ffn_gemm1_gelu": k_gemm1, "ffn_gemm2": k_gemm2})
     replays = max(10, args.steps // 4)
@@ -206,6 +226,13 @@ def main():
         "indexgen": 2 * idx_bytes + 4 * E,
         "dispatch": R * D * es + P * D * es + idx_bytes,
         "combine": R * D * es + T * D * es + idx_bytes,
+        "combine_gather": R * D * es + T * D * es + idx_bytes,
+    }
+    # what the kernels have to touch: the tag-driven combine reads 4 bytes of tag per row
+    # instead of the [T,E] index matrix, dispatch writes those tags
+    moved = {
+        "dispatch": bytes_["dispatch"] + 4 * P,
+        "combine": 2 * R * D * es + 4 * P,
     }
     flops = {"ffn_gemm1_gelu": 2.0 * R * D * DFF, "ffn_gemm2": 2.0 * R * DFF * D}
     dc_bytes = bytes_["dispatch"] + bytes_["combine"]
@@ -223,6 +250,7 @@ def main():
         "traffic": MEASURED_TRAFFIC_BYTES.get(dominant),
         "avg_us": round(us[dominant], 3),
         "algorithmic_bytes": bytes_[dominant],
+        "bytes_the_kernel_must_move": moved[dominant],
     }
     per_kernel = {}
     for name in us:

@@ -858,6 +858,10 @@ __global__ __launch_bounds__(kBlock, 8) void dispatch_lean_kernel(DispatchArgs a
       if (ok) gate = load_gate(a.gates, DT, static_cast<size_t>(r0 + row) * E + e);
     }
     const unsigned long long m = __ballot(ok);
+    if (a.new_tags != nullptr && ok) {  // the lane that holds (token, path) tags the row
+      const int tok = static_cast<int>(r0) + row;
+      a.new_tags[dst_row] = a.old_tags != nullptr ? a.old_tags[tok] : tok + 1;
+    }
     for (int tb = 0; tb < tokens; tb += GROUPS) {
       const int i = tb + gidx;  // token of this lane group
       const unsigned long long mine = i < tokens ? (m >> (i * ep)) & seg0 : 0ull;
@@ -872,10 +876,6 @@ __global__ __launch_bounds__(kBlock, 8) void dispatch_lean_kernel(DispatchArgs a
           float g = 1.0f;
           if constexpr (DT >= 0)
             g = __int_as_float(__builtin_amdgcn_ds_bpermute(b << 2, __float_as_int(gate)));
-          if (a.new_tags != nullptr && has && glane == 0 && off0 == 0) {
-            const int tok = static_cast<int>(r0) + step * rps + i;
-            a.new_tags[d] = a.old_tags != nullptr ? a.old_tags[tok] : tok + 1;
-          }
 #pragma unroll
           for (int u = 0; u < UPR; ++u) {
             const int off = off0 + u * LPR + glane;
