@@ -39,8 +39,11 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # FETCH_SIZE and WRITE_SIZE (KiB), each scaled by what the same counter reads for
 # a 12 MiB device-to-device copy (fetch x1.996, write x1.000).
 MEASURED_TRAFFIC_BYTES = {
-    "dispatch": int((7203.0 * 1.996 + 12288.0) * 1024),
-    "combine": None,
+    "dispatch": int((7207.5 * 1.996 + 12482.4) * 1024),
+    "combine": int((6221.5 * 1.996 + 12288.0) * 1024),
+    "combine_gather": int((7210.0 * 1.996 + 12288.0) * 1024),
+    "ffn_gemm1_gelu": int((155525.2 * 1.996 + 49152.0) * 1024),
+    "ffn_gemm2": int((177207.9 * 1.996 + 12288.0) * 1024),
 }
 
 T, D, E, DFF = 8192, 768, 64, 3072
@@ -261,6 +264,10 @@ def main():
         if name in flops:
             entry["TFLOPs"] = round(flops[name] / us[name] / 1e6, 1)
             entry["mfma_frac"] = round(flops[name] / us[name] / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4)
+            # the expert FFN at 128 rows per expert streams its weights: HBM is the bound
+            hbm = MEASURED_TRAFFIC_BYTES[name]
+            entry["hbm_GBps"] = round(hbm / us[name] / 1e3, 1)
+            entry["hbm_frac"] = round(hbm / us[name] / 1e3 / HBM_PEAK_GBPS, 4)
         per_kernel[name] = entry
 
     # ------------------------------------------------------------ CPU baseline
