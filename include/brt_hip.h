@@ -177,7 +177,8 @@ int brt_hip_combine_by_tags(const void* src, void* dst, const int32_t* row_tags,
  *   device array of E pointers to b_e [N] bf16, or NULL; `loads` [E] int32 is
  *   read on the device (no host copy, any non-negative values, sum <= P).
  *   One launch covers all experts; accumulation is fp32 on the bf16 MFMA units.
- *   K must be a multiple of 32 and N a multiple of 16.
+ *   K and N must be multiples of 8 (16-byte rows; BRT_E_UNSUPPORTED otherwise), x and out
+ *   16-byte aligned.  `act` is one of BRT_ACT_*; GELU is the erf form.
  */
 int brt_hip_grouped_gemm(const void* x, const void* const* weights, const void* const* biases,
                          void* out, const int32_t* loads, int E, int P, int K, int N, int act,
