@@ -96,3 +96,14 @@ def test_full_size_switch_ffn():
     loads = np.minimum(rng.multinomial(8192, [1 / 64] * 64), 160).tolist()
     run(loads, 768, 3072, act="gelu")
     run(loads, 3072, 768)
+
+
+def test_ragged_dirichlet_loads_task_moe_shape():
+    # BASELINE configs[4] at reduced size: loads ~ Dirichlet(0.3) (many empty experts, a few
+    # with hundreds of rows), one launch over the ragged batches, both FFN shapes
+    rng = np.random.default_rng(4)
+    E, rows = 48, 4096
+    loads = rng.multinomial(rows, rng.dirichlet(np.full(E, 0.3))).tolist()
+    assert min(loads) == 0 and max(loads) > 320
+    run(loads, 512, 2048, act="gelu", bias=True)
+    run(loads, 2048, 512, slack=3)
