@@ -209,6 +209,36 @@ def main():
     wall_ms = (time.perf_counter() - t0) * 1e3
     ms_per_step = ms_total / args.steps
 
+    # ------------- kernel durations inside the step (cold inputs, real neighbours): the same step
+    # launched eagerly with an event after every launch.  The two GEMMs keep the GPU busy long
+    # enough for the host to stay ahead, so the intervals are kernel time, not launch time.
+    order = [("indexgen", k_indexgen), ("dispatch", k_dispatch)]
+    if have_ffn:
+        order += [("ffn_gemm1_gelu", k_gemm1), ("ffn_gemm2", k_gemm2)]
+    order.append(("combine", k_combine))
+    n_eager = max(20, min(args.steps, 100))
+    marks = [[torch.cuda.Event(enable_timing=True) for _ in range(len(order) + 1)]
+             for _ in range(n_eager)]
+    with torch.cuda.stream(stream):
+        for _ in range(3):
+            step()
+        for ev in marks:
+            ev[0].record(stream)
+            for j, (_, fn) in enumerate(order):
+                fn()
+                ev[j + 1].record(stream)
+        blank = [torch.cuda.Event(enable_timing=True) for _ in range(64)]
+        k_gemm2() if have_ffn else k_dispatch()       # something to queue behind
+        for ev in blank:
+            ev.record(stream)
+    stream.synchronize()
+    gaps = sorted(blank[i].elapsed_time(blank[i + 1]) * 1e3 for i in range(8, 63))
+    event_us = gaps[len(gaps) // 2]                   # what an event record itself costs
+    in_step_us = {}
+    for j, (name, _) in enumerate(order):
+        spans = sorted(ev[j].elapsed_time(ev[j + 1]) * 1e3 for ev in marks)
+        in_step_us[name] = max(spans[len(spans) // 2] - event_us, 0.0)  # median
+
     # ---------------------------------------- per-kernel durations (same process)
     INNER = 20
     kernels = {"indexgen": k_indexgen, "dispatch": k_dispatch, "combine": k_combine,
@@ -323,6 +353,15 @@ def main():
             "step": "indexgen+dispatch+" + ("ffn(2 grouped GEMMs)+" if have_ffn else "") + "combine, one HIP graph",
         },
         "hbm_peak_frac": round(value / HBM_PEAK_GBPS, 4),
+        "in_step": {
+            "note": "medians of event-to-event intervals of the same step launched eagerly, minus "
+                    "the interval of two adjacent event records: inputs come from HBM after the "
+                    "FFN has swept the caches, unlike the back-to-back launches on one set of "
+                    "buffers that `kernels` and `value` are measured on",
+            "event_record_us": round(event_us, 2),
+            "us": {k: round(v, 2) for k, v in in_step_us.items()},
+            "dispatch_combine_GBps": round(dc_bytes / (in_step_us["dispatch"] + in_step_us["combine"]) / 1e3, 1),
+        },
         "layer_us": round(ms_per_step * 1e3, 2),
         "wall_ms_timed_region": round(wall_ms, 3),
         "algorithmic_bytes_dispatch_combine": dc_bytes,
