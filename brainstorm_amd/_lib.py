@@ -58,6 +58,11 @@ SIGNATURES = {
         _c_int,
         [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     ),
+    "brt_hip_grouped_gemm_routed": (
+        _c_int,
+        [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int,
+         _c_int, _c_int, _c_int, _c_ptr],
+    ),
 }
 
 _lib = None

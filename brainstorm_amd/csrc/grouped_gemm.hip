@@ -60,7 +60,9 @@ struct GemmArgs {
   const __bf16* const* bias;
   __bf16* out;
   const int* loads;
-  int E, P, K, N;
+  const int* tags;  // [T,E] tag matrix (column e: 1-based cells of path e in seat order) or null
+  int E, P, K, N, T;
+  int gather, scatter;  // rows of x / of out are addressed through the tags
   int tiles_n, tiles_m_max;
 };
 
@@ -102,7 +104,7 @@ __global__ __launch_bounds__(WAVES * 64) void grouped_gemm_kernel(GemmArgs a) {
   static_assert(BN % ROWS_PER_PASS == 0 && ROWS_PER_PASS % 8 == 0, "tile shape");
   constexpr int OUT_ROW = BN * 2 + 16;
   extern __shared__ __attribute__((aligned(16))) char smem[];
-  __shared__ int s_tile[3];  // expert, first row, valid rows
+  __shared__ int s_tile[4];  // expert, first row, valid rows, first row counted inside the expert
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -133,6 +135,7 @@ __global__ __launch_bounds__(WAVES * 64) void grouped_gemm_kernel(GemmArgs a) {
           s_tile[0] = e;
           s_tile[1] = carry_m + incl_m - m + local * BM;
           s_tile[2] = min(BM, m - local * BM);
+          s_tile[3] = local * BM;
         }
       }
       carry_t += __shfl(incl_t, kWave - 1, kWave);
@@ -145,6 +148,7 @@ __global__ __launch_bounds__(WAVES * 64) void grouped_gemm_kernel(GemmArgs a) {
   if (e < 0) return;  // beyond the last tile
   const int row0 = __builtin_amdgcn_readfirstlane(s_tile[1]);
   const int rows = __builtin_amdgcn_readfirstlane(s_tile[2]);
+  const int seat0 = __builtin_amdgcn_readfirstlane(s_tile[3]);
   const int row_tiles = (rows + 31) >> 5;
   const int n0 = nt * BN;
   const int K = a.K;
@@ -160,9 +164,13 @@ __global__ __launch_bounds__(WAVES * 64) void grouped_gemm_kernel(GemmArgs a) {
   // Buffer loads: a wave-uniform resource (base, byte extent) per operand, a 32-bit
   // per-lane byte offset and the K offset as the scalar offset, so the loop carries no
   // 64-bit address arithmetic; reads past the extent return zero instead of faulting.
-  const char* xa = reinterpret_cast<const char*>(a.x + static_cast<size_t>(row0) * K);
+  // Gather mode: row s of expert e is cell tags[s,e]-1 of x (the dispatch is folded into the
+  // operand load); an empty tag addresses past the extent and so reads a row of zeros, which
+  // is what dispatch writes for a padding row.
+  const bool gather = a.gather != 0;
+  const char* xa = reinterpret_cast<const char*>(gather ? a.x : a.x + static_cast<size_t>(row0) * K);
   const char* wb = reinterpret_cast<const char*>(a.w[e] + static_cast<size_t>(n0) * K);
-  const size_t xa_bytes = static_cast<size_t>(a.P - row0) * K * 2;
+  const size_t xa_bytes = static_cast<size_t>(gather ? a.T : a.P - row0) * K * 2;
   const size_t wb_bytes = static_cast<size_t>(a.N - n0) * K * 2;
   const __amdgpu_buffer_rsrc_t res_a = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<char*>(xa), 0, static_cast<int>(std::min<size_t>(xa_bytes, 0x7fffffff)), 0x00020000);
@@ -172,8 +180,15 @@ __global__ __launch_bounds__(WAVES * 64) void grouped_gemm_kernel(GemmArgs a) {
   const bool a_last = A_EXACT || lr + (A_LOADS - 1) * ROWS_PER_PASS < BM;
   uint32_t off_a[A_LOADS], off_b[B_LOADS];
 #pragma unroll
-  for (int i = 0; i < A_LOADS; ++i)
-    off_a[i] = (static_cast<uint32_t>(min(min(lr + i * ROWS_PER_PASS, BM - 1), rows - 1)) * K + lc * 8) * 2;
+  for (int i = 0; i < A_LOADS; ++i) {
+    const int r = min(min(lr + i * ROWS_PER_PASS, BM - 1), rows - 1);
+    if (gather) {
+      const int tag = a.tags[static_cast<size_t>(seat0 + r) * a.E + e];
+      off_a[i] = (tag >= 1 && tag <= a.T) ? (static_cast<uint32_t>(tag - 1) * K + lc * 8) * 2 : 0x80000000u;
+    } else {
+      off_a[i] = (static_cast<uint32_t>(r) * K + lc * 8) * 2;
+    }
+  }
 #pragma unroll
   for (int i = 0; i < B_LOADS; ++i)
     off_b[i] = (static_cast<uint32_t>(min(lr + i * ROWS_PER_PASS, a.N - n0 - 1)) * K + lc * 8) * 2;
@@ -345,11 +360,18 @@ __global__ __launch_bounds__(WAVES * 64) void grouped_gemm_kernel(GemmArgs a) {
   }
   __syncthreads();
   constexpr int OUT_CHUNKS = BN / 8;
-  __bf16* __restrict__ oc = a.out + static_cast<size_t>(row0) * a.N + n0;
+  // Scatter mode: row s of expert e goes to cell tags[s,e]-1 of out (the combine of a
+  // single-path route is folded into the store); rows without a tag are dropped.
+  __bf16* __restrict__ oc = a.out + (a.scatter ? 0 : static_cast<size_t>(row0) * a.N) + n0;
   for (int q = tid; q < rows * OUT_CHUNKS; q += THREADS) {
     const int r = q / OUT_CHUNKS, c = q - r * OUT_CHUNKS;
-    if (n0 + c * 8 < a.N)
-      *reinterpret_cast<u32x4*>(oc + static_cast<size_t>(r) * a.N + c * 8) =
+    long to = r;
+    if (a.scatter) {
+      const int tag = a.tags[static_cast<size_t>(seat0 + r) * a.E + e];
+      to = (tag >= 1 && tag <= a.T) ? tag - 1 : -1;
+    }
+    if (to >= 0 && n0 + c * 8 < a.N)
+      *reinterpret_cast<u32x4*>(oc + static_cast<size_t>(to) * a.N + c * 8) =
           *reinterpret_cast<const u32x4*>(smem + r * OUT_ROW + c * 16);
   }
 }
@@ -387,16 +409,23 @@ int launch(GemmArgs& a, int act, hipStream_t st) {
 
 using namespace brt;
 
-extern "C" int brt_hip_grouped_gemm(const void* x, const void* const* weights,
-                                    const void* const* biases, void* out, const int32_t* loads,
-                                    int E, int P, int K, int N, int act, void* stream) {
-  if (E <= 0 || P < 0 || K <= 0 || N <= 0) return fail(BRT_E_INVALID, "bad shape E=%d P=%d K=%d N=%d", E, P, K, N);
+namespace {
+
+int grouped_gemm_impl(const void* x, const void* const* weights, const void* const* biases, void* out,
+                      const int32_t* loads, const int32_t* tags, int E, int P, int T, int K, int N,
+                      int act, int gather_in, int scatter_out, void* stream) {
+  if (E <= 0 || P < 0 || K <= 0 || N <= 0 || T < 0)
+    return fail(BRT_E_INVALID, "bad shape E=%d P=%d T=%d K=%d N=%d", E, P, T, K, N);
   if (K % 8 != 0 || N % 8 != 0)
     return fail(BRT_E_UNSUPPORTED, "K and N must be multiples of 8 (16-byte rows), got K=%d N=%d", K, N);
   if (act != BRT_ACT_NONE && act != BRT_ACT_GELU && act != BRT_ACT_RELU)
     return fail(BRT_E_INVALID, "unknown activation %d", act);
   if (P == 0) return BRT_OK;
+  if ((gather_in || scatter_out) && T == 0) return BRT_OK;
   if (!x || !weights || !out || !loads) return fail(BRT_E_INVALID, "null argument");
+  if ((gather_in || scatter_out) && !tags) return fail(BRT_E_INVALID, "gather/scatter need the tag matrix");
+  if (gather_in && static_cast<size_t>(T) * K * 2 > 0x7fffffffull)
+    return fail(BRT_E_UNSUPPORTED, "gathered input of %d x %d exceeds 2 GiB", T, K);
   if (!aligned(x, 16) || !aligned(out, 16)) return fail(BRT_E_INVALID, "x/out must be 16-byte aligned");
   GemmArgs a{};
   a.x = static_cast<const __bf16*>(x);
@@ -404,7 +433,9 @@ extern "C" int brt_hip_grouped_gemm(const void* x, const void* const* weights,
   a.bias = reinterpret_cast<const __bf16* const*>(biases);
   a.out = static_cast<__bf16*>(out);
   a.loads = loads;
-  a.E = E; a.P = P; a.K = K; a.N = N;
+  a.tags = tags;
+  a.E = E; a.P = P; a.K = K; a.N = N; a.T = T;
+  a.gather = gather_in != 0; a.scatter = scatter_out != 0;
   // Tile choice: a wavefront owns 160 x 64 outputs (7 LDS fragment reads feed 10 MFMAs;
   // LDS read bandwidth is what bounds the inner loop).  Wide outputs use 4 wavefronts
   // (160 x 256 per workgroup); narrow ones use 2 (160 x 128) so that the grid still
@@ -416,3 +447,19 @@ extern "C" int brt_hip_grouped_gemm(const void* x, const void* const* weights,
   return launch<5, 1, 4>(a, act, as_stream(stream));
 }
 
+}  // namespace
+
+extern "C" int brt_hip_grouped_gemm(const void* x, const void* const* weights,
+                                    const void* const* biases, void* out, const int32_t* loads,
+                                    int E, int P, int K, int N, int act, void* stream) {
+  return grouped_gemm_impl(x, weights, biases, out, loads, nullptr, E, P, 0, K, N, act, 0, 0, stream);
+}
+
+extern "C" int brt_hip_grouped_gemm_routed(const void* x, const void* const* weights,
+                                           const void* const* biases, void* out,
+                                           const int32_t* loads, const int32_t* tags, int E, int P,
+                                           int T, int K, int N, int act, int gather_in,
+                                           int scatter_out, void* stream) {
+  return grouped_gemm_impl(x, weights, biases, out, loads, tags, E, P, T, K, N, act, gather_in,
+                           scatter_out, stream);
+}

@@ -43,10 +43,19 @@ class _PointerTable:
 
 def grouped_linear(x: torch.Tensor, out: torch.Tensor, weight_table: torch.Tensor,
                    bias_table: Optional[torch.Tensor], loads: torch.Tensor, in_features: int,
-                   out_features: int, activation: Optional[str] = None) -> torch.Tensor:
+                   out_features: int, activation: Optional[str] = None, *,
+                   tags: Optional[torch.Tensor] = None, gather: bool = False,
+                   scatter: bool = False, rows: Optional[int] = None) -> torch.Tensor:
     """``out[s_e : s_e + loads[e]] = act(x[s_e : s_e + loads[e]] @ W_e^T + b_e)`` for every
     branch e, ``s_e = sum(loads[:e])``, in one launch.  ``weight_table`` /
-    ``bias_table`` are int64 device tensors holding the branch pointers."""
+    ``bias_table`` are int64 device tensors holding the branch pointers.
+
+    With ``tags`` (the ``[cells, paths]`` tag-index matrix of
+    ``generate_indices_and_loads(..., is_tag_index=True)``) the routing is folded into the
+    GEMM: ``gather=True`` reads row s of branch e from ``x[tags[s, e] - 1]`` (``x`` is the
+    cell-major tensor, no dispatch needed), ``scatter=True`` stores it to
+    ``out[tags[s, e] - 1]`` (``out`` is cell-major and doubles as the residual; single-path
+    routes only).  ``rows`` bounds ``sum(loads)`` when neither side is path-major."""
     if x.dtype != torch.bfloat16 or out.dtype != torch.bfloat16:
         raise NotImplementedError("the grouped GEMM computes in bf16 (fp32 accumulation)")
     if not (x.is_cuda and out.is_cuda and loads.is_cuda):
@@ -55,15 +64,37 @@ def grouped_linear(x: torch.Tensor, out: torch.Tensor, weight_table: torch.Tenso
         raise RuntimeError("capacities must be int32")
     if not (x.is_contiguous() and out.is_contiguous()):
         raise RuntimeError("shared inputs must be contiguous")
-    rows = x.shape[0]
-    if x.numel() != rows * in_features or out.numel() != rows * out_features:
+    if x.numel() != x.shape[0] * in_features or out.numel() != out.shape[0] * out_features:
         raise RuntimeError("shared inputs do not match [rows, in_features] / [rows, out_features]")
+    routed = gather or scatter
+    cells = 0
+    if routed:
+        if tags is None or not tags.is_cuda or tags.dtype != torch.int32 or not tags.is_contiguous():
+            raise RuntimeError("gather/scatter need the contiguous int32 tag-index matrix on the device")
+        cells = tags.shape[0]
+        if tags.shape[1] != loads.numel():
+            raise RuntimeError("tags must have one column per branch")
+        if (gather and x.shape[0] != cells) or (scatter and out.shape[0] != cells):
+            raise RuntimeError("a gathered input / scattered output has one row per cell")
+    if rows is None:
+        rows = out.shape[0] if not scatter else (x.shape[0] if not gather else tags.numel())
+    elif (not gather and rows > x.shape[0]) or (not scatter and rows > out.shape[0]):
+        raise RuntimeError("rows exceeds the path-major buffer")
+    if not routed and x.shape[0] != out.shape[0]:
+        raise RuntimeError("shared inputs must have the same number of rows")
     with torch.cuda.device(x.device):
-        _lib.check(_lib.lib().brt_hip_grouped_gemm(
-            x.data_ptr(), weight_table.data_ptr(),
-            None if bias_table is None else bias_table.data_ptr(), out.data_ptr(),
-            loads.data_ptr(), loads.numel(), rows, in_features, out_features, _ACT[activation],
-            torch.cuda.current_stream().cuda_stream))
+        lib = _lib.lib()
+        stream = torch.cuda.current_stream().cuda_stream
+        bias_ptr = None if bias_table is None else bias_table.data_ptr()
+        if routed:
+            _lib.check(lib.brt_hip_grouped_gemm_routed(
+                x.data_ptr(), weight_table.data_ptr(), bias_ptr, out.data_ptr(), loads.data_ptr(),
+                tags.data_ptr(), loads.numel(), rows, cells, in_features, out_features,
+                _ACT[activation], int(gather), int(scatter), stream))
+        else:
+            _lib.check(lib.brt_hip_grouped_gemm(
+                x.data_ptr(), weight_table.data_ptr(), bias_ptr, out.data_ptr(), loads.data_ptr(),
+                loads.numel(), rows, in_features, out_features, _ACT[activation], stream))
     return out
 
 

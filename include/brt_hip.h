@@ -184,6 +184,30 @@ int brt_hip_grouped_gemm(const void* x, const void* const* weights, const void* 
                          void* out, const int32_t* loads, int E, int P, int K, int N, int act,
                          void* stream);
 
+/*
+ * The same grouped GEMM with the routing folded into it (no counterpart in the
+ * reference, which dispatches, runs the expert kernel and combines in separate
+ * launches; this is the fusion of src/router/route.cu:13-282 into the operand load
+ * and the result store of the expert kernel).  `tags` is the [T,E] tag-index matrix
+ * that brt_hip_generate_indices_and_loads writes with is_tag_index=1: column e
+ * lists, in seat order, the 1-based cells routed to path e; 0 = empty slot.
+ *
+ *   gather_in=1   x is the cell-major tensor [T,K]; row s of expert e is
+ *                 x[tags[s,e]-1] (what dispatch would have copied there), an empty
+ *                 slot is a row of zeros.  gather_in=0: x is [P,K] as above.
+ *   scatter_out=1 out is cell-major [T,N]; row s of expert e is stored to
+ *                 out[tags[s,e]-1] (what combine does for a route in which no cell is
+ *                 on more than one path, without gates, with out as the residual);
+ *                 rows of empty slots are dropped.  scatter_out=0: out is [P,N].
+ *   Only rows s < loads[e] of column e are used, so a clipped capacity drops the
+ *   overflow exactly as seat indices beyond loads[e] do.  With gather_in the cell-major
+ *   input is limited to 2 GiB.
+ */
+int brt_hip_grouped_gemm_routed(const void* x, const void* const* weights,
+                                const void* const* biases, void* out, const int32_t* loads,
+                                const int32_t* tags, int E, int P, int T, int K, int N, int act,
+                                int gather_in, int scatter_out, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -107,3 +107,81 @@ def test_ragged_dirichlet_loads_task_moe_shape():
     assert min(loads) == 0 and max(loads) > 320
     run(loads, 512, 2048, act="gelu", bias=True)
     run(loads, 2048, 512, slack=3)
+
+
+# --------------------------------------------------- routing folded into the GEMM
+def _expert_tables(E, K, N, seed):
+    g = torch.Generator().manual_seed(seed)
+    ws = [(torch.randn(N, K, generator=g) * 0.05).to(torch.bfloat16).cuda() for _ in range(E)]
+    return ws, torch.tensor([w.data_ptr() for w in ws], dtype=torch.int64, device="cuda")
+
+
+@pytest.mark.parametrize("T,E,d,dff,cap,pad", [
+    (2048, 16, 256, 512, 160, False),     # clip: overflow dropped
+    (2048, 16, 256, 512, 160, True),      # every expert padded to 160 rows (empty slots = zero rows)
+    (1000, 8, 136, 264, 400, False),      # several row blocks per expert, K and N tails
+    (300, 64, 64, 128, 16, False),        # most experts nearly empty
+])
+def test_ffn_with_gather_and_scatter_equals_dispatch_ffn_combine(T, E, d, dff, cap, pad):
+    """index generation in tag mode -> GEMM reading cells through the tags -> GEMM storing
+    through the tags must give bit for bit what dispatch -> GEMM -> GEMM -> combine gives."""
+    import oracle
+    from brainstorm_amd._C import router as c_router
+    from brainstorm_amd.jit import grouped_linear
+    from routing_cases import topk_mask
+
+    mask, _ = topk_mask(T, E, 1, seed=T + E)
+    d_mask = torch.from_numpy(mask).cuda()
+    caps = torch.tensor([cap], dtype=torch.int32, device="cuda")
+    x = torch.randn(T, d, generator=torch.Generator().manual_seed(T)).to(torch.bfloat16).cuda()
+    w1, t1 = _expert_tables(E, d, dff, 1)
+    w2, t2 = _expert_tables(E, dff, d, 2)
+
+    # the unfused path
+    idx, loads = c_router.generate_indices_and_loads(d_mask, caps, pad)
+    (y,) = c_router.dispatch_with_indices_and_loads(x, idx, loads)
+    P = y.shape[0]
+    h = torch.empty(P, dff, dtype=torch.bfloat16, device="cuda")
+    y2 = torch.empty(P, d, dtype=torch.bfloat16, device="cuda")
+    grouped_linear(y, h, t1, None, loads, d, dff, "gelu")
+    grouped_linear(h, y2, t2, None, loads, dff, d)
+    (want,) = c_router.combine_with_indices_and_loads(y2, idx, loads, None, x.clone())
+
+    # the fused path
+    tags, loads_t = c_router.generate_indices_and_loads(d_mask, caps, pad, False, True)
+    assert torch.equal(loads_t, loads)
+    o_tags, _ = oracle.generate_indices_and_loads(mask, [cap], capacity_padding=pad, is_tag_index=True)
+    assert np.array_equal(tags.cpu().numpy(), o_tags)
+    hf = torch.full((P + 7, dff), float("nan"), dtype=torch.bfloat16, device="cuda")
+    out = x.clone()
+    grouped_linear(x, hf, t1, None, loads, d, dff, "gelu", tags=tags, gather=True, rows=P)
+    assert torch.equal(hf[:P].view(torch.int16), h.view(torch.int16))
+    assert torch.isnan(hf[P:].float()).all()
+    grouped_linear(hf, out, t2, None, loads, dff, d, tags=tags, scatter=True, rows=P)
+    assert torch.equal(out.view(torch.int16), want.view(torch.int16))
+
+    # and both agree with per-expert torch matmuls on the cells each expert kept
+    lh = loads.cpu().tolist()
+    ref = x.float().clone()
+    for e in range(E):
+        cells = np.nonzero(mask[:, e])[0][: lh[e]]
+        if len(cells):
+            hid = torch.nn.functional.gelu(x[cells].float() @ w1[e].float().t()).to(torch.bfloat16)
+            ref[cells] = hid.float() @ w2[e].float().t()
+    scale = ref.abs().max()
+    assert (out.float() - ref).abs().max() / scale < 1e-2
+
+
+def test_routed_gemm_argument_checks():
+    from brainstorm_amd.jit import grouped_linear
+
+    x = torch.zeros(8, 64, dtype=torch.bfloat16, device="cuda")
+    out = torch.zeros(8, 64, dtype=torch.bfloat16, device="cuda")
+    loads = torch.tensor([8], dtype=torch.int32, device="cuda")
+    _, table = _expert_tables(1, 64, 64, 3)
+    with pytest.raises(RuntimeError):
+        grouped_linear(x, out, table, None, loads, 64, 64, gather=True)           # no tags
+    tags = torch.arange(1, 9, dtype=torch.int32, device="cuda").view(8, 1)
+    with pytest.raises(RuntimeError):
+        grouped_linear(x[:4], out, table, None, loads, 64, 64, tags=tags, gather=True)  # x not cell-major
+    grouped_linear(x, out, table, None, loads, 64, 64, tags=tags, gather=True, scatter=True)
