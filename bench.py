@@ -159,6 +159,35 @@ def main():
             combine_src.data_ptr(), out_gather.data_ptr(), None, idx.data_ptr(), loads.data_ptr(),
             T, D, E, P, 0, 1, _lib.BF16, _lib.BF16, _lib.F32, sptr()))
 
+    # the same layer with dispatch folded into the operand load of the first GEMM and combine
+    # into the result store of the second one (tag-index matrix instead of seat indices)
+    tag_idx = torch.zeros_like(mask)
+    loads_counts_t = torch.empty(2, E, dtype=torch.int32, device=dev)
+    out_fused = x.clone()
+    h_fused = torch.empty(P, DFF, dtype=torch.bfloat16, device=dev)
+
+    def k_indexgen_tags():
+        _lib.check(L.brt_hip_generate_indices_and_loads(
+            mask.data_ptr(), tag_idx.data_ptr(), loads_counts_t[0].data_ptr(),
+            loads_counts_t[1].data_ptr(), T, E, caps.data_ptr(), 1, 0, 0, 1, ws.data_ptr(),
+            ws.numel(), sptr()))
+
+    def k_gemm1_gather():
+        _lib.check(L.brt_hip_grouped_gemm_routed(
+            x.data_ptr(), wi_tab.data_ptr(), None, h_fused.data_ptr(), loads_counts_t[0].data_ptr(),
+            tag_idx.data_ptr(), E, P, T, D, DFF, _lib.ACT_GELU, 1, 0, sptr()))
+
+    def k_gemm2_scatter():
+        _lib.check(L.brt_hip_grouped_gemm_routed(
+            h_fused.data_ptr(), wo_tab.data_ptr(), None, out_fused.data_ptr(),
+            loads_counts_t[0].data_ptr(), tag_idx.data_ptr(), E, P, T, DFF, D, _lib.ACT_NONE, 0, 1,
+            sptr()))
+
+    def step_fused():
+        k_indexgen_tags()
+        k_gemm1_gather()
+        k_gemm2_scatter()
+
     def step():
         k_indexgen()
         k_dispatch()
@@ -195,6 +224,12 @@ def main():
     stream.synchronize()
     if not torch.equal(out.view(torch.int16), out_gather.view(torch.int16)):
         sys.exit("bench.py: tag-driven and index-driven combine disagree")
+    if have_ffn:
+        with torch.cuda.stream(stream):
+            step_fused()
+        stream.synchronize()
+        if not torch.equal(out.view(torch.int16), out_fused.view(torch.int16)):
+            sys.exit("bench.py: the layer with routing folded into the GEMMs disagrees")
 
     # ------------------------------------------------------- timed region: K steps
     g_step = capture(step)
@@ -208,6 +243,11 @@ def main():
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3
     ms_per_step = ms_total / args.steps
+    fused_layer_us = None
+    if have_ffn:
+        g_fused = capture(step_fused)
+        timed(g_fused, args.warmup)
+        fused_layer_us = timed(g_fused, args.steps) / args.steps * 1e3
 
     # ------------- kernel durations inside the step (cold inputs, real neighbours): the same step
     # launched eagerly with an event after every launch.  The two GEMMs keep the GPU busy long
@@ -244,7 +284,9 @@ def main():
     kernels = {"indexgen": k_indexgen, "dispatch": k_dispatch, "combine": k_combine,
                "combine_gather": k_combine_gather}
     if have_ffn:
-        kernels.update({"ffn_gemm1_gelu": k_gemm1, "ffn_gemm2": k_gemm2})
+        kernels.update({"ffn_gemm1_gelu": k_gemm1, "ffn_gemm2": k_gemm2,
+                        "indexgen_tags": k_indexgen_tags, "ffn_gemm1_gelu_gather": k_gemm1_gather,
+                        "ffn_gemm2_scatter": k_gemm2_scatter})
     replays = max(10, args.steps // 4)
     us = {}
     for name, fn in kernels.items():
@@ -268,6 +310,9 @@ def main():
         "combine": 2 * R * D * es + 4 * P,
     }
     flops = {"ffn_gemm1_gelu": 2.0 * R * D * DFF, "ffn_gemm2": 2.0 * R * DFF * D}
+    flops["ffn_gemm1_gelu_gather"] = flops["ffn_gemm1_gelu"]
+    flops["ffn_gemm2_scatter"] = flops["ffn_gemm2"]
+    bytes_["indexgen_tags"] = bytes_["indexgen"]
     dc_bytes = bytes_["dispatch"] + bytes_["combine"]
     dc_us = us["dispatch"] + us["combine"]
     value = dc_bytes / dc_us / 1e3  # GB/s
@@ -295,7 +340,7 @@ def main():
             entry["TFLOPs"] = round(flops[name] / us[name] / 1e6, 1)
             entry["mfma_frac"] = round(flops[name] / us[name] / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4)
             # the expert FFN at 128 rows per expert streams its weights: HBM is the bound
-            hbm = MEASURED_TRAFFIC_BYTES[name]
+            hbm = MEASURED_TRAFFIC_BYTES.get(name.replace("_gather", "").replace("_scatter", ""))
             entry["hbm_GBps"] = round(hbm / us[name] / 1e3, 1)
             entry["hbm_frac"] = round(hbm / us[name] / 1e3 / HBM_PEAK_GBPS, 4)
         per_kernel[name] = entry
@@ -363,6 +408,8 @@ def main():
             "dispatch_combine_GBps": round(dc_bytes / (in_step_us["dispatch"] + in_step_us["combine"]) / 1e3, 1),
         },
         "layer_us": round(ms_per_step * 1e3, 2),
+        "layer_fused_us": None if fused_layer_us is None else round(fused_layer_us, 2),
+        "layer_fused_step": "indexgen(tag indices)+GEMM1 gathering cells+GEMM2 scattering to cells, one HIP graph",
         "wall_ms_timed_region": round(wall_ms, 3),
         "algorithmic_bytes_dispatch_combine": dc_bytes,
         "kernels": per_kernel,
