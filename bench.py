@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
-Workload (BASELINE.json configs[1]): Switch-MoE layer, bf16, 8192 tokens x d=768,
+Workload: the Switch-MoE layer of the baseline configurations, bf16, 8192 tokens x d=768,
 64 experts, top-1 softmax gate over N(0,1) logits, capacity factor 1.25
 (capacity 160, overflow dropped), expert FFN 768->3072->768 GELU with N(0,0.02)
 weights; seeded synthetic data, everything resident in HBM before timing.

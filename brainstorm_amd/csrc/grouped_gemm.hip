@@ -436,13 +436,31 @@ int grouped_gemm_impl(const void* x, const void* const* weights, const void* con
   a.tags = tags;
   a.E = E; a.P = P; a.K = K; a.N = N; a.T = T;
   a.gather = gather_in != 0; a.scatter = scatter_out != 0;
-  // Tile choice: a wavefront owns 160 x 64 outputs (7 LDS fragment reads feed 10 MFMAs;
-  // LDS read bandwidth is what bounds the inner loop).  Wide outputs use 4 wavefronts
-  // (160 x 256 per workgroup); narrow ones use 2 (160 x 128) so that the grid still
-  // has more workgroups than the chip has compute units.
+  // Tile choice.  A wavefront owns 160 x 64 outputs (7 LDS fragment reads feed 10 MFMAs); a
+  // workgroup is 2, 3 or 4 of them side by side.  The kernel is bound by how fast a CU can fill
+  // its L1 (about 29 KB/us, L2 hits included), so the shape is the one that gives the busiest CU
+  // the fewest operand bytes: wide tiles re-read the activation rows less often, narrow ones
+  // keep all CUs busy when there are few tiles (only the 2-wavefront tile fits twice on a CU).
   static const int forced = std::getenv("BRT_GEMM_SHAPE") ? std::atoi(std::getenv("BRT_GEMM_SHAPE")) : 0;
-  const int shape = forced ? forced : (N >= 2048 ? 24 : 22);
+  int shape = forced;
+  if (shape == 0) {
+    static const int cus = [] {
+      int dev = 0, n = 256;
+      if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
+      return std::max(n, 1);
+    }();
+    const long row_blocks = std::max<long>((P + 159) / 160, std::min(E, P));  // estimate; loads live on the device
+    double best = 0;
+    for (int waves = 4; waves >= 2; --waves) {
+      const long tiles = row_blocks * ((N + 64 * waves - 1) / (64 * waves));
+      const long slots = static_cast<long>(cus) * (waves == 2 ? 2 : 1);
+      const double rounds = static_cast<double>((tiles + slots - 1) / slots) * (waves == 2 ? 2 : 1);
+      const double cost = rounds * (160 + 64 * waves);  // operand rows the busiest CU streams per K
+      if (shape == 0 || cost < best) { best = cost; shape = 20 + waves; }
+    }
+  }
   if (shape == 24) return launch<5, 2, 4>(a, act, as_stream(stream));
+  if (shape == 23) return launch<5, 2, 3>(a, act, as_stream(stream));
   if (shape == 22) return launch<5, 2, 2>(a, act, as_stream(stream));
   return launch<5, 1, 4>(a, act, as_stream(stream));
 }

@@ -68,7 +68,8 @@ ScanGeometry scan_geometry(int T, int E) {
   // over earlier bands every band has to form.
   const long one_batch = static_cast<long>(kWavesPB) * kBatch * rps;
   const int fit = static_cast<int>(std::min<long>(kMaxBands, (T + one_batch - 1) / one_batch));
-  const int want = env_int("BRT_SCAN_BANDS", std::max(128, fit));
+  static const int forced_bands = env_int("BRT_SCAN_BANDS", 0);  // tuning knob, read once
+  const int want = forced_bands > 0 ? forced_bands : std::max(128, fit);
   long rows_pb = (static_cast<long>(T) + want - 1) / want;
   rows_pb = std::max<long>(rows_pb, (static_cast<long>(T) + kMaxBands - 1) / kMaxBands);
   long rows_pw = (rows_pb + kWavesPB - 1) / kWavesPB;

@@ -1155,9 +1155,20 @@ int pick_unit_bytes(size_t row_bytes, int elem, const void* p0, const void* p1, 
   return 0;
 }
 
+// Tuning knobs from the environment, read once per process.
 int env_int(const char* name, int fallback) {
   const char* v = getenv(name);
   return v ? atoi(v) : fallback;
+}
+struct Knobs {
+  int dispatch_rows = env_int("BRT_DISPATCH_ROWS", 0);
+  int combine_rows = env_int("BRT_COMBINE_ROWS", 0);
+  int waves_pb = env_int("BRT_WAVES_PB", kBlock / kWave);
+  bool no_lean = env_int("BRT_NO_LEAN", 0) != 0;
+};
+const Knobs& knobs() {
+  static const Knobs k;
+  return k;
 }
 
 StepMap make_step_map(int E) {
@@ -1173,8 +1184,8 @@ StepMap make_step_map(int E) {
 // Rows of the index matrix per wavefront: enough units that each lane has a
 // handful of 16-byte accesses in flight, few enough index words that one batch
 // of kSteps loads covers them.
-int rows_per_wave(const char* env, int cpr, int E, long T) {
-  int rows = env_int(env, 0);
+int rows_per_wave(int forced_rows, int cpr, int E, long T) {
+  int rows = forced_rows;
   if (rows <= 0) {
     rows = std::max(1, 384 / std::max(cpr, 1));
     while (rows > 1 && (T + rows - 1) / rows < 4096) rows >>= 1;  // keep every SIMD busy
@@ -1198,7 +1209,7 @@ struct LaunchShape {
 bool launch_shape(long T, int rows_pw, int lds_pw_ints, LaunchShape* out) {
   const size_t per_wave = static_cast<size_t>(lds_pw_ints) * 4;
   if (per_wave > 60 * 1024) return false;
-  int waves = std::max(1, std::min(kBlock / kWave, env_int("BRT_WAVES_PB", kBlock / kWave)));
+  int waves = std::max(1, std::min(kBlock / kWave, knobs().waves_pb));
   while (waves > 1 && per_wave * waves > 60 * 1024) waves >>= 1;
   const long n_waves = std::max(1l, (T + rows_pw - 1) / rows_pw);
   out->waves_pb = waves;
@@ -1220,7 +1231,7 @@ template <int BYTES, int DT>
 void launch_dispatch(const DispatchArgs& a, const LaunchShape& sh, hipStream_t st) {
   const dim3 grid(sh.grid), block(sh.waves_pb * kWave);
   if constexpr (BYTES == 16) {
-    if (a.E <= kWave && a.is_1d && !a.is_tag_index && env_int("BRT_NO_LEAN", 0) == 0) {
+    if (a.E <= kWave && a.is_1d && !a.is_tag_index && !knobs().no_lean) {
 #define BRT_LAUNCH(LS, UPR) \
   hipLaunchKernelGGL((dispatch_lean_kernel<DT, LS, UPR>), grid, block, 0, st, a);
       BRT_LEAN_SHAPES(BRT_LAUNCH)
@@ -1243,10 +1254,9 @@ template <int BYTES, int IN_DT, int OUT_DT>
 void launch_combine(const CombineArgs& a, const LaunchShape& sh, hipStream_t st) {
   const dim3 grid(sh.grid), block(sh.waves_pb * kWave);
   if constexpr (BYTES == 16) {
-    if (a.E <= kWave && env_int("BRT_NO_LEAN", 0) == 0) {
+    if (a.E <= kWave && !knobs().no_lean) {
 #define BRT_LAUNCH(LS, UPR) \
   hipLaunchKernelGGL((combine_lean_kernel<IN_DT, OUT_DT, LS, UPR>), grid, block, 0, st, a);
-      if (env_int("BRT_COMBINE_UPR1", 0) && a.cpr > kWave) { BRT_LAUNCH(6, 1) return; }
       BRT_LEAN_SHAPES(BRT_LAUNCH)
 #undef BRT_LAUNCH
       return;
@@ -1298,7 +1308,7 @@ extern "C" int brt_hip_dispatch(const void* src, void* dst, const void* gates,
   a.cpr = static_cast<int>(row_bytes / bytes);
   a.is_1d = is_1d_routing; a.is_tag_index = is_tag_index;
   a.map = make_step_map(E);
-  a.rows_pw = rows_per_wave("BRT_DISPATCH_ROWS", a.cpr, E, T);
+  a.rows_pw = rows_per_wave(knobs().dispatch_rows, a.cpr, E, T);
   a.lds_pw = 3 * E + 1 + 3 * a.rows_pw * E;
   LaunchShape sh;
   if (!launch_shape(T, a.rows_pw, a.lds_pw, &sh))
@@ -1347,7 +1357,7 @@ extern "C" int brt_hip_combine(const void* src, void* dst, const void* gates,
   a.cpr = static_cast<int>(row_bytes / bytes);
   a.is_residual = is_residual; a.gate_dtype = gate_dtype;
   a.map = make_step_map(E);
-  a.rows_pw = rows_per_wave("BRT_COMBINE_ROWS", a.cpr, E, T);
+  a.rows_pw = rows_per_wave(knobs().combine_rows, a.cpr, E, T);
   a.lds_pw = 2 * E + a.rows_pw + 2 * a.rows_pw * E;
   LaunchShape sh;
   if (!launch_shape(T, a.rows_pw, a.lds_pw, &sh))
@@ -1388,7 +1398,7 @@ extern "C" int brt_hip_combine_by_tags(const void* src, void* dst, const int32_t
   CombineRowsArgs a{};
   a.src = src; a.dst = dst; a.row_tags = row_tags; a.T = T; a.P = P;
   a.cpr = static_cast<int>(row_bytes / 16);
-  int rows = env_int("BRT_COMBINE_ROWS", 0);
+  int rows = knobs().combine_rows;
   if (rows <= 0) {
     rows = std::max(1, 384 / a.cpr);
     while (rows > 1 && (P + rows - 1) / rows < 4096) rows >>= 1;

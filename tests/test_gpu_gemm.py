@@ -91,7 +91,7 @@ def test_make_jit_kernel_homo_fuse_contract():
 
 
 def test_full_size_switch_ffn():
-    # BASELINE configs[1]: 64 experts, 768 -> 3072 -> 768, ~128 rows per expert
+    # the Switch-MoE benchmark shape: 64 experts, 768 -> 3072 -> 768, ~128 rows per expert
     rng = np.random.default_rng(2)
     loads = np.minimum(rng.multinomial(8192, [1 / 64] * 64), 160).tolist()
     run(loads, 768, 3072, act="gelu")
@@ -99,7 +99,7 @@ def test_full_size_switch_ffn():
 
 
 def test_ragged_dirichlet_loads_task_moe_shape():
-    # BASELINE configs[4] at reduced size: loads ~ Dirichlet(0.3) (many empty experts, a few
+    # the ragged task-MoE benchmark shape at reduced size: loads ~ Dirichlet(0.3) (many empty experts, a few
     # with hundreds of rows), one launch over the ragged batches, both FFN shapes
     rng = np.random.default_rng(4)
     E, rows = 48, 4096
