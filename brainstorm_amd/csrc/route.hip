@@ -951,138 +951,68 @@ __global__ __launch_bounds__(kBlock) void combine_lean_kernel(CombineArgs a) {
   const U* __restrict__ src = static_cast<const U*>(a.src);
   char* __restrict__ dst = static_cast<char*>(a.dst);
 
-  auto load_idx = [&](int step) {
-    const int row = step * rps + sub;
-    return (step < n_steps && row < nt && e < E) ? idx0[row * E + e] : 0;
-  };
-  // index vectors are fetched two steps ahead of their use
-  int v_cur = load_idx(0), v_next = load_idx(1);
+  int v_next = (sub < nt && e < E) ? idx0[sub * E + e] : 0;
   const SmallTables tab = small_tables(a.loads, E, a.mpl, ep_shift, lane);
 
-  // per step (64 >> ep_shift tokens): source row and gate of (token sub, path e) in lane
-  // sub*ep + e, and the mask of routed (token, path) pairs
-  struct StepVec {
-    int src_row;
-    float gate;
-    unsigned long long m;
-    int tokens;
-    long t_first;
-  };
-  auto make_step = [&](int step, int v) {
-    StepVec s;
+  for (int step = 0; step < n_steps; ++step) {
+    const int v = v_next;
     const int row = step * rps + sub;
-    s.src_row = tab.start_e + v - 1;
-    const bool ok = row < nt && e < E && v >= 1 && v <= tab.load_e && s.src_row < a.P;
-    s.gate = 1.0f;
+    {
+      const int nrow = row + rps;
+      v_next = (step + 1 < n_steps && nrow < nt && e < E) ? idx0[nrow * E + e] : 0;
+    }
+    const int src_row = tab.start_e + v - 1;
+    const bool ok = row < nt && e < E && v >= 1 && v <= tab.load_e && src_row < a.P;
+    float gate = 1.0f;
     if (ok && a.gates != nullptr)
-      s.gate = load_gate(a.gates, a.gate_dtype, static_cast<size_t>(t0 + row) * E + e);
-    s.m = __ballot(ok);
-    s.tokens = min(rps, nt - step * rps);
-    s.t_first = t0 + step * rps;
-    return s;
-  };
-
-  // One item = GROUPS tokens (one per lane group) x one pass of LPR*UPR units.  Its first
-  // path's rows are loaded when the item is prepared and consumed one item later, so the
-  // loads of two consecutive items (tokens) are in flight together; further paths of a
-  // token (top-k > 1) are walked in ascending order when the item is consumed.
-  struct Item {
-    unsigned long long mine;
-    size_t to;
-    int i, off0, src_vec;  // i: token slot inside its step
-    float gate_vec, g;
-    bool live, has;
-    U val[UPR];
-  };
-  auto prepare = [&](const StepVec& s, int tb, int off0) {
-    Item it;
-    const int i = tb + gidx;
-    it.i = i;
-    it.live = i < s.tokens;
-    it.mine = it.live ? (s.m >> (i * ep)) & seg0 : 0ull;
-    it.has = it.mine != 0;
-    it.to = static_cast<size_t>(s.t_first + i) * cpr;
-    it.off0 = off0;
-    it.src_vec = s.src_row;
-    it.gate_vec = s.gate;
-    const int b = (i * ep + __builtin_ctzll(it.mine | (1ull << 63))) & (kWave - 1);
-    const int sr = __builtin_amdgcn_ds_bpermute(b << 2, s.src_row);
-    it.g = __int_as_float(__builtin_amdgcn_ds_bpermute(b << 2, __float_as_int(s.gate)));
+      gate = load_gate(a.gates, a.gate_dtype, static_cast<size_t>(t0 + row) * E + e);
+    const unsigned long long m = __ballot(ok);
+    const int tokens = min(rps, nt - step * rps);
+    for (int tb = 0; tb < tokens; tb += GROUPS) {
+      const int i = tb + gidx;
+      const unsigned long long mine = i < tokens ? (m >> (i * ep)) & seg0 : 0ull;
+      const size_t to = static_cast<size_t>(t0 + step * rps + i) * cpr;
+      for (int off0 = 0; off0 < cpr; off0 += LPR * UPR) {
+        float acc[UPR][NE];
 #pragma unroll
-    for (int u = 0; u < UPR; ++u) {
-      const int off = off0 + u * LPR + glane;
-      it.val[u] = U{};
-      if (it.has && off < cpr) it.val[u] = src[static_cast<size_t>(sr) * cpr + off];
-    }
-    return it;
-  };
-  auto consume = [&](const Item& it) {
-    float acc[UPR][NE];
+        for (int u = 0; u < UPR; ++u)
 #pragma unroll
-    for (int u = 0; u < UPR; ++u) {
-      float x[NE];
-      unpack<IN_DT, 16>(it.val[u], x);
-      // one rounding for the product, one for the sum (no fused multiply-add); the sum
-      // starts from +0 like the sequential reference
+          for (int q = 0; q < NE; ++q) acc[u][q] = 0.0f;
+        unsigned long long rem = mine;
+        while (__ballot(rem != 0) != 0) {  // ascending path order: lowest set bit first
+          const bool has = rem != 0;
+          const int b = i * ep + __builtin_ctzll(rem | (1ull << 63));
+          rem &= rem - 1;
+          const int sr = __builtin_amdgcn_ds_bpermute(b << 2, src_row);
+          const float g = __int_as_float(__builtin_amdgcn_ds_bpermute(b << 2, __float_as_int(gate)));
+          U val[UPR];
 #pragma unroll
-      for (int q = 0; q < NE; ++q) acc[u][q] = it.has ? 0.0f + x[q] * it.g : 0.0f;
-    }
-    unsigned long long rem = it.mine & (it.mine - 1);
-    while (__ballot(rem != 0) != 0) {  // ascending path order: lowest set bit first
-      const bool has = rem != 0;
-      const int b = (it.i * ep + __builtin_ctzll(rem | (1ull << 63))) & (kWave - 1);
-      rem &= rem - 1;
-      const int sr = __builtin_amdgcn_ds_bpermute(b << 2, it.src_vec);
-      const float g = __int_as_float(__builtin_amdgcn_ds_bpermute(b << 2, __float_as_int(it.gate_vec)));
-      U val[UPR];
+          for (int u = 0; u < UPR; ++u) {
+            const int off = off0 + u * LPR + glane;
+            if (has && off < cpr) val[u] = src[static_cast<size_t>(sr) * cpr + off];
+          }
 #pragma unroll
-      for (int u = 0; u < UPR; ++u) {
-        const int off = it.off0 + u * LPR + glane;
-        if (has && off < cpr) val[u] = src[static_cast<size_t>(sr) * cpr + off];
-      }
+          for (int u = 0; u < UPR; ++u) {
+            const int off = off0 + u * LPR + glane;
+            if (has && off < cpr) {
+              float x[NE];
+              unpack<IN_DT, 16>(val[u], x);
+              // one rounding for the product, one for the sum (no fused multiply-add)
 #pragma unroll
-      for (int u = 0; u < UPR; ++u) {
-        const int off = it.off0 + u * LPR + glane;
-        if (has && off < cpr) {
-          float x[NE];
-          unpack<IN_DT, 16>(val[u], x);
+              for (int q = 0; q < NE; ++q) acc[u][q] = acc[u][q] + x[q] * g;
+            }
+          }
+        }
+        if (i < tokens && (mine != 0 || !a.is_residual)) {
 #pragma unroll
-          for (int q = 0; q < NE; ++q) acc[u][q] = acc[u][q] + x[q] * g;
+          for (int u = 0; u < UPR; ++u) {
+            const int off = off0 + u * LPR + glane;
+            if (off < cpr) pack_store<OUT_DT, NE>(dst + (to + off) * OUT_BYTES, acc[u]);
+          }
         }
       }
     }
-    if (it.live && (it.mine != 0 || !a.is_residual)) {
-#pragma unroll
-      for (int u = 0; u < UPR; ++u) {
-        const int off = it.off0 + u * LPR + glane;
-        if (off < cpr) pack_store<OUT_DT, NE>(dst + (it.to + off) * OUT_BYTES, acc[u]);
-      }
-    }
-  };
-
-  Item pend;
-  pend.mine = 0; pend.to = 0; pend.i = 0; pend.off0 = 0; pend.src_vec = 0; pend.gate_vec = 0.0f; pend.g = 0.0f;
-  pend.live = false; pend.has = false;
-#pragma unroll
-  for (int u = 0; u < UPR; ++u) pend.val[u] = U{};
-
-  StepVec cur = make_step(0, v_cur);
-  for (int step = 0; step < n_steps; ++step) {
-    StepVec nxt = cur;
-    if (step + 1 < n_steps) {
-      nxt = make_step(step + 1, v_next);
-      v_next = load_idx(step + 2);
-    }
-    for (int tb = 0; tb < cur.tokens; tb += GROUPS) {
-      for (int off0 = 0; off0 < cpr; off0 += LPR * UPR) {
-        const Item fresh = prepare(cur, tb, off0);
-        consume(pend);
-        pend = fresh;
-      }
-    }
-    cur = nxt;
   }
-  consume(pend);
 }
 
 // Combine in scatter form for routes where no cell owns more than one row (top-1):
