@@ -283,10 +283,29 @@ def main():
         spans = sorted(ev[j].elapsed_time(ev[j + 1]) * 1e3 for ev in marks)
         in_step_us[name] = max(spans[len(spans) // 2] - event_us, 0.0)  # median
 
+    # gate front-end (reported separately, not part of the step): scores -> hot mask
+    gate_mask = torch.empty_like(mask)
+    probs_d = probs.to(dev)
+
+    def k_gate():
+        _lib.check(L.brt_hip_topk_hot_mask(probs_d.data_ptr(), gate_mask.data_ptr(), T, E, 1,
+                                           _lib.F32, sptr()))
+
+    def k_gate_torch():  # what the reference's TopKProtocol launches
+        torch.zeros_like(probs_d, dtype=torch.int32).scatter_(
+            1, torch.topk(probs_d, 1, dim=1).indices, 1)
+
+    with torch.cuda.stream(stream):
+        k_gate()
+    stream.synchronize()
+    if not torch.equal(gate_mask, mask):
+        sys.exit("bench.py: the gate kernel does not reproduce the argmax mask")
+
     # ---------------------------------------- per-kernel durations (same process)
     INNER = 20
     kernels = {"indexgen": k_indexgen, "dispatch": k_dispatch, "combine": k_combine,
-               "combine_gather": k_combine_gather}
+               "combine_gather": k_combine_gather, "gate_topk_mask": k_gate,
+               "gate_topk_mask_torch_ops": k_gate_torch}
     if have_ffn:
         kernels.update({"ffn_gemm1_gelu": k_gemm1, "ffn_gemm2": k_gemm2,
                         "indexgen_tags": k_indexgen_tags, "ffn_gemm1_gelu_gather": k_gemm1_gather,
@@ -317,6 +336,7 @@ def main():
     flops["ffn_gemm1_gelu_gather"] = flops["ffn_gemm1_gelu"]
     flops["ffn_gemm2_scatter"] = flops["ffn_gemm2"]
     bytes_["indexgen_tags"] = bytes_["indexgen"]
+    bytes_["gate_topk_mask"] = 2 * idx_bytes  # fp32 scores in, int32 mask out
     dc_bytes = bytes_["dispatch"] + bytes_["combine"]
     dc_us = us["dispatch"] + us["combine"]
     value = dc_bytes / dc_us / 1e3  # GB/s

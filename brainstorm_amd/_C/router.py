@@ -19,6 +19,7 @@ from brainstorm_amd import _lib
 _DT = {torch.float32: _lib.F32, torch.float16: _lib.F16, torch.bfloat16: _lib.BF16}
 
 __all__ = [
+    "topk_hot_mask",
     "throttle_hotmask",
     "generate_indices_and_loads",
     "convert_index_format",
@@ -104,6 +105,27 @@ def _paired_counts(route_indices: torch.Tensor, loads: torch.Tensor) -> Optional
 
 
 # ------------------------------------------------------------------------- ops
+def topk_hot_mask(score: torch.Tensor, top_k: int) -> torch.Tensor:
+    """Not in the reference's extension: the hot mask of ``TopKProtocol``
+    (protocol/topk.py:26-31: ``topk`` + ``zeros_like`` + ``scatter_``) in one kernel.  int32
+    ``[cells, paths]`` with ones at the ``top_k`` largest scores of every row; NaN ranks
+    highest, equal scores go to the lowest path."""
+    _check_on_device(score, "score")
+    if score.dim() != 2:
+        raise RuntimeError("score must be [cells, paths]")
+    if score.dtype not in _DT:
+        raise NotImplementedError("score data type is not supported")
+    T, E = score.shape
+    if not 0 <= top_k <= E:
+        raise RuntimeError("selected index k out of range")  # the message torch.topk gives
+    score = score.contiguous()
+    with torch.cuda.device(score.device):
+        mask = torch.empty((T, E), dtype=torch.int32, device=score.device)
+        _lib.check(_lib.lib().brt_hip_topk_hot_mask(
+            _ptr(score), _ptr(mask), T, E, int(top_k), _DT[score.dtype], _stream()))
+    return mask
+
+
 def throttle_hotmask(
     hot_mask: torch.Tensor, prefix: torch.Tensor, threshold: torch.Tensor
 ) -> Tuple[torch.Tensor, torch.Tensor]:

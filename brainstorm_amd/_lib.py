@@ -54,6 +54,10 @@ SIGNATURES = {
         _c_int,
         [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     ),
+    "brt_hip_topk_hot_mask": (
+        _c_int,
+        [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    ),
     "brt_hip_grouped_gemm": (
         _c_int,
         [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],

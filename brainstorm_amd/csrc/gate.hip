@@ -1,0 +1,151 @@
+// Gate front-end: scores -> int32 hot mask with ones at the k largest scores of every row.
+//
+// Replaces the three torch launches of the reference's TopKProtocol
+// (python/brt/router/protocol/topk.py:26-31: torch.topk, zeros_like, scatter_) with one pass
+// that reads the scores once and writes the mask once.  Order of torch.topk: NaN above every
+// number; among equal scores (which torch leaves unspecified) the lowest column wins.
+//
+// Lanes are columns.  Up to 64 columns: a wavefront takes 64/ep rows per step (ep = columns
+// rounded up to a power of two) and every selection is a butterfly max inside the row's lane
+// segment plus a ballot that picks the lowest lane holding the maximum.  More than 64 columns:
+// one row per step, every lane keeps the columns lane, lane+64, ... in registers.
+#include <algorithm>
+
+#include "common.hpp"
+
+namespace brt {
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kMaxPerLane = 16;  // columns per lane in the wide path: up to 1024 columns
+
+struct GateArgs {
+  const void* scores;
+  int* mask;
+  int T, E, k;
+  int ep_shift;  // log2 of the lane segment of a row (E <= 64)
+  int rows_pw;   // rows per wavefront
+};
+
+// Scores as unsigned keys whose order is torch.topk's: larger key = ranked higher, NaN on top.
+// 0 is below every real key and marks a column that is taken (or does not exist).
+__device__ __forceinline__ uint32_t score_key(float f) {
+  if (f != f) return 0xffffffffu;
+  const uint32_t u = f == 0.0f ? 0u : __float_as_uint(f);  // -0 and +0 are one score
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);       // never 0: ~u of a number is >= 0x007fffff
+}
+
+template <int DT>
+__device__ __forceinline__ float load_score(const void* p, size_t i) {
+  if (DT == BRT_F32) return static_cast<const float*>(p)[i];
+  return half_bits_to_float<DT>(static_cast<const uint16_t*>(p)[i]);
+}
+
+template <int DT>
+__global__ __launch_bounds__(kBlock) void topk_mask_kernel(GateArgs a) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const long wave = static_cast<long>(blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  const int ep = 1 << a.ep_shift, rps = kWave >> a.ep_shift;
+  const int e = lane & (ep - 1), sub = lane >> a.ep_shift;
+  const unsigned long long seg = (ep == kWave ? ~0ull : ((1ull << ep) - 1ull)) << (sub * ep);
+  const long t0 = wave * a.rows_pw;
+  const int nt = static_cast<int>(max(0l, min(static_cast<long>(a.rows_pw), a.T - t0)));
+  for (int r0 = 0; r0 < nt; r0 += rps) {
+    const int row = r0 + sub;
+    const bool live = row < nt && e < a.E;
+    uint32_t key = live ? score_key(load_score<DT>(a.scores, static_cast<size_t>(t0 + row) * a.E + e)) : 0u;
+    int taken = 0;
+    for (int pass = 0; pass < a.k; ++pass) {
+      uint32_t best = key;
+      for (int d = 1; d < ep; d <<= 1) best = max(best, static_cast<uint32_t>(__shfl_xor(static_cast<int>(best), d, kWave)));
+      const unsigned long long tied = __ballot(key == best && key != 0) & seg;
+      if (tied != 0 && lane == __builtin_ctzll(tied)) {
+        taken = 1;
+        key = 0;
+      }
+    }
+    if (live) a.mask[static_cast<size_t>(t0 + row) * a.E + e] = taken;
+  }
+}
+
+template <int DT>
+__global__ __launch_bounds__(kBlock) void topk_mask_wide_kernel(GateArgs a) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const long wave = static_cast<long>(blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  const long t0 = wave * a.rows_pw;
+  const int nt = static_cast<int>(max(0l, min(static_cast<long>(a.rows_pw), a.T - t0)));
+  const int per_lane = (a.E + kWave - 1) / kWave;
+  for (int row = 0; row < nt; ++row) {
+    const size_t base = static_cast<size_t>(t0 + row) * a.E;
+    uint32_t key[kMaxPerLane];
+    unsigned taken = 0;
+#pragma unroll
+    for (int c = 0; c < kMaxPerLane; ++c) {
+      const int col = c * kWave + lane;
+      key[c] = (c < per_lane && col < a.E) ? score_key(load_score<DT>(a.scores, base + col)) : 0u;
+    }
+    for (int pass = 0; pass < a.k; ++pass) {
+      uint32_t mine = 0;
+#pragma unroll
+      for (int c = 0; c < kMaxPerLane; ++c) mine = max(mine, key[c]);
+      uint32_t best = mine;
+      for (int d = 1; d < kWave; d <<= 1) best = max(best, static_cast<uint32_t>(__shfl_xor(static_cast<int>(best), d, kWave)));
+      // lowest column holding the maximum: lowest c first, then lowest lane
+      int my_c = kMaxPerLane;
+#pragma unroll
+      for (int c = kMaxPerLane - 1; c >= 0; --c)
+        if (key[c] == best && best != 0) my_c = c;
+      int low_c = my_c;
+      for (int d = 1; d < kWave; d <<= 1) low_c = min(low_c, __shfl_xor(low_c, d, kWave));
+      const unsigned long long tied = __ballot(my_c == low_c && my_c < kMaxPerLane);
+      if (tied != 0 && lane == __builtin_ctzll(tied)) {
+#pragma unroll
+        for (int c = 0; c < kMaxPerLane; ++c)
+          if (c == low_c) { key[c] = 0; taken |= 1u << c; }
+      }
+    }
+#pragma unroll
+    for (int c = 0; c < kMaxPerLane; ++c) {
+      const int col = c * kWave + lane;
+      if (c < per_lane && col < a.E) a.mask[base + col] = (taken >> c) & 1u;
+    }
+  }
+}
+
+}  // namespace
+}  // namespace brt
+
+using namespace brt;
+
+extern "C" int brt_hip_topk_hot_mask(const void* scores, int32_t* hot_mask, int T, int E, int k,
+                                     int dtype, void* stream) {
+  if (T < 0 || E <= 0 || k < 0 || k > E) return fail(BRT_E_INVALID, "bad shape T=%d E=%d k=%d", T, E, k);
+  if (dtype != BRT_F32 && dtype != BRT_F16 && dtype != BRT_BF16)
+    return fail(BRT_E_UNSUPPORTED, "dtype %d is not supported", dtype);
+  if (E > kWave * kMaxPerLane) return fail(BRT_E_UNSUPPORTED, "more than %d paths", kWave * kMaxPerLane);
+  if (static_cast<long>(T) * E >= (1l << 31)) return fail(BRT_E_UNSUPPORTED, "T*E >= 2^31");
+  if (T == 0) return BRT_OK;
+  if (!scores || !hot_mask) return fail(BRT_E_INVALID, "null argument");
+  GateArgs a{};
+  a.scores = scores; a.mask = hot_mask; a.T = T; a.E = E; a.k = k;
+  int shift = 0;
+  while ((1 << shift) < std::min(E, kWave)) ++shift;
+  a.ep_shift = shift;
+  const int rps = E <= kWave ? kWave >> shift : 1;
+  // enough wavefronts to cover the chip a few times over, whole steps per wavefront
+  long rows = std::max<long>(rps, (T + 8191) / 8192 * rps);
+  rows = std::min<long>(rows, 16l * rps);
+  a.rows_pw = static_cast<int>(rows);
+  const long n_waves = (T + a.rows_pw - 1) / a.rows_pw;
+  const int waves_pb = kBlock / kWave;
+  const dim3 grid(static_cast<unsigned>((n_waves + waves_pb - 1) / waves_pb)), block(kBlock);
+  hipStream_t st = as_stream(stream);
+#define BRT_GATE_LAUNCH(DT)                                                            \
+  if (E <= kWave) hipLaunchKernelGGL((topk_mask_kernel<DT>), grid, block, 0, st, a);   \
+  else hipLaunchKernelGGL((topk_mask_wide_kernel<DT>), grid, block, 0, st, a);
+  if (dtype == BRT_F32) { BRT_GATE_LAUNCH(BRT_F32) }
+  else if (dtype == BRT_F16) { BRT_GATE_LAUNCH(BRT_F16) }
+  else { BRT_GATE_LAUNCH(BRT_BF16) }
+#undef BRT_GATE_LAUNCH
+  return check_launch("topk_mask_kernel");
+}

@@ -388,8 +388,9 @@ int launch_act(GemmArgs& a, hipStream_t st) {
   const long grid = static_cast<long>(a.tiles_m_max) * a.tiles_n;
   static bool configured = false;
   if (!configured) {
-    hipFuncSetAttribute(reinterpret_cast<const void*>(&grouped_gemm_kernel<MT, NT, WAVES, ACT>),
-                        hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&grouped_gemm_kernel<MT, NT, WAVES, ACT>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)) != hipSuccess)
+      return fail(BRT_E_LAUNCH, "cannot reserve %zu bytes of LDS", lds);
     configured = true;
   }
   hipLaunchKernelGGL((grouped_gemm_kernel<MT, NT, WAVES, ACT>), dim3(static_cast<unsigned>(grid)),

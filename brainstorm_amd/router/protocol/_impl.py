@@ -74,6 +74,9 @@ class TopKProtocol(ProtocolBase):
         self.single_path = top_k == 1
 
     def make_route_decision(self, score):
+        if (score.is_cuda and score.dim() == 2 and score.shape[1] <= 1024
+                and score.dtype in (torch.float32, torch.float16, torch.bfloat16)):
+            return c_router.topk_hot_mask(score, self.top_k)  # one kernel instead of three
         return _one_hot_int32(torch.topk(score, self.top_k, dim=1).indices, score)
 
 

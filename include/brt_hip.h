@@ -165,6 +165,17 @@ int brt_hip_combine_by_tags(const void* src, void* dst, const int32_t* row_tags,
                             int T, int in_dtype, int out_dtype, void* stream);
 
 /*
+ * Gate front-end (the three torch launches of TopKProtocol.make_route_decision,
+ * python/brt/router/protocol/topk.py:26-31: topk, zeros_like, scatter_, in one pass):
+ *   hot_mask[t,e] = 1 if scores[t,e] is among the k largest of row t, else 0.
+ *   scores [T,E] in `dtype`, hot_mask [T,E] int32 (every element is written).
+ *   NaN ranks above every number (torch.topk); among equal scores the lowest
+ *   column wins (torch leaves that choice unspecified).  0 <= k <= E <= 1024.
+ */
+int brt_hip_topk_hot_mask(const void* scores, int32_t* hot_mask, int T, int E, int k, int dtype,
+                          void* stream);
+
+/*
  * Replaces the homo-fused expert kernel launch jit::CUDACompiler::HomoExecute
  * (src/jit/compiler.cu:151-246, binding src/backend/torch/jit.cc:54-75) for
  * Linear branches (python/brt/jit/modules/linear.py:15-61):

@@ -108,6 +108,17 @@ def throttle_hotmask(mask, prefix, threshold) -> Tuple[np.ndarray, np.ndarray]:
     return out, prefix
 
 
+def topk_hot_mask(score, k: int) -> np.ndarray:
+    """``TopKProtocol.make_route_decision`` (protocol/topk.py:26-31): int32 mask with ones at
+    the k largest scores of every row (NaN counts as largest, ties go to the lowest column)."""
+    score = np.ascontiguousarray(score, dtype=np.float32)
+    T, E = score.shape
+    assert 0 <= k <= E
+    mask = np.zeros((T, E), dtype=np.int32)
+    lib().oracle_topk_hot_mask(_p(score), _p(mask), T, E, int(k))
+    return mask
+
+
 def convert_index_format(indices, loads, tag_to_seat: bool) -> np.ndarray:
     """Permutation inversion between seat and tag formats (location.cu:259-333).
 

@@ -9,6 +9,7 @@
  *   src/router/route.cu      dispatch_with_{seat,tag}_indices_{1d,2d},
  *                            combine_with_seat_indices, init_with_seat_indices
  *   src/backend/torch/router.cc   shape/dtype conventions around them
+ *   python/brt/router/protocol/topk.py:26-31   top-k hot mask (torch.topk + scatter_)
  *
  * Only tests, the smoke check and the bench's cpu_baseline leg may link or call
  * this file; the product path never does.
@@ -367,5 +368,34 @@ void oracle_combine(const void* src, void* dst, const void* gates, const int32_t
       if (any || !is_residual) store_elem(dst, out_dtype, (size_t)t * cell + j, acc);
     }
     (void)routed;
+  }
+}
+
+
+/* ---------- gate front-end: top-k hot mask ----------
+ * python/brt/router/protocol/topk.py:26-31:
+ *   hot_mask = zeros_like(score, int32).scatter_(1, topk(score, k, dim=1).indices, 1)
+ * torch.topk orders NaN above every number; which of several equal scores it returns is
+ * not specified, here the lowest column wins.  Scores arrive as fp32 (16-bit inputs are
+ * widened exactly by the caller).  Selection by k passes of "largest remaining". */
+static int score_greater(float a, float b) { /* a strictly above b in topk's order */
+  const int a_nan = a != a, b_nan = b != b;
+  if (a_nan || b_nan) return a_nan && !b_nan;
+  return a > b;
+}
+
+void oracle_topk_hot_mask(const float* score, int32_t* mask, int T, int E, int k) {
+  for (int t = 0; t < T; ++t) {
+    const float* row = score + (size_t)t * E;
+    int32_t* out = mask + (size_t)t * E;
+    for (int e = 0; e < E; ++e) out[e] = 0;
+    for (int pass = 0; pass < k && pass < E; ++pass) {
+      int best = -1;
+      for (int e = 0; e < E; ++e) {
+        if (out[e]) continue;
+        if (best < 0 || score_greater(row[e], row[best])) best = e;
+      }
+      out[best] = 1;
+    }
   }
 }

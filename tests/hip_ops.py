@@ -175,3 +175,13 @@ def combine_by_tags(y_bits, row_tags, residual_bits, in_dtype="f32", out_dtype=N
         ptr(d_y), ptr(d_out), ptr(d_tags), P, cell, T, DT[in_dtype], DT[out_dtype], stream()))
     torch.cuda.synchronize()
     return host(d_out, True)
+
+
+def topk_hot_mask(score_bits, k, dtype="f32"):
+    score_bits = np.ascontiguousarray(score_bits)
+    T, E = score_bits.shape
+    d_s = dev(score_bits)
+    d_m = torch.full((T, E), -7, dtype=torch.int32, device="cuda")
+    _lib.check(_lib.lib().brt_hip_topk_hot_mask(ptr(d_s), ptr(d_m), T, E, k, DT[dtype], stream()))
+    torch.cuda.synchronize()
+    return host(d_m)

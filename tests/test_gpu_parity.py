@@ -274,6 +274,33 @@ def test_combine_max_path_padding_and_odd_rows(hip):
             assert same_bits(got, want)
 
 
+# ------------------------------------------------- gate front-end: top-k hot mask
+@pytest.mark.parametrize("T,E,k,dtype", [
+    (8192, 64, 1, "f32"), (16384, 32, 2, "f32"), (100352, 8, 1, "f16"), (1000, 5, 3, "bf16"),
+    (777, 64, 64, "f32"), (513, 100, 7, "f32"), (300, 128, 2, "bf16"), (40, 1000, 9, "f32"),
+    (7, 1, 1, "f32"), (9, 16, 0, "f32"),
+])
+def test_topk_hot_mask_bit_exact(hip, T, E, k, dtype):
+    rng = np.random.default_rng(T + E + k)
+    score = rng.standard_normal((T, E)).astype(np.float32)
+    bits = as_dtype_bits(score, dtype)                        # 16-bit inputs produce many ties
+    want = oracle.topk_hot_mask(bits_to_f32(bits, dtype), k)
+    got = hip.topk_hot_mask(bits, k, dtype)
+    assert np.array_equal(got, want)
+    assert (got.sum(1) == k).all()
+
+
+def test_topk_hot_mask_special_values(hip):
+    score = np.array([[1.0, 1.0, 1.0, 1.0], [0.0, -0.0, 0.0, -1.0],
+                      [np.nan, 5.0, np.inf, -np.inf], [-np.inf, -np.inf, np.nan, np.nan]], dtype=np.float32)
+    for k in range(5):
+        assert np.array_equal(hip.topk_hot_mask(score, k), oracle.topk_hot_mask(score, k)), k
+    wide = np.zeros((3, 200), dtype=np.float32)                # all equal: the first k columns
+    assert np.array_equal(hip.topk_hot_mask(wide, 70), oracle.topk_hot_mask(wide, 70))
+    with pytest.raises(RuntimeError):
+        hip.topk_hot_mask(score, 5)
+
+
 # ------------------------------------------------- tag-driven combine (single-path routes)
 @pytest.mark.parametrize("T,E,cell,in_dtype,out_dtype", [
     (1024, 16, 512, "f32", "f32"),

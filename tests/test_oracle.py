@@ -432,3 +432,45 @@ def test_combine_max_path_padding():
     y, _ = oracle.dispatch(x, idx, loads, max_path_padding=True, max_path_load=200)
     assert y.shape[0] == 800
     assert np.array_equal(oracle.combine(y, idx, loads, max_path_padding=True), x)
+
+
+# ------------------------------------------------------------------ top-k hot mask
+def _topk_mask_by_stable_sort(score, k):
+    """Independent statement: stable sort of the columns by descending score (NaN first)."""
+    key = np.where(np.isnan(score), np.inf, score)
+    mask = np.zeros(score.shape, dtype=np.int32)
+    for t in range(score.shape[0]):  # NaN ahead of +inf, then by value, then by column
+        cols = sorted(range(score.shape[1]),
+                      key=lambda e: (0 if np.isnan(score[t, e]) else 1, -key[t, e], e))
+        mask[t, cols[:k]] = 1
+    return mask
+
+
+@pytest.mark.parametrize("T,E,k", [(64, 4, 1), (200, 16, 2), (50, 64, 4), (33, 100, 7), (10, 8, 8), (5, 3, 0)])
+def test_topk_hot_mask_matches_torch_topk_and_a_stable_sort(T, E, k):
+    import torch
+
+    rng = np.random.default_rng(T * E + k)
+    score = rng.standard_normal((T, E)).astype(np.float32)   # no ties: torch's choice is defined
+    got = oracle.topk_hot_mask(score, k)
+    want = torch.zeros(T, E, dtype=torch.int32)
+    if k:
+        want.scatter_(1, torch.topk(torch.from_numpy(score), k, dim=1).indices, 1)  # topk.py:26-31
+    assert np.array_equal(got, want.numpy())
+    assert np.array_equal(got, _topk_mask_by_stable_sort(score, k))
+    assert (got.sum(1) == k).all()
+
+
+def test_topk_hot_mask_ties_nan_and_infinities():
+    import torch
+
+    score = np.array([[1.0, 1.0, 1.0, 1.0],                       # ties: lowest columns
+                      [0.0, -0.0, 0.0, -1.0],                     # -0 and +0 are one score
+                      [np.nan, 5.0, np.inf, -np.inf],             # NaN above +inf (torch.topk order)
+                      [-np.inf, -np.inf, np.nan, np.nan]], dtype=np.float32)
+    got = oracle.topk_hot_mask(score, 2)
+    assert got.tolist() == [[1, 1, 0, 0], [1, 1, 0, 0], [1, 0, 1, 0], [0, 0, 1, 1]]
+    assert np.array_equal(got, _topk_mask_by_stable_sort(score, 2))
+    # torch agrees wherever its answer is defined (rows without ties among the selected)
+    picked = torch.topk(torch.from_numpy(score[2:]), 2, dim=1).indices
+    assert sorted(picked[0].tolist()) == [0, 2] and sorted(picked[1].tolist()) == [2, 3]

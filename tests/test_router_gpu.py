@@ -208,6 +208,23 @@ def test_fused_moe_path_top2_keeps_the_gather_combine(brt_mod):
                           oracle.combine(o_y1, i1, l1, out_data=np.full((T, d), 3.0, dtype=np.float32)))
 
 
+def test_topk_protocol_uses_the_fused_mask_kernel(brt_mod):
+    """TopKProtocol (protocol/topk.py:26-31) gives the mask torch.topk + scatter_ gives."""
+    _, c_router, ScatterRouter, _ = brt_mod
+    from brt.router.protocol import make_protocol
+
+    score = torch.randn(3000, 24, device="cuda")
+    for k in (1, 3):
+        proto = make_protocol("topk", {"top_k": k})
+        mask = proto(score)
+        want = torch.zeros_like(score, dtype=torch.int32).scatter_(1, torch.topk(score, k, dim=1).indices, 1)
+        assert mask.dtype == torch.int32 and torch.equal(mask, want)
+        assert getattr(mask, "_brt_single_path", False) == (k == 1)
+    assert int(c_router.topk_hot_mask(score.half(), 2).sum()) == 2 * score.shape[0]
+    with pytest.raises(RuntimeError):
+        c_router.topk_hot_mask(score, 25)
+
+
 def test_shim_signatures_and_errors(brt_mod):
     _, c_router, _, _ = brt_mod
     mask, logits = topk_mask(300, 4, 2, seed=9)
