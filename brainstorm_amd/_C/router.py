@@ -48,7 +48,28 @@ def _ptr(t: Optional[torch.Tensor]):
 
 
 def _stream() -> int:
-    return torch.cuda.current_stream().cuda_stream
+    """Raw handle of the current stream of the current device (the ops run under a guard for
+    the tensors' device).  The private accessor avoids building a ``torch.cuda.Stream``."""
+    return torch._C._cuda_getCurrentRawStream(torch._C._cuda_getDevice())
+
+
+class _NoGuard:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_GUARD = _NoGuard()
+
+
+def _device_guard(device: torch.device):
+    """``CUDAGuard`` of the reference bindings (router.cc:55,144,384); free when the tensors
+    already live on the current device."""
+    if device.index is None or device.index == torch._C._cuda_getDevice():
+        return _NO_GUARD
+    return torch.cuda.device(device)
 
 
 _workspaces = {}
@@ -119,7 +140,7 @@ def topk_hot_mask(score: torch.Tensor, top_k: int) -> torch.Tensor:
     if not 0 <= top_k <= E:
         raise RuntimeError("selected index k out of range")  # the message torch.topk gives
     score = score.contiguous()
-    with torch.cuda.device(score.device):
+    with _device_guard(score.device):
         mask = torch.empty((T, E), dtype=torch.int32, device=score.device)
         _lib.check(_lib.lib().brt_hip_topk_hot_mask(
             _ptr(score), _ptr(mask), T, E, int(top_k), _DT[score.dtype], _stream()))
@@ -139,7 +160,7 @@ def throttle_hotmask(
         raise RuntimeError("prefix/threshold must have one entry per path")
     hot_mask = hot_mask.contiguous()
     T, E = hot_mask.shape
-    with torch.cuda.device(hot_mask.device):
+    with _device_guard(hot_mask.device):
         throttled = torch.empty_like(hot_mask)
         if T > 0:
             ws = _scan_workspace(hot_mask.device, T, E)
@@ -165,7 +186,7 @@ def generate_indices_and_loads(
     _check_on_device(hot_mask, "hot_mask")
     _check_int32(hot_mask, "hot_mask")
     T, E = hot_mask.size(0), hot_mask.size(1)
-    with torch.cuda.device(hot_mask.device):
+    with _device_guard(hot_mask.device):
         if hot_mask.numel() == 0:  # router.cc:59-62
             return (torch.zeros((0, E), dtype=hot_mask.dtype, device=hot_mask.device),
                     torch.zeros((E,), dtype=hot_mask.dtype, device=hot_mask.device))
@@ -220,7 +241,7 @@ def _convert(origin_indices, loads, tag_to_seat: bool) -> torch.Tensor:
     _check_int32(origin_indices, "origin_indices")
     origin_indices = origin_indices.contiguous()
     T, E = origin_indices.shape
-    with torch.cuda.device(origin_indices.device):
+    with _device_guard(origin_indices.device):
         dev_loads = loads
         if tag_to_seat:
             _check_int32(loads, "loads")
@@ -251,7 +272,7 @@ def dispatch_with_indices_and_loads(
     device = in_data.device
     T = in_data.size(0)
     E = route_indices.size(1)
-    with torch.cuda.device(device):
+    with _device_guard(device):
         if T == 0:  # router.cc:150-168
             shape = list(in_data.shape)
             if is_1d_routing:
@@ -416,7 +437,7 @@ def combine_with_indices_and_loads(
     _check_on_device(route_indices, "route_indices")
     device = in_data.device
     T = route_indices.size(0)
-    with torch.cuda.device(device):
+    with _device_guard(device):
         if T == 0:  # router.cc:386-397
             if not is_tag_index:
                 return [out_data if out_data is not None else torch.empty_like(in_data)]

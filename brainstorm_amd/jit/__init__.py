@@ -84,7 +84,7 @@ def grouped_linear(x: torch.Tensor, out: torch.Tensor, weight_table: torch.Tenso
         raise RuntimeError("shared inputs must have the same number of rows")
     with torch.cuda.device(x.device):
         lib = _lib.lib()
-        stream = torch.cuda.current_stream().cuda_stream
+        stream = torch._C._cuda_getCurrentRawStream(torch._C._cuda_getDevice())
         bias_ptr = None if bias_table is None else bias_table.data_ptr()
         if routed:
             _lib.check(lib.brt_hip_grouped_gemm_routed(
