@@ -42,8 +42,8 @@ MEASURED_TRAFFIC_BYTES = {
     "dispatch": int((7207.5 * 1.996 + 12482.4) * 1024),
     "combine": int((6221.5 * 1.996 + 12288.0) * 1024),
     "combine_gather": int((7210.0 * 1.996 + 12288.0) * 1024),
-    "ffn_gemm1_gelu": int((155525.2 * 1.996 + 49152.0) * 1024),
-    "ffn_gemm2": int((177207.9 * 1.996 + 12288.0) * 1024),
+    "ffn_gemm1_gelu": int((155668.3 * 1.996 + 49152.0) * 1024),
+    "ffn_gemm2": int((172255.1 * 1.996 + 12288.0) * 1024),
 }
 
 T, D, E, DFF = 8192, 768, 64, 3072
