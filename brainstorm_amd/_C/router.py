@@ -200,8 +200,7 @@ def generate_indices_and_loads(
         if capacity_padding and n_caps < 1:  # CHECK_GE, location.cu:350,365
             raise RuntimeError("capacity_padding requires at least one supported capacity")
         hot_mask = hot_mask.contiguous()
-        # seat mode writes every element; the tag list is sparse and starts from zeros
-        indices = torch.zeros_like(hot_mask) if is_tag_index else torch.empty_like(hot_mask)
+        indices = torch.empty_like(hot_mask)  # the kernel writes every element in both formats
         loads_and_counts = torch.empty((2, E), dtype=torch.int32, device=hot_mask.device)
         loads, counts = loads_and_counts[0], loads_and_counts[1]
         ws = _scan_workspace(hot_mask.device, T, E)

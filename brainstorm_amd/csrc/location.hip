@@ -120,8 +120,8 @@ __device__ __forceinline__ int sum_over_rows_in_wave(int v, int ep_shift) {
 // lane's, tot = sum over all groups).
 template <int MODE>
 __device__ __forceinline__ void walk_batch(const int (&m)[kBatch], int i0, int n_ins, int& carry,
-                                           int thr, long row_w, int rps, int ep, int sub, int e,
-                                           int lane, int col, bool col_ok, const ScanArgs& a) {
+                                           int thr, int total, long row_w, int rps, int ep, int sub,
+                                           int e, int lane, int col, bool col_ok, const ScanArgs& a) {
   int incl[kBatch], tot[kBatch];
 #pragma unroll
   for (int u = 0; u < kBatch; ++u) {
@@ -151,6 +151,8 @@ __device__ __forceinline__ void walk_batch(const int (&m)[kBatch], int i0, int n
         const int index = run * m[u];
         if (index >= 1 && index <= a.T)
           a.out[static_cast<size_t>(index - 1) * a.E + col] = static_cast<int>(r) + 1;
+        // slots past the path's last tag are nobody's to write but this row's owner
+        if (r >= total) a.out[r * a.E + col] = 0;
       }
     }
   }
@@ -209,6 +211,7 @@ template <int MODE>
 __global__ __launch_bounds__(kBlock) void band_apply_kernel(ScanArgs a) {
   __shared__ int s_above[kWavesPB][kWave];  // each wave's share of the sum over earlier bands
   __shared__ int s_own[kWavesPB][kWave];    // column sums of each wave's own rows
+  __shared__ int s_below[kWavesPB][kWave];  // tag mode: share of the sum over later bands
   const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
   const int E = a.E, band = blockIdx.x;
   const int ep = 1 << a.ep_shift, rps = kWave >> a.ep_shift;
@@ -223,7 +226,7 @@ __global__ __launch_bounds__(kBlock) void band_apply_kernel(ScanArgs a) {
     int m0[kBatch];
     load_batch(m0, 0, n_ins, row_w, rps, sub, col, col_ok, a);
     // ---- this wave's share of the offset: bands wave, wave+4, ... above this one ----
-    int above = 0;
+    int above = 0, below = 0;
     for (int j0 = wave + sub * kWavesPB; j0 < band; j0 += kWavesPB * rps * kPartialBatch) {
       int v[kPartialBatch];
 #pragma unroll
@@ -233,6 +236,19 @@ __global__ __launch_bounds__(kBlock) void band_apply_kernel(ScanArgs a) {
       }
 #pragma unroll
       for (int u = 0; u < kPartialBatch; ++u) above += v[u];
+    }
+    if (MODE == kTag) {  // the tag list of a path ends at its total: the later bands count too
+      for (int j0 = band + 1 + wave + sub * kWavesPB; j0 < a.bands; j0 += kWavesPB * rps * kPartialBatch) {
+        int v[kPartialBatch];
+#pragma unroll
+        for (int u = 0; u < kPartialBatch; ++u) {
+          const int j = j0 + u * kWavesPB * rps;
+          v[u] = (j < a.bands && col_ok) ? a.partial[static_cast<size_t>(j) * E + col] : 0;
+        }
+#pragma unroll
+        for (int u = 0; u < kPartialBatch; ++u) below += v[u];
+      }
+      below = sum_over_rows_in_wave(below, a.ep_shift);
     }
     int own = 0;
 #pragma unroll
@@ -249,14 +265,16 @@ __global__ __launch_bounds__(kBlock) void band_apply_kernel(ScanArgs a) {
     if (sub == 0) {
       s_above[wave][e] = above;
       s_own[wave][e] = own;
+      if (MODE == kTag) s_below[wave][e] = below;
     }
     __syncthreads();
-    int carry = 0, band_total = 0;
+    int carry = 0, band_total = 0, later = 0;
 #pragma unroll
     for (int k = 0; k < kWavesPB; ++k) {
       carry += s_above[k][e];
       band_total += s_own[k][e];
       if (k < wave) carry += s_own[k][e];
+      if (MODE == kTag) later += s_below[k][e];
     }
     band_total += carry;
 #pragma unroll
@@ -270,11 +288,12 @@ __global__ __launch_bounds__(kBlock) void band_apply_kernel(ScanArgs a) {
     }
 
     // ---- walk the rows again: running sum per path, one result per element ----------
-    walk_batch<MODE>(m0, 0, n_ins, carry, thr, row_w, rps, ep, sub, e, lane, col, col_ok, a);
+    const int total = band_total + later;  // tag mode: entries of this path's list
+    walk_batch<MODE>(m0, 0, n_ins, carry, thr, total, row_w, rps, ep, sub, e, lane, col, col_ok, a);
     for (int i0 = kBatch; i0 < n_ins; i0 += kBatch) {
       int v[kBatch];
       load_batch(v, i0, n_ins, row_w, rps, sub, col, col_ok, a);
-      walk_batch<MODE>(v, i0, n_ins, carry, thr, row_w, rps, ep, sub, e, lane, col, col_ok, a);
+      walk_batch<MODE>(v, i0, n_ins, carry, thr, total, row_w, rps, ep, sub, e, lane, col, col_ok, a);
     }
 
     // ---- totals: loads / counts / throttle prefix (last band only) ---------------------

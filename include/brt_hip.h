@@ -58,10 +58,10 @@ size_t brt_hip_scan_workspace_bytes(int T, int E);
  * src/router/location.cu:212-257,335-379).
  *
  *   mask     [T,E] int32 hot mask
- *   indices  [T,E] int32 out.  Seat mode (is_tag_index=0): every element is
- *            written (cumsum(mask,0)*mask), no pre-zeroing needed.  Tag mode:
- *            must be zero-filled by the caller; slot [s-1,e] receives row+1 of
- *            the s-th routed row of column e.
+ *   indices  [T,E] int32 out; every element is written, no pre-zeroing needed.
+ *            Seat mode (is_tag_index=0): cumsum(mask,0)*mask.  Tag mode: slot
+ *            [s-1,e] receives row+1 of the s-th routed row of column e, the
+ *            slots past a column's last tag receive 0.
  *   loads    [E] int32 out, after the capacity rules of location.cu:222-256
  *   counts   [E] int32 out or NULL: the un-clipped, un-padded per-path counts
  *            (sum(mask,0)); brt_hip_dispatch uses them to zero-fill padding rows

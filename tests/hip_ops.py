@@ -60,13 +60,10 @@ def generate_indices_and_loads(mask, caps=None, capacity_padding=False, path_wis
         d_mask.copy_(torch.from_numpy(mask))
         obuf = torch.full((T * E + 1,), -7, dtype=torch.int32, device="cuda")
         d_idx = obuf[1:].view(T, E)
-        if is_tag_index:
-            d_idx.zero_()
     else:
         d_mask = dev(mask)
-        d_idx = (torch.zeros if is_tag_index else torch.empty)((T, E), dtype=torch.int32, device="cuda")
-        if not is_tag_index:
-            d_idx.fill_(-7)  # poison: seat mode must overwrite everything
+        # poison: both index formats must overwrite every element
+        d_idx = torch.full((T, E), -7, dtype=torch.int32, device="cuda")
     d_loads = torch.full((E,), -1, dtype=torch.int32, device="cuda")
     d_counts = torch.full((E,), -1, dtype=torch.int32, device="cuda") if want_counts else None
     d_caps = None if caps is None else dev(np.asarray(caps, dtype=np.int32))
