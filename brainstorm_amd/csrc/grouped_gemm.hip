@@ -386,12 +386,15 @@ int launch_act(GemmArgs& a, hipStream_t st) {
   // sum over experts of ceil(M_e/BM) never exceeds P/BM + E; rounded up to whole XCD rounds
   a.tiles_m_max = ((a.P + BM - 1) / BM + a.E + kXcds - 1) / kXcds * kXcds;
   const long grid = static_cast<long>(a.tiles_m_max) * a.tiles_n;
-  static bool configured = false;
-  if (!configured) {
+  // more than 64 KB of dynamic LDS has to be allowed once per device and kernel
+  static bool configured[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 63;
+  if (!configured[dev] || dev == 63) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(&grouped_gemm_kernel<MT, NT, WAVES, ACT>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)) != hipSuccess)
       return fail(BRT_E_LAUNCH, "cannot reserve %zu bytes of LDS", lds);
-    configured = true;
+    configured[dev] = true;
   }
   hipLaunchKernelGGL((grouped_gemm_kernel<MT, NT, WAVES, ACT>), dim3(static_cast<unsigned>(grid)),
                      dim3(WAVES * 64), lds, st, a);

@@ -185,3 +185,39 @@ def test_routed_gemm_argument_checks():
     with pytest.raises(RuntimeError):
         grouped_linear(x[:4], out, table, None, loads, 64, 64, tags=tags, gather=True)  # x not cell-major
     grouped_linear(x, out, table, None, loads, 64, 64, tags=tags, gather=True, scatter=True)
+
+
+def test_full_size_switch_layer_fused_equals_unfused():
+    """The benchmark layer (8192 x 768 bf16, 64 experts, capacity 160, 768 -> 3072 -> 768):
+    the three-launch form (tag indices, gathering GEMM, scattering GEMM) against the five-launch
+    form, bit for bit, with and without capacity padding."""
+    from brainstorm_amd._C import router as c_router
+    from brainstorm_amd.jit import grouped_linear
+
+    T, E, d, dff, cap = 8192, 64, 768, 3072, 160
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(T, d, generator=g).to(torch.bfloat16).cuda()
+    score = torch.randn(T, E, generator=g).cuda()
+    mask = c_router.topk_hot_mask(score, 1)
+    caps = torch.tensor([cap], dtype=torch.int32, device="cuda")
+    w1, t1 = _expert_tables(E, d, dff, 11)
+    w2, t2 = _expert_tables(E, dff, d, 12)
+    for pad in (False, True):
+        idx, loads = c_router.generate_indices_and_loads(mask, caps, pad, single_path=True)
+        (y,) = c_router.dispatch_with_indices_and_loads(x, idx, loads)
+        P = y.shape[0]
+        h = torch.empty(P, dff, dtype=torch.bfloat16, device="cuda")
+        y2 = torch.empty(P, d, dtype=torch.bfloat16, device="cuda")
+        grouped_linear(y, h, t1, None, loads, d, dff, "gelu")
+        grouped_linear(h, y2, t2, None, loads, dff, d)
+        (want,) = c_router.combine_with_indices_and_loads(y2, idx, loads, None, x.clone())
+        tags, _ = c_router.generate_indices_and_loads(mask, caps, pad, False, True)
+        hf = torch.empty(P, dff, dtype=torch.bfloat16, device="cuda")
+        out = x.clone()
+        grouped_linear(x, hf, t1, None, loads, d, dff, "gelu", tags=tags, gather=True, rows=P)
+        grouped_linear(hf, out, t2, None, loads, dff, d, tags=tags, scatter=True, rows=P)
+        assert torch.equal(out.view(torch.int16), want.view(torch.int16)), pad
+        # linearity of the second GEMM (no activation): doubling its input doubles its output
+        y4 = torch.empty_like(y2)
+        grouped_linear((h.float() * 2).to(torch.bfloat16), y4, t2, None, loads, dff, d)
+        assert torch.equal(y4.float(), (y2.float() * 2).to(torch.bfloat16).float())
