@@ -189,7 +189,8 @@ int brt_hip_topk_hot_mask(const void* scores, int32_t* hot_mask, int T, int E, i
  *   read on the device (no host copy, any non-negative values, sum <= P).
  *   One launch covers all experts; accumulation is fp32 on the bf16 MFMA units.
  *   K and N must be multiples of 8 (16-byte rows; BRT_E_UNSUPPORTED otherwise), x and out
- *   16-byte aligned.  `act` is one of BRT_ACT_*; GELU is the erf form.
+ *   16-byte aligned.  `act` is one of BRT_ACT_*; GELU is the erf form
+ *   (v * Phi(v), to 4.3e-6 absolute before the rounding to bf16).
  */
 int brt_hip_grouped_gemm(const void* x, const void* const* weights, const void* const* biases,
                          void* out, const int32_t* loads, int E, int P, int K, int N, int act,

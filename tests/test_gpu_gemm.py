@@ -221,3 +221,50 @@ def test_full_size_switch_layer_fused_equals_unfused():
         y4 = torch.empty_like(y2)
         grouped_linear((h.float() * 2).to(torch.bfloat16), y4, t2, None, loads, dff, d)
         assert torch.equal(y4.float(), (y2.float() * 2).to(torch.bfloat16).float())
+
+
+def test_gelu_epilogue_on_every_bf16_value():
+    """The GELU epilogue on its own: an identity weight matrix carries every finite bf16 value to the
+    epilogue unchanged, so the output is GELU of that value rounded to bf16.  torch's erf GELU in
+    fp64, rounded to bf16, is the reference (in fp32 its 1 + erf cancels below -4 and is itself off
+    by more than a bf16 step); the two may round a value that sits next to a bf16 tie differently, so
+    the bar is one bf16 step, with all but a small fraction identical.  Infinite
+    pre-activations arrive through the bias (an infinite operand times a zero weight would be NaN)."""
+    from brainstorm_amd import _lib
+
+    bits = torch.arange(0, 1 << 16, dtype=torch.int32)
+    vals = bits.to(torch.int16).view(torch.bfloat16)
+    keep = torch.isfinite(vals.float()) & ((vals.float().abs() >= 1e-30) | (vals.float() == 0))
+    vals = vals[keep]
+    K = N = 64
+    rows = (vals.numel() + K - 1) // K
+    x = torch.zeros(rows * K, dtype=torch.bfloat16)
+    x[:vals.numel()] = vals
+    x = x.view(rows, K).cuda()
+    w = torch.eye(K, dtype=torch.bfloat16, device="cuda")
+    bias = torch.zeros(N, dtype=torch.bfloat16, device="cuda")
+    bias[3], bias[5] = float("inf"), float("-inf")
+    out = torch.full((rows, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    wt = torch.tensor([w.data_ptr()], dtype=torch.int64, device="cuda")
+    bt = torch.tensor([bias.data_ptr()], dtype=torch.int64, device="cuda")
+    loads = torch.tensor([rows], dtype=torch.int32, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def launch(bias_table):
+        _lib.check(_lib.lib().brt_hip_grouped_gemm(
+            x.data_ptr(), wt.data_ptr(), bias_table, out.data_ptr(), loads.data_ptr(),
+            1, rows, K, N, ACT["gelu"], stream))
+        torch.cuda.synchronize()
+
+    launch(None)
+    got = out.float().flatten()[:vals.numel()].cpu()
+    want = torch.nn.functional.gelu(vals.double()).to(torch.bfloat16).float()
+    assert torch.isfinite(got).all()
+    step = torch.maximum(want.abs(), torch.tensor(2.0 ** -126)) * 2.0 ** -7  # one bf16 step at `want`
+    tiny = want.abs() < 1e-12            # below -7 or so: both are rounding noise next to zero
+    off = ((got - want).abs() > step) & ~tiny
+    assert not off.any(), (vals[off][:8], got[off][:8], want[off][:8])
+    assert (got[tiny].abs() < 1e-11).all()
+    assert (got != want)[~tiny].float().mean() < 0.02
+    launch(bt.data_ptr())
+    assert (out[:, 3].float() == float("inf")).all() and (out[:, 5].float() == 0).all()
