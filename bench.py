@@ -301,15 +301,81 @@ def main():
     if not torch.equal(gate_mask, mask):
         sys.exit("bench.py: the gate kernel does not reproduce the argmax mask")
 
+    # the library's batched GEMM on the same FFN, every expert padded to the full capacity (the
+    # only shape a batched routine takes), GELU as its own elementwise launch: reported beside
+    # the grouped kernel, not part of the step
+    xb = torch.randn(E, CAPACITY, D, device=dev).to(torch.bfloat16)
+    hb = torch.empty(E, CAPACITY, DFF, dtype=torch.bfloat16, device=dev)
+    yb = torch.empty(E, CAPACITY, D, dtype=torch.bfloat16, device=dev)
+
+    def k_bmm1():
+        torch.bmm(xb, wi.transpose(1, 2), out=hb)
+
+    def k_bmm_gelu():
+        torch.nn.functional.gelu(hb)
+
+    def k_bmm2():
+        torch.bmm(hb, wo.transpose(1, 2), out=yb)
+
+    # generic tag-index gather (the default gather path of the reference: unique over the row
+    # tags, then a sum of the rows that carry the same tag) on this step's rows and tags,
+    # beside the library calls the reference makes for it; reported only, not part of the step
+    n_unique_d = torch.empty(1, dtype=torch.int32, device=dev)
+    uniq = torch.empty(P, dtype=torch.int32, device=dev)
+    inverse = torch.empty(P, dtype=torch.int64, device=dev)
+    ws_u = torch.empty(L.brt_hip_unique_tags_workspace_bytes(0, T), dtype=torch.uint8, device=dev)
+    ws_s = torch.empty(L.brt_hip_combine_by_index_workspace_bytes(P, T), dtype=torch.uint8, device=dev)
+    gathered = torch.empty(P, D, dtype=torch.bfloat16, device=dev)
+
+    def k_tag_unique():
+        _lib.check(L.brt_hip_unique_tags(row_tags.data_ptr(), 32, P, 0, T, ws_u.data_ptr(),
+                                         ws_u.numel(), uniq.data_ptr(), inverse.data_ptr(),
+                                         n_unique_d.data_ptr(), sptr()))
+
+    def k_tag_sum():
+        _lib.check(L.brt_hip_combine_by_index(
+            combine_src.data_ptr(), gathered.data_ptr(), inverse.data_ptr(), 64, P, D, P,
+            ws_s.data_ptr(), ws_s.numel(), _lib.BF16, _lib.BF16, sptr()))
+
+    def k_tag_sum_torch():   # router.cc:451,459-460
+        torch.zeros(P, D, dtype=torch.bfloat16, device=dev).scatter_reduce(
+            0, inverse.view(-1, 1).repeat(1, D), combine_src, "sum")
+
+    with torch.cuda.stream(stream):
+        k_tag_unique()
+        k_tag_sum()
+        t_u, t_i = torch.unique(row_tags, sorted=True, return_inverse=True)
+    stream.synchronize()
+    n_u = int(n_unique_d.item())
+    if n_u != t_u.numel() or not torch.equal(uniq[:n_u], t_u) or not torch.equal(inverse, t_i):
+        sys.exit("bench.py: the tag unique kernels disagree with torch.unique")
+    # every tag is carried by one row here, so the sum is the rows in tag order
+    if not torch.equal(gathered[inverse].view(torch.int16), combine_src.view(torch.int16)):
+        sys.exit("bench.py: the tag-index sum does not reproduce the rows")
+    with torch.cuda.stream(stream):      # torch.unique synchronises: timed eagerly
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        for _ in range(3):
+            torch.unique(row_tags, sorted=True, return_inverse=True)
+        e0.record(stream)
+        for _ in range(20):
+            torch.unique(row_tags, sorted=True, return_inverse=True)
+        e1.record(stream)
+    stream.synchronize()
+    unique_torch_us = e0.elapsed_time(e1) * 1e3 / 20
+
     # ---------------------------------------- per-kernel durations (same process)
     INNER = 20
     kernels = {"indexgen": k_indexgen, "dispatch": k_dispatch, "combine": k_combine,
                "combine_gather": k_combine_gather, "gate_topk_mask": k_gate,
-               "gate_topk_mask_torch_ops": k_gate_torch}
+               "gate_topk_mask_torch_ops": k_gate_torch,
+               "tag_gather_unique": k_tag_unique, "tag_gather_sum": k_tag_sum,
+               "tag_gather_sum_torch_ops": k_tag_sum_torch}
     if have_ffn:
         kernels.update({"ffn_gemm1_gelu": k_gemm1, "ffn_gemm2": k_gemm2,
                         "indexgen_tags": k_indexgen_tags, "ffn_gemm1_gelu_gather": k_gemm1_gather,
-                        "ffn_gemm2_scatter": k_gemm2_scatter})
+                        "ffn_gemm2_scatter": k_gemm2_scatter,
+                        "ffn_gemm1_library_bmm": k_bmm1, "ffn_gelu_library": k_bmm_gelu,
+                        "ffn_gemm2_library_bmm": k_bmm2})
     replays = max(10, args.steps // 4)
     us = {}
     for name, fn in kernels.items():
@@ -318,6 +384,7 @@ def main():
         runs = [timed(gk, replays) for _ in range(3)]
         us[name] = sum(runs) / len(runs) * 1e3 / (replays * INNER)  # average launch duration
 
+    us["tag_gather_unique_torch_op_eager"] = unique_torch_us
     es = 2  # bf16
     idx_bytes = 4 * T * E
     bytes_ = {

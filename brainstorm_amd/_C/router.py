@@ -407,9 +407,34 @@ def fuse_split_cells_from_paths(
         if tags is None:
             raise RuntimeError("is_tag_fuse needs tags")
         out_tags = torch.cat(tags, 0)
-        new_tags, global_seat_indices = torch.unique(out_tags, sorted=True, return_inverse=True)
+        new_tags, global_seat_indices = _unique_tags(out_tags)
         return [out_data, new_tags, global_seat_indices]
     return [out_data]
+
+
+def _unique_tags(tags: torch.Tensor):
+    """``torch.unique(tags, sorted=True, return_inverse=True)`` (router.cc:362-366) without the
+    sort: tags are cell numbers, so a presence table over ``[min, max]`` and one prefix sum give
+    the same two tensors.  Tag sets that are sparse in their range (or not a 1-d int32 / int64
+    device vector) take the library call."""
+    n = tags.numel()
+    if not (tags.is_cuda and tags.dim() == 1 and n > 0 and tags.dtype in (torch.int32, torch.int64)):
+        return torch.unique(tags, sorted=True, return_inverse=True)
+    with _device_guard(tags.device):
+        tags = tags.contiguous()
+        lo, hi = (int(v) for v in torch.stack(torch.aminmax(tags)).tolist())
+        span = hi - lo + 1
+        ws_bytes = _lib.lib().brt_hip_unique_tags_workspace_bytes(lo, hi)
+        if ws_bytes == 0 or span > 16 * n + (1 << 16):
+            return torch.unique(tags, sorted=True, return_inverse=True)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=tags.device)
+        unique = torch.empty(min(n, span), dtype=tags.dtype, device=tags.device)
+        inverse = torch.empty(n, dtype=torch.int64, device=tags.device)
+        count = torch.empty(1, dtype=torch.int32, device=tags.device)
+        _lib.check(_lib.lib().brt_hip_unique_tags(
+            _ptr(tags), 32 if tags.dtype == torch.int32 else 64, n, lo, hi, _ptr(ws), ws_bytes,
+            _ptr(unique), _ptr(inverse), _ptr(count), _stream()))
+        return unique[:int(count.item())], inverse
 
 
 def combine_with_indices_and_loads(
@@ -506,8 +531,6 @@ def _combine_with_tags(in_data, route_indices, out_data, ever_padded, tags):
     # router.cc:449-472
     if tags is None:
         raise RuntimeError("tag-index combine needs tags")
-    cell = in_data.numel() // in_data.size(0)
-    index = route_indices.view(-1, 1).repeat(1, cell).view_as(in_data)
     tags_value = tags
     n = tags_value.size(0)
     if out_data is not None:
@@ -516,17 +539,41 @@ def _combine_with_tags(in_data, route_indices, out_data, ever_padded, tags):
             raise RuntimeError("out_data must hold one row per unique tag")
         result = out_data
         # out-of-place and discarded, as in the reference (router.cc:456)
+        cell = in_data.numel() // in_data.size(0)
+        index = route_indices.view(-1, 1).repeat(1, cell).view_as(in_data)
         torch.scatter_reduce(result, 0, index, in_data, "sum", include_self=False)
     else:
         shape = list(in_data.shape)
         shape[0] = n
-        result = torch.zeros(shape, dtype=in_data.dtype, device=in_data.device)
-        result = torch.scatter_reduce(result, 0, index, in_data, "sum")
+        result = _sum_rows_by_index(in_data, route_indices, n, shape)
         if ever_padded and int(tags_value[0].item()) == 0:
             result = result.narrow(0, 1, n - 1)
             tags_value = tags_value.narrow(0, 1, n - 1)
     out_loads = torch.tensor([tags_value.numel()], dtype=torch.int32, device=in_data.device)
     return [result, tags_value, out_loads]
+
+
+def _sum_rows_by_index(in_data, index, n, shape):
+    """``zeros(n, ...).scatter_reduce(0, index repeated per element, in_data, "sum")``
+    (router.cc:451,459-460) as one pass over the rows: no per-element index tensor, rows added
+    in ascending row order in fp32."""
+    P = in_data.size(0)
+    if (in_data.dtype not in _DT or index.dtype not in (torch.int32, torch.int64)
+            or index.numel() != P or not index.is_cuda):
+        cell = in_data.numel() // P
+        expanded = index.view(-1, 1).repeat(1, cell).view_as(in_data)
+        zeros = torch.zeros(shape, dtype=in_data.dtype, device=in_data.device)
+        return torch.scatter_reduce(zeros, 0, expanded, in_data, "sum")
+    in_data = in_data.contiguous()
+    index = index.contiguous()
+    cell = in_data.numel() // P
+    result = torch.empty(shape, dtype=in_data.dtype, device=in_data.device)
+    ws_bytes = _lib.lib().brt_hip_combine_by_index_workspace_bytes(P, n)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=in_data.device)
+    _lib.check(_lib.lib().brt_hip_combine_by_index(
+        _ptr(in_data), _ptr(result), _ptr(index), 32 if index.dtype == torch.int32 else 64, P, cell,
+        n, _ptr(ws), ws_bytes, _DT[in_data.dtype], _DT[in_data.dtype], _stream()))
+    return result
 
 
 # legacy name (sample/cpp/router.ipynb:258-266) of the seat-index combine

@@ -67,6 +67,18 @@ SIGNATURES = {
         [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int,
          _c_int, _c_int, _c_int, _c_ptr],
     ),
+    "brt_hip_unique_tags_workspace_bytes": (_c_size, [ctypes.c_long, ctypes.c_long]),
+    "brt_hip_unique_tags": (
+        _c_int,
+        [_c_ptr, _c_int, ctypes.c_long, ctypes.c_long, ctypes.c_long, _c_ptr, _c_size, _c_ptr, _c_ptr,
+         _c_ptr, _c_ptr],
+    ),
+    "brt_hip_combine_by_index_workspace_bytes": (_c_size, [_c_int, _c_int]),
+    "brt_hip_combine_by_index": (
+        _c_int,
+        [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_size, _c_int, _c_int,
+         _c_ptr],
+    ),
 }
 
 _lib = None

@@ -18,94 +18,12 @@
 #include <type_traits>
 
 #include "common.hpp"
+#include "rows.hpp"
 
 namespace brt {
 namespace {
 
 constexpr int kBlock = 256;
-
-// Copy units are native vector types, so that arrays of them live in registers.
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-typedef float f32x2 __attribute__((ext_vector_type(2)));
-
-template <int BYTES> struct Unit;
-template <> struct Unit<16> { using type = u32x4; };
-template <> struct Unit<8> { using type = u32x2; };
-template <> struct Unit<4> { using type = uint32_t; };
-template <> struct Unit<2> { using type = uint16_t; };
-
-template <int BYTES>
-__device__ __forceinline__ uint32_t unit_word(const typename Unit<BYTES>::type& v, int i) {
-  if constexpr (BYTES >= 8) return v[i];
-  else return v;
-}
-
-constexpr int elem_bytes(int dt) { return dt == BRT_F32 ? 4 : 2; }
-
-// Unpacks BYTES of DT elements to fp32.
-template <int DT, int BYTES>
-__device__ __forceinline__ void unpack(const typename Unit<BYTES>::type& v,
-                                       float (&x)[BYTES / elem_bytes(DT)]) {
-  if constexpr (BYTES == 2) {
-    x[0] = half_bits_to_float<DT>(v);
-  } else {
-#pragma unroll
-    for (int i = 0; i < BYTES / 4; ++i) {
-      const uint32_t w = unit_word<BYTES>(v, i);
-      if constexpr (DT == BRT_F32) {
-        x[i] = __uint_as_float(w);
-      } else {
-        x[2 * i] = half_bits_to_float<DT>(w & 0xffffu);
-        x[2 * i + 1] = half_bits_to_float<DT>(w >> 16);
-      }
-    }
-  }
-}
-
-// Packs N fp32 values to DT (round to nearest even) and stores them at p.
-template <int DT, int N>
-__device__ __forceinline__ void pack_store(void* p, const float (&x)[N]) {
-  if constexpr (DT == BRT_F32) {
-    if constexpr (N % 4 == 0) {
-#pragma unroll
-      for (int i = 0; i < N / 4; ++i) {
-        f32x4 o = {x[4 * i], x[4 * i + 1], x[4 * i + 2], x[4 * i + 3]};
-        static_cast<f32x4*>(p)[i] = o;
-      }
-    } else if constexpr (N == 2) {
-      f32x2 o = {x[0], x[1]};
-      *static_cast<f32x2*>(p) = o;
-    } else {
-      *static_cast<float*>(p) = x[0];
-    }
-  } else {
-    if constexpr (N == 1) {
-      *static_cast<uint16_t*>(p) = static_cast<uint16_t>(float_to_half_bits<DT>(x[0]));
-    } else {
-      uint32_t w[N / 2];
-#pragma unroll
-      for (int i = 0; i < N / 2; ++i)
-        w[i] = float_to_half_bits<DT>(x[2 * i]) | (float_to_half_bits<DT>(x[2 * i + 1]) << 16);
-      if constexpr (N == 8) {
-        u32x4 o = {w[0], w[1], w[2], w[3]};
-        *static_cast<u32x4*>(p) = o;
-      } else if constexpr (N == 4) {
-        u32x2 o = {w[0], w[1]};
-        *static_cast<u32x2*>(p) = o;
-      } else {
-        *static_cast<uint32_t*>(p) = w[0];
-      }
-    }
-  }
-}
-
-template <int BYTES>
-__device__ __forceinline__ typename Unit<BYTES>::type zero_unit() {
-  typename Unit<BYTES>::type z = {};
-  return z;
-}
 
 // ------------------------------------------------------- wave-level plumbing
 // Every wavefront works on its own: it owns `rows_pw` consecutive rows of the

@@ -220,6 +220,39 @@ int brt_hip_grouped_gemm_routed(const void* x, const void* const* weights,
                                 const int32_t* tags, int E, int P, int T, int K, int N, int act,
                                 int gather_in, int scatter_out, void* stream);
 
+/* ---------------------------------------------------------------------------
+ * Tag-index gather (the default GatherRouter path of the reference).
+ *
+ * brt_hip_unique_tags replaces the `_unique(cat(tags), sorted, return_inverse)` call of
+ *   fuse_split_cells_from_paths (src/backend/torch/router.cc:348-369): `tags` [n] (int32 or
+ *   int64, `tag_bits` 32 or 64) with every value in [lo, hi] (the caller's min and max; values
+ *   outside get inverse -1 and are left out) -> `unique_tags` (same element type, room for
+ *   min(n, hi-lo+1) values, ascending), `inverse` [n] int64 (position of tags[i] in
+ *   unique_tags), `n_unique` [1] int32 on the device.  No sort: a presence table over the range
+ *   and one prefix sum.  hi-lo+1 may be at most 2^25 (BRT_E_UNSUPPORTED beyond; the workspace
+ *   size query returns 0 then).
+ *
+ * brt_hip_combine_by_index replaces the tag-mode branch of combine_with_indices_and_loads
+ *   (router.cc:449-472: `repeat` of the index to one int64 per element + `scatter_reduce`
+ *   "sum" into zeros): out_data[r] = sum of in_data[p] over the rows p with index[p] == r, for
+ *   r < n_out; rows nobody points to become zero, rows with an index outside [0, n_out) are
+ *   left out.  `index` is int32 or int64 (`index_bits`).  The sum runs in ascending p in fp32 and
+ *   is rounded once, so it is reproducible (the reference's atomics add in arrival order).
+ *   dtypes as brt_hip_combine: fp32, fp16, bf16, or a 16-bit input with fp32 output.
+ *   out_data is written whole; it needs no zero fill.
+ *
+ * Both take a caller-provided workspace (4-byte aligned, size from the query functions) and
+ * queue 1 to 5 small launches on `stream` (small inputs are handled by a single workgroup).
+ */
+size_t brt_hip_unique_tags_workspace_bytes(long lo, long hi);
+int brt_hip_unique_tags(const void* tags, int tag_bits, long n, long lo, long hi, void* workspace,
+                        size_t workspace_bytes, void* unique_tags, int64_t* inverse,
+                        int32_t* n_unique, void* stream);
+size_t brt_hip_combine_by_index_workspace_bytes(int P, int n_out);
+int brt_hip_combine_by_index(const void* in_data, void* out_data, const void* index, int index_bits,
+                             int P, int cell, int n_out, void* workspace, size_t workspace_bytes,
+                             int in_dtype, int out_dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

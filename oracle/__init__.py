@@ -47,6 +47,9 @@ def lib() -> ctypes.CDLL:
         _lib.oracle_bf16_to_float.argtypes = [ctypes.c_uint16]
         _lib.oracle_float_to_bf16.restype = ctypes.c_uint16
         _lib.oracle_float_to_bf16.argtypes = [ctypes.c_float]
+        _lib.oracle_unique_tags.restype = ctypes.c_int64
+        _lib.oracle_unique_tags.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p,
+                                            ctypes.c_void_p]
     return _lib
 
 
@@ -117,6 +120,37 @@ def topk_hot_mask(score, k: int) -> np.ndarray:
     mask = np.zeros((T, E), dtype=np.int32)
     lib().oracle_topk_hot_mask(_p(score), _p(mask), T, E, int(k))
     return mask
+
+
+def unique_tags(tags) -> Tuple[np.ndarray, np.ndarray]:
+    """``_unique(tags, sorted=True, return_inverse=True)`` of ``fuse_split_cells_from_paths``
+    (router.cc:362-366): ascending distinct tags and the position of every input tag in them
+    (int64, as the library returns it)."""
+    tags = np.ascontiguousarray(tags)
+    kind = tags.dtype
+    t64 = np.ascontiguousarray(tags.reshape(-1), dtype=np.int64)
+    unique = np.empty_like(t64)
+    inverse = np.empty_like(t64)
+    m = lib().oracle_unique_tags(_p(t64), t64.size, _p(unique), _p(inverse))
+    return unique[:m].astype(kind), inverse
+
+
+def combine_by_index(in_data, index, n_out: int, in_dtype: str = "f32",
+                     out_dtype: Optional[str] = None) -> np.ndarray:
+    """Tag-mode ``combine_with_indices_and_loads`` (router.cc:449-460) on flattened cells:
+    ``out[index[p]] += in_data[p]`` into zeros, rows added in ascending ``p`` in fp32."""
+    out_dtype = out_dtype or in_dtype
+    x = _data(in_data, in_dtype)
+    P = x.shape[0]
+    x = x.reshape(P, -1) if P > 0 else x.reshape(0, int(np.prod(x.shape[1:])))
+    cell = x.shape[1]
+    idx = np.ascontiguousarray(np.asarray(index).reshape(-1), dtype=np.int64)
+    assert idx.size == P
+    out = np.zeros((n_out, cell), dtype=_NP[out_dtype])
+    if n_out > 0 and cell > 0:
+        lib().oracle_combine_by_index(_p(x), _p(out), _p(idx), P, cell, int(n_out),
+                                      _DT[in_dtype], _DT[out_dtype])
+    return out
 
 
 def convert_index_format(indices, loads, tag_to_seat: bool) -> np.ndarray:

@@ -10,6 +10,7 @@
  *                            combine_with_seat_indices, init_with_seat_indices
  *   src/backend/torch/router.cc   shape/dtype conventions around them
  *   python/brt/router/protocol/topk.py:26-31   top-k hot mask (torch.topk + scatter_)
+ *   src/backend/torch/router.cc:348-369,449-472   tag-index gather (_unique + scatter_reduce)
  *
  * Only tests, the smoke check and the bench's cpu_baseline leg may link or call
  * this file; the product path never does.
@@ -29,6 +30,7 @@
 #include <stdint.h>
 #include <stddef.h>
 #include <string.h>
+#include <stdlib.h>
 
 enum { ORACLE_F32 = 0, ORACLE_F16 = 1, ORACLE_BF16 = 2 };
 
@@ -398,4 +400,50 @@ void oracle_topk_hot_mask(const float* score, int32_t* mask, int T, int E, int k
       out[best] = 1;
     }
   }
+}
+
+/* ---------- tag-index gather (router.cc:348-369, 449-472) ----------
+ * fuse_split_cells_from_paths hands the concatenated tags to `_unique(sorted, return_inverse)`:
+ * the distinct values in ascending order and, for every input element, the position of its
+ * value in that list.  Restated the way the library does it: sort a copy, drop repeats, then
+ * look every element up by bisection. */
+static int cmp_i64(const void* a, const void* b) {
+  int64_t x = *(const int64_t*)a, y = *(const int64_t*)b;
+  return (x > y) - (x < y);
+}
+
+int64_t oracle_unique_tags(const int64_t* tags, int64_t n, int64_t* unique, int64_t* inverse) {
+  if (n <= 0) return 0;
+  memcpy(unique, tags, (size_t)n * sizeof(int64_t));
+  qsort(unique, (size_t)n, sizeof(int64_t), cmp_i64);
+  int64_t m = 0;
+  for (int64_t i = 0; i < n; ++i)
+    if (i == 0 || unique[i] != unique[m - 1]) unique[m++] = unique[i];
+  for (int64_t i = 0; i < n; ++i) {
+    int64_t lo = 0, hi = m - 1;
+    while (lo < hi) {
+      int64_t mid = (lo + hi) / 2;
+      if (unique[mid] < tags[i]) lo = mid + 1; else hi = mid;
+    }
+    inverse[i] = lo;
+  }
+  return m;
+}
+
+/* The tag-mode combine is zeros(n_out, cell).scatter_reduce(0, index per element, in, "sum")
+ * (router.cc:451,459-460): out[index[p]] += in[p].  The reference's atomics add in arrival
+ * order; the order is fixed here to ascending p, with an fp32 accumulator that starts at zero
+ * and one rounding to the output type at the end. */
+void oracle_combine_by_index(const void* src, void* dst, const int64_t* index, int P, int cell,
+                             int n_out, int in_dtype, int out_dtype) {
+  float* acc = (float*)calloc((size_t)(cell > 0 ? cell : 1), sizeof(float));
+  for (int r = 0; r < n_out; ++r) {
+    for (int c = 0; c < cell; ++c) acc[c] = 0.0f;
+    for (int p = 0; p < P; ++p) {
+      if (index[p] != r) continue;
+      for (int c = 0; c < cell; ++c) acc[c] += load_elem(src, in_dtype, (size_t)p * cell + c);
+    }
+    for (int c = 0; c < cell; ++c) store_elem(dst, out_dtype, (size_t)r * cell + c, acc[c]);
+  }
+  free(acc);
 }

@@ -182,3 +182,47 @@ def topk_hot_mask(score_bits, k, dtype="f32"):
     _lib.check(_lib.lib().brt_hip_topk_hot_mask(ptr(d_s), ptr(d_m), T, E, k, DT[dtype], stream()))
     torch.cuda.synchronize()
     return host(d_m)
+
+
+def unique_tags(tags, lo=None, hi=None):
+    """-> (unique, inverse); tags int32 or int64."""
+    tags = np.ascontiguousarray(tags)
+    n = tags.size
+    lo = int(tags.min()) if lo is None else lo
+    hi = int(tags.max()) if hi is None else hi
+    L = _lib.lib()
+    need = L.brt_hip_unique_tags_workspace_bytes(lo, hi)
+    assert need > 0
+    ws = torch.full((need,), 0xA5, dtype=torch.uint8, device="cuda")
+    d_tags = dev(tags)
+    d_unique = torch.full((min(n, hi - lo + 1),), -9, dtype=d_tags.dtype, device="cuda")
+    d_inverse = torch.full((n,), -9, dtype=torch.int64, device="cuda")
+    d_count = torch.full((1,), -9, dtype=torch.int32, device="cuda")
+    _lib.check(L.brt_hip_unique_tags(
+        ptr(d_tags), 8 * tags.dtype.itemsize, n, lo, hi, ptr(ws), need, ptr(d_unique),
+        ptr(d_inverse), ptr(d_count), stream()))
+    torch.cuda.synchronize()
+    m = int(d_count.item())
+    return host(d_unique)[:m], host(d_inverse)
+
+
+def combine_by_index(y_bits, index, n_out, in_dtype="f32", out_dtype=None):
+    out_dtype = out_dtype or in_dtype
+    y_bits = np.ascontiguousarray(y_bits)
+    index = np.ascontiguousarray(index)
+    P = y_bits.shape[0]
+    cell = y_bits.size // max(P, 1)
+    L = _lib.lib()
+    need = L.brt_hip_combine_by_index_workspace_bytes(P, n_out)
+    ws = torch.full((need,), 0xA5, dtype=torch.uint8, device="cuda")
+    d_y = dev(y_bits.reshape(P, -1))
+    if out_dtype == "f32":
+        d_out = torch.full((n_out, cell), float("nan"), device="cuda")
+    else:
+        d_out = torch.full((n_out, cell), 0x55, dtype=torch.int16, device="cuda")
+    d_index = dev(index)
+    _lib.check(L.brt_hip_combine_by_index(
+        ptr(d_y), ptr(d_out), ptr(d_index), 8 * index.dtype.itemsize, P, cell, n_out, ptr(ws), need,
+        DT[in_dtype], DT[out_dtype], stream()))
+    torch.cuda.synchronize()
+    return host(d_out, True)

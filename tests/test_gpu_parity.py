@@ -357,6 +357,85 @@ def _route(hip, mask, caps=None, pad=False):
     return idx, loads, counts
 
 
+# ----------------------------------------------------------- tag-index gather
+@pytest.mark.parametrize("n,lo,hi,kind", [
+    (1, 7, 7, np.int32), (50, 0, 9, np.int32), (8192, 1, 8192, np.int32),
+    (20000, 0, 8191, np.int64),          # one scan block, every tag many times
+    (30000, -5000, 60000, np.int32),     # 8 scan blocks, negative tags
+    (100000, 100, 1500000, np.int64),    # 184 scan blocks, most tags absent
+])
+def test_unique_tags_bit_exact(hip, n, lo, hi, kind):
+    rng = np.random.default_rng(n + hi)
+    tags = rng.integers(lo, hi + 1, size=n).astype(kind)
+    tags[0], tags[-1] = lo, hi
+    unique, inverse = hip.unique_tags(tags)
+    want_u, want_i = oracle.unique_tags(tags)
+    assert unique.dtype == kind and np.array_equal(unique, want_u)
+    assert np.array_equal(inverse, want_i)
+
+
+def test_unique_tags_with_a_wider_range_than_the_data(hip):
+    tags = np.array([5, 3, 5, 9], dtype=np.int32)
+    unique, inverse = hip.unique_tags(tags, lo=0, hi=20000)
+    assert unique.tolist() == [3, 5, 9] and inverse.tolist() == [1, 0, 1, 2]
+    # a tag outside the stated range is left out and flagged in the inverse
+    unique, inverse = hip.unique_tags(tags, lo=4, hi=9)
+    assert unique.tolist() == [5, 9] and inverse.tolist() == [0, -1, 0, 1]
+
+
+@pytest.mark.parametrize("P,n_out,cell,in_dtype,out_dtype,kind", [
+    (1, 1, 8, "f32", "f32", np.int64),
+    (300, 100, 1, "f32", "f32", np.int32),
+    (300, 100, 3, "f16", "f16", np.int64),
+    (1000, 400, 5, "bf16", "bf16", np.int32),
+    (2000, 1500, 96, "f32", "f32", np.int64),
+    (4096, 2048, 768, "bf16", "bf16", np.int64),
+    (4096, 4096, 768, "bf16", "f32", np.int64),
+    (3000, 1000, 1000, "f16", "f32", np.int32),
+    (500, 7, 40, "f32", "f32", np.int64),     # lists of about 70 rows: longer than a wavefront
+    (70000, 66000, 4, "bf16", "bf16", np.int64),
+])
+def test_combine_by_index_bit_exact(hip, P, n_out, cell, in_dtype, out_dtype, kind):
+    rng = np.random.default_rng(P + cell)
+    bits = as_dtype_bits(rng.standard_normal((P, cell)).astype(np.float32), in_dtype)
+    index = rng.integers(0, n_out, size=P).astype(kind)
+    if P > 10:
+        index[3], index[5] = -1, n_out           # left out
+        index[index == 1] = 0                    # row 1 has no contributor
+    got = hip.combine_by_index(bits, index, n_out, in_dtype, out_dtype)
+    want = oracle.combine_by_index(bits, index, n_out, in_dtype, out_dtype)
+    assert same_bits(got, want)
+
+
+def test_combine_by_index_order_and_single_rounding(hip):
+    x = np.array([[1e8] * 4, [1.0] * 4, [-1e8] * 4], dtype=np.float32)
+    assert hip.combine_by_index(x, np.zeros(3, dtype=np.int64), 1).tolist() == [[0.0] * 4]
+    assert hip.combine_by_index(x[[0, 2, 1]], np.zeros(3, dtype=np.int64), 1).tolist() == [[1.0] * 4]
+    b = as_dtype_bits(np.array([[1.0] * 8, [2.0 ** -8] * 8, [2.0 ** -8] * 8], dtype=np.float32), "bf16")
+    got = bits_to_f32(hip.combine_by_index(b, np.zeros(3, dtype=np.int32), 1, "bf16"), "bf16")
+    assert (got == 1.0 + 2.0 ** -7).all()
+
+
+def test_tag_index_gather_against_the_library_calls(hip):
+    """The two entry points chained as the gather fabric chains them, against what the reference
+    calls (router.cc:362-366, 449-460): torch.unique + scatter_reduce over expanded indices."""
+    import torch
+
+    rng = np.random.default_rng(5)
+    loads = [700, 0, 1300, 48]
+    tags = np.concatenate([rng.permutation(2048)[:m] + 1 for m in loads]).astype(np.int32)
+    x = rng.standard_normal((sum(loads), 192)).astype(np.float32)
+    unique, inverse = hip.unique_tags(tags)
+    out = hip.combine_by_index(x, inverse, unique.size)
+    t_tags, t_x = torch.from_numpy(tags).cuda(), torch.from_numpy(x).cuda()
+    want_u, want_i = torch.unique(t_tags, sorted=True, return_inverse=True)
+    want = torch.zeros(want_u.numel(), 192, device="cuda").scatter_reduce(
+        0, want_i.view(-1, 1).repeat(1, 192), t_x, "sum")
+    assert np.array_equal(unique, want_u.cpu().numpy())
+    assert np.array_equal(inverse, want_i.cpu().numpy())
+    assert np.abs(out - want.cpu().numpy()).max() < 1e-5
+
+
 def test_config1_top1_capacity_drop_roundtrip(hip):
     # 1024 tokens x 512 fp32, 16 paths, capacity 64 with drop, identity experts
     T, E, d, cap = 1024, 16, 512, 64

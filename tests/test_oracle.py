@@ -474,3 +474,55 @@ def test_topk_hot_mask_ties_nan_and_infinities():
     # torch agrees wherever its answer is defined (rows without ties among the selected)
     picked = torch.topk(torch.from_numpy(score[2:]), 2, dim=1).indices
     assert sorted(picked[0].tolist()) == [0, 2] and sorted(picked[1].tolist()) == [2, 3]
+
+
+# ----------------------------------------------------------- tag-index gather
+@pytest.mark.parametrize("n,lo,hi,kind", [
+    (1, 5, 5, np.int32), (17, 0, 3, np.int32), (1000, 0, 4000, np.int32),
+    (5000, -300, 300, np.int64), (4096, 1, 4096, np.int64),
+])
+def test_unique_tags_is_numpy_unique(n, lo, hi, kind):
+    rng = np.random.default_rng(n + hi)
+    tags = rng.integers(lo, hi + 1, size=n).astype(kind)
+    unique, inverse = oracle.unique_tags(tags)
+    want_u, want_i = np.unique(tags, return_inverse=True)
+    assert unique.dtype == kind and np.array_equal(unique, want_u)
+    assert np.array_equal(inverse, want_i.astype(np.int64))
+    assert np.array_equal(unique[inverse], tags)
+
+
+def test_combine_by_index_permutation_moves_rows_unchanged():
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((64, 24)).astype(np.float32)
+    perm = rng.permutation(64)
+    out = oracle.combine_by_index(x, perm, 64)
+    assert np.array_equal(out[perm], x)
+    bits = as_dtype_bits(x, "bf16")
+    assert np.array_equal(oracle.combine_by_index(bits, perm, 64, "bf16")[perm], bits)
+
+
+def test_combine_by_index_adds_in_ascending_row_order_with_one_rounding():
+    # fp32: (1e8 + 1) - 1e8 is 0 in ascending order, any other order gives 1
+    x = np.array([[1e8], [1.0], [-1e8]], dtype=np.float32)
+    assert oracle.combine_by_index(x, [0, 0, 0], 1)[0, 0] == 0.0
+    assert oracle.combine_by_index(x[[0, 2, 1]], [0, 0, 0], 1)[0, 0] == 1.0
+    # bf16: 1 + 2^-8 + 2^-8 is 1 + 2^-7 when rounded once, 1 when rounded after every add
+    b = as_dtype_bits(np.array([[1.0], [2.0 ** -8], [2.0 ** -8]], dtype=np.float32), "bf16")
+    got = bits_to_f32(oracle.combine_by_index(b, [0, 0, 0], 1, "bf16"), "bf16")
+    assert got[0, 0] == 1.0 + 2.0 ** -7
+    # rows nobody points to are zero, indices outside [0, n_out) are left out
+    out = oracle.combine_by_index(np.ones((3, 2), dtype=np.float32), [2, 7, -1], 4)
+    assert out.tolist() == [[0, 0], [0, 0], [1, 1], [0, 0]]
+
+
+@pytest.mark.parametrize("dtype,tol", [("f32", 1e-6), ("f16", 2e-3), ("bf16", 1e-2)])
+def test_combine_by_index_against_float64_accumulation(dtype, tol):
+    rng = np.random.default_rng(11)
+    P, n_out, cell = 700, 200, 17
+    x = rng.standard_normal((P, cell)).astype(np.float32)
+    bits = as_dtype_bits(x, dtype)
+    index = rng.integers(0, n_out, size=P)
+    want = np.zeros((n_out, cell))
+    np.add.at(want, index, bits_to_f32(bits, dtype).astype(np.float64))
+    got = bits_to_f32(oracle.combine_by_index(bits, index, n_out, dtype), dtype)
+    assert np.abs(got - want).max() <= tol * max(1.0, np.abs(want).max())

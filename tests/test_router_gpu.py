@@ -307,3 +307,36 @@ def test_throttle_and_swin_scatter(brt_mod):
     kept = thr.any(1)
     assert torch.equal(out[torch.from_numpy(kept).cuda()], x[torch.from_numpy(kept).cuda()])
     assert not out[torch.from_numpy(~kept).cuda()].any()
+
+
+def test_tag_index_gather_ops_run_native_and_match_the_oracle(brt_mod):
+    """fuse_split_cells_from_paths(is_tag_fuse) + combine_with_indices_and_loads(is_tag_index)
+    (router.cc:348-369, 449-472) on the rows of three paths, one of them padded with empty
+    (tag 0) rows: sorted unique tags, inverse, the ascending-row fp32 sum, and the drop of the
+    tag-0 row."""
+    _, c_router, _, _ = brt_mod
+    rng = np.random.default_rng(21)
+    tags = [rng.permutation(500)[:m] + 1 for m in (200, 0, 350)] + [np.array([7, 0, 0, 9, 0])]
+    tags = [t.astype(np.int32) for t in tags]
+    datas = [rng.standard_normal((t.size, 40)).astype(np.float32) for t in tags]
+    d_tags = [torch.from_numpy(t).cuda() for t in tags]
+    d_datas = [torch.from_numpy(d).cuda().to(torch.bfloat16) for d in datas]
+    fused, new_tags, seats = c_router.fuse_split_cells_from_paths(d_datas, is_tag_fuse=True, tags=d_tags)
+    all_tags = np.concatenate(tags)
+    want_u, want_i = oracle.unique_tags(all_tags)
+    assert new_tags.dtype == torch.int32 and np.array_equal(new_tags.cpu().numpy(), want_u)
+    assert seats.dtype == torch.int64 and np.array_equal(seats.cpu().numpy(), want_i)
+    out, out_tags, n = c_router.combine_with_indices_and_loads(
+        fused, seats, None, tags=new_tags, is_tag_index=True)
+    bits = fused.view(torch.int16).cpu().numpy().view(np.uint16)
+    want = oracle.combine_by_index(bits, want_i, want_u.size, "bf16")
+    assert want_u[0] == 0                                    # the padded path's empty rows
+    assert np.array_equal(out.view(torch.int16).cpu().numpy().view(np.uint16), want[1:])
+    assert np.array_equal(out_tags.cpu().numpy(), want_u[1:]) and n.item() == want_u.size - 1
+    kept, kept_tags, _ = c_router.combine_with_indices_and_loads(
+        fused, seats, None, tags=new_tags, is_tag_index=True, ever_padded=False)
+    assert kept.shape[0] == want_u.size and torch.equal(kept[1:], out)
+    # tags spread thinly over a huge range take the library's sort; same results
+    far = torch.tensor([3, 2_000_000_000, 3, -5], dtype=torch.int64, device="cuda")
+    _, u, inv = c_router.fuse_split_cells_from_paths([fused[:4]], is_tag_fuse=True, tags=[far])
+    assert u.tolist() == [-5, 3, 2_000_000_000] and inv.tolist() == [1, 2, 1, 0]
