@@ -39,11 +39,11 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # FETCH_SIZE and WRITE_SIZE (KiB), each scaled by what the same counter reads for
 # a 12 MiB device-to-device copy (fetch x1.996, write x1.000).
 MEASURED_TRAFFIC_BYTES = {
-    "dispatch": int((7207.5 * 1.996 + 12482.4) * 1024),
+    "dispatch": int((7207.5 * 1.996 + 12482.5) * 1024),
     "combine": int((6221.5 * 1.996 + 12288.0) * 1024),
-    "combine_gather": int((7210.0 * 1.996 + 12288.0) * 1024),
-    "ffn_gemm1_gelu": int((155668.3 * 1.996 + 49152.0) * 1024),
-    "ffn_gemm2": int((172255.1 * 1.996 + 12288.0) * 1024),
+    "combine_gather": int((7197.0 * 1.996 + 12288.0) * 1024),
+    "ffn_gemm1_gelu": int((155549.8 * 1.996 + 49152.0) * 1024),
+    "ffn_gemm2": int((172254.3 * 1.996 + 12288.0) * 1024),
 }
 
 T, D, E, DFF = 8192, 768, 64, 3072
@@ -404,6 +404,7 @@ def main():
     flops["ffn_gemm2_scatter"] = flops["ffn_gemm2"]
     bytes_["indexgen_tags"] = bytes_["indexgen"]
     bytes_["gate_topk_mask"] = 2 * idx_bytes  # fp32 scores in, int32 mask out
+    bytes_["tag_gather_sum"] = 2 * P * D * es + 8 * P + 4 * (2 * P)  # rows in/out, index, lists
     dc_bytes = bytes_["dispatch"] + bytes_["combine"]
     dc_us = us["dispatch"] + us["combine"]
     value = dc_bytes / dc_us / 1e3  # GB/s
