@@ -64,6 +64,16 @@ def _one_hot_int32(indices: torch.Tensor, like: torch.Tensor) -> torch.Tensor:
     return torch.zeros(like.shape, dtype=torch.int32, device=like.device).scatter_(1, indices, 1)
 
 
+def _topk_hot_mask(score, top_k):
+    """int32 mask with ones at the ``top_k`` largest scores of every row (``torch.topk`` +
+    ``zeros_like`` + ``scatter_``, protocol/topk.py:26-31): one kernel where the score is a 2-d
+    device tensor of up to 1024 paths, the three torch launches otherwise."""
+    if (score.is_cuda and score.dim() == 2 and score.shape[1] <= 1024
+            and score.dtype in (torch.float32, torch.float16, torch.bfloat16)):
+        return c_router.topk_hot_mask(score, top_k)
+    return _one_hot_int32(torch.topk(score, top_k, dim=1).indices, score)
+
+
 @register_protocol("topk")
 class TopKProtocol(ProtocolBase):
     """protocol/topk.py:13-31."""
@@ -74,10 +84,7 @@ class TopKProtocol(ProtocolBase):
         self.single_path = top_k == 1
 
     def make_route_decision(self, score):
-        if (score.is_cuda and score.dim() == 2 and score.shape[1] <= 1024
-                and score.dtype in (torch.float32, torch.float16, torch.bfloat16)):
-            return c_router.topk_hot_mask(score, self.top_k)  # one kernel instead of three
-        return _one_hot_int32(torch.topk(score, self.top_k, dim=1).indices, score)
+        return _topk_hot_mask(score, self.top_k)
 
 
 @register_protocol("switch_top1")
@@ -234,6 +241,8 @@ def throttle_to_capacity(hot_mask, prefix, capacity, by_score=False, score=None)
 class SwinMoEProtocol(ProtocolBase):
     """protocol/swin_moe.py:69-144 (the maintained ``make_route_decision``)."""
 
+    single_path = True  # only the first of the top-k choices is routed (swin_moe.py:138-144)
+
     def __init__(self, top_k=2, capacity_factor=0, gate_noise=0.0, group=None, is_postscore=True,
                  batch_prioritized_routing=False, normalize_gate=True, is_gshard_loss=True,
                  alignment=1, **kwargs):
@@ -256,8 +265,7 @@ class SwinMoEProtocol(ProtocolBase):
 
     def make_route_decision(self, score, logits_wo_noise, logits):
         paths = score.size(1)
-        first_choice = torch.topk(score, self.top_k, dim=1).indices[:, :1]
-        mask = _one_hot_int32(first_choice, score)
+        mask = _topk_hot_mask(score, 1)  # the first of the top-k choices (swin_moe.py:101-107)
         loss = self.generate_auxiliary(score, logits_wo_noise, logits, None)
         cap = self.runtime_capacity(score.size(0), paths)
         runtime_capacities = torch.full((paths,), cap, dtype=torch.int32, device=score.device)
