@@ -64,6 +64,7 @@ struct GemmArgs {
   int E, P, K, N, T;
   int gather, scatter;  // rows of x / of out are addressed through the tags
   int tiles_n, tiles_m_max;
+  int walk, groups_n;  // column tiles one workgroup walks, ceil(tiles_n / walk)
 };
 
 // GELU(v) = v * Phi(v) = max(v, 0) - |v| * Phi(-|v|), branch free.  The tail probability is
@@ -97,7 +98,7 @@ struct Staged {
   u32x4 v[N];
 };
 
-template <int MT, int NT, int WAVES, int ACT>
+template <int MT, int NT, int WAVES, int ACT, bool WALKS>
 __global__ __launch_bounds__(WAVES * 64) void grouped_gemm_kernel(GemmArgs a) {
   constexpr int THREADS = WAVES * 64;
   constexpr int BM = MT * 32, WN = NT * 32, BN = WAVES * WN;
@@ -121,7 +122,8 @@ __global__ __launch_bounds__(WAVES * 64) void grouped_gemm_kernel(GemmArgs a) {
   // that really exist -- only the device knows how many -- spread evenly), and the
   // column tiles of one row block are consecutive workgroups of that XCD.
   const int xcd = blockIdx.x % kXcds, idx = blockIdx.x / kXcds;
-  const int mt = (idx / a.tiles_n) * kXcds + xcd, nt = idx % a.tiles_n;
+  const int mt = (idx / a.groups_n) * kXcds + xcd, nt_first = (idx % a.groups_n) * a.walk;
+  const int nt_end = WALKS ? min(nt_first + a.walk, a.tiles_n) : nt_first + 1;  // this workgroup's column tiles
   if (mt >= a.tiles_m_max) return;
   if (tid < kWave) {
     int carry_t = 0, carry_m = 0;
@@ -156,7 +158,7 @@ __global__ __launch_bounds__(WAVES * 64) void grouped_gemm_kernel(GemmArgs a) {
   const int rows = __builtin_amdgcn_readfirstlane(s_tile[2]);
   const int seat0 = __builtin_amdgcn_readfirstlane(s_tile[3]);
   const int row_tiles = (rows + 31) >> 5;
-  const int n0 = nt * BN;
+  int n0 = nt_first * BN;
   const int K = a.K;
 
   // ---- global -> register staging ------------------------------------------------
@@ -175,13 +177,18 @@ __global__ __launch_bounds__(WAVES * 64) void grouped_gemm_kernel(GemmArgs a) {
   // is what dispatch writes for a padding row.
   const bool gather = a.gather != 0;
   const char* xa = reinterpret_cast<const char*>(gather ? a.x : a.x + static_cast<size_t>(row0) * K);
-  const char* wb = reinterpret_cast<const char*>(a.w[e] + static_cast<size_t>(n0) * K);
+  const __bf16* const w_e = a.w[e];
   const size_t xa_bytes = static_cast<size_t>(gather ? a.T : a.P - row0) * K * 2;
-  const size_t wb_bytes = static_cast<size_t>(a.N - n0) * K * 2;
   const __amdgpu_buffer_rsrc_t res_a = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<char*>(xa), 0, static_cast<int>(std::min<size_t>(xa_bytes, 0x7fffffff)), 0x00020000);
-  const __amdgpu_buffer_rsrc_t res_b = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<char*>(wb), 0, static_cast<int>(std::min<size_t>(wb_bytes, 0x7fffffff)), 0x00020000);
+  // weight rows from column `first` on; rows past N lie past the extent and read as zeros
+  auto weight_rows = [&](int first) {
+    const size_t bytes = static_cast<size_t>(a.N - first) * K * 2;
+    return __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<char*>(reinterpret_cast<const char*>(w_e + static_cast<size_t>(first) * K)), 0,
+        static_cast<int>(std::min<size_t>(bytes, 0x7fffffff)), 0x00020000);
+  };
+  __amdgpu_buffer_rsrc_t res_b = weight_rows(n0);
   // when ROWS_PER_PASS does not divide BM only the lower wavefronts take the last pass
   const bool a_last = A_EXACT || lr + (A_LOADS - 1) * ROWS_PER_PASS < BM;
   uint32_t off_a[A_LOADS], off_b[B_LOADS];
@@ -197,7 +204,7 @@ __global__ __launch_bounds__(WAVES * 64) void grouped_gemm_kernel(GemmArgs a) {
   }
 #pragma unroll
   for (int i = 0; i < B_LOADS; ++i)
-    off_b[i] = (static_cast<uint32_t>(min(lr + i * ROWS_PER_PASS, a.N - n0 - 1)) * K + lc * 8) * 2;
+    off_b[i] = (static_cast<uint32_t>(lr + i * ROWS_PER_PASS) * K + lc * 8) * 2;
   // LDS slot of chunk c of row r is c ^ (r & 7); ROWS_PER_PASS is a multiple of 8, so
   // the swizzle is the same for every pass of this thread
   const int slot = lr * kRowBytes + ((lc ^ (lr & 7)) << 4);
@@ -241,10 +248,6 @@ __global__ __launch_bounds__(WAVES * 64) void grouped_gemm_kernel(GemmArgs a) {
   };
 
   f32x16 acc[MT][NT];
-#pragma unroll
-  for (int i = 0; i < MT; ++i)
-#pragma unroll
-    for (int j = 0; j < NT; ++j) acc[i][j] = f32x16{};
 
   // MFMA operand: this lane feeds row (lane % 32), k-half (lane / 32) of a 32 x 16 block
   const int frag_row = lane & 31, frag_k = lane >> 5;
@@ -300,110 +303,208 @@ __global__ __launch_bounds__(WAVES * 64) void grouped_gemm_kernel(GemmArgs a) {
 
   // ---- K loop: tile kt in LDS stage kt&1, tile kt+1 in one register set (written to LDS
   // during step kt), tile kt+2 being loaded into the other ------------------------------
+  // A workgroup walks `walk` column tiles of its row block.  When K is a whole, even number
+  // of K-steps the load stream does not stop at a tile boundary: the last two K-steps of a
+  // tile already fetch the first two of the next one (same activation rows, next weight
+  // rows), so the expert lookup and the two exposed load latencies are paid once per
+  // workgroup and the next tile's operands arrive while the epilogue runs.
   const int k_tiles = (K + kBK - 1) / kBK;
+  const bool seamless = !k_tail && (k_tiles & 1) == 0 && k_tiles >= 2;
+  const global_bf16 bias = a.bias != nullptr ? (global_bf16)(a.bias[e]) : (global_bf16)nullptr;
   Staged<LOADS> s0, s1;
+  // first K-step of the first tile into LDS stage 0
 #pragma unroll
   for (int p = 0; p < kSteps; ++p) fetch_slice(s0, 0, p);
-  if (k_tiles > 1) {
+  if (!WALKS && k_tiles > 1) {  // one tile per workgroup: the second K-step starts right away
 #pragma unroll
     for (int p = 0; p < kSteps; ++p) fetch_slice(s1, kBK, p);
   }
 #pragma unroll
   for (int p = 0; p < kSteps; ++p) stash_slice(s0, 0, 0, p, Yes{});
   __syncthreads();
-  int kt = 0;
-  for (; kt + 3 < k_tiles; kt += 2) {
-    step(0, s0, s1, (kt + 2) * kBK, (kt + 1) * kBK, Yes{}, Yes{}, No{});
-    __syncthreads();
-    step(1, s1, s0, (kt + 3) * kBK, (kt + 2) * kBK, Yes{}, Yes{}, No{});
-    __syncthreads();
-  }
-  const int left = k_tiles - kt;  // 1, 2 or 3 tiles; kt is even, so the next tile is in stage 0
-  if (left == 3) {
-    step(0, s0, s1, (kt + 2) * kBK, (kt + 1) * kBK, Yes{}, Yes{}, No{});
-    __syncthreads();
-    step(1, s1, s0, 0, (kt + 2) * kBK, No{}, Yes{}, Yes{});
-    __syncthreads();
-    step(0, s0, s1, 0, 0, No{}, No{}, No{});
-  } else if (left == 2) {
-    step(0, s0, s1, 0, (kt + 1) * kBK, No{}, Yes{}, Yes{});
-    __syncthreads();
-    step(1, s1, s0, 0, 0, No{}, No{}, No{});
-  } else {
-    step(0, s0, s1, 0, 0, No{}, No{}, No{});
-  }
-  __syncthreads();
-
-  // ---- epilogue: bias + activation, bf16, through LDS, 16-byte row stores ---------------
-  // transposed accumulator: element r of tile (i, j) is output row 32 i + lane%32, column
-  // (of this wavefront's 32 j .. 32 j + 31) 8*(r/4) + 4*(lane/32) + r%4
-  const global_bf16 bias = a.bias != nullptr ? (global_bf16)(a.bias[e]) : (global_bf16)nullptr;
+  for (int nt = nt_first; nt < nt_end; ++nt, n0 += BN) {
+    // here LDS stage 0 holds the first K-step of this tile; the second one starts now.
+    // Nothing is carried in registers from one tile to the next: a staged set or an
+    // accumulator that lives around the tile loop costs the K loop more registers than
+    // it has.
+    if (WALKS && k_tiles > 1) {
 #pragma unroll
-  for (int j = 0; j < NT; ++j) {
-    float bv[4][4];
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const int col = n0 + wave * WN + j * 32 + 8 * g + 4 * frag_k;
-      bf16x4 b4 = {};
-      if (a.bias != nullptr && col < a.N) b4 = *(global_bf16x4)(bias + col);
-#pragma unroll
-      for (int q = 0; q < 4; ++q) bv[g][q] = static_cast<float>(b4[q]);
+      for (int p = 0; p < kSteps; ++p) fetch_slice(s1, kBK, p);
     }
 #pragma unroll
-    for (int i = 0; i < MT; ++i) {
-      if (i < row_tiles) {
-        char* dst = smem + (i * 32 + frag_row) * OUT_ROW + (wave * WN + j * 32 + 4 * frag_k) * 2;
+    for (int i = 0; i < MT; ++i)
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          bf16x4 o;
+      for (int j = 0; j < NT; ++j) acc[i][j] = f32x16{};
+    const bool ahead = seamless && nt + 1 < nt_end;  // the tail fetches into the next tile
+    int kt = 0;
+    for (; kt + 3 < k_tiles; kt += 2) {
+      step(0, s0, s1, (kt + 2) * kBK, (kt + 1) * kBK, Yes{}, Yes{}, No{});
+      __syncthreads();
+      step(1, s1, s0, (kt + 3) * kBK, (kt + 2) * kBK, Yes{}, Yes{}, No{});
+      __syncthreads();
+    }
+    if (ahead) {  // two K-steps left: the first K-step of the next tile rides along
+      res_b = weight_rows(n0 + BN);
+      step(0, s0, s1, 0, (kt + 1) * kBK, Yes{}, Yes{}, No{});
+      __syncthreads();
+      step(1, s1, s0, 0, 0, No{}, Yes{}, Yes{});
+      __syncthreads();
+    } else {
+      const int left = k_tiles - kt;  // 1, 2 or 3 tiles; kt is even, so the next tile is in stage 0
+      if (left == 3) {
+        step(0, s0, s1, (kt + 2) * kBK, (kt + 1) * kBK, Yes{}, Yes{}, No{});
+        __syncthreads();
+        step(1, s1, s0, 0, (kt + 2) * kBK, No{}, Yes{}, Yes{});
+        __syncthreads();
+        step(0, s0, s1, 0, 0, No{}, No{}, No{});
+      } else if (left == 2) {
+        step(0, s0, s1, 0, (kt + 1) * kBK, No{}, Yes{}, Yes{});
+        __syncthreads();
+        step(1, s1, s0, 0, 0, No{}, No{}, No{});
+      } else {
+        step(0, s0, s1, 0, 0, No{}, No{}, No{});
+      }
+      __syncthreads();
+    }
+
+    // ---- epilogue: bias + activation, bf16, through LDS, 16-byte row stores -------------
+    // transposed accumulator: element r of tile (i, j) is output row 32 i + lane%32, column
+    // (of this wavefront's 32 j .. 32 j + 31) 8*(r/4) + 4*(lane/32) + r%4.
+    // A walking workgroup sends the tile out in two passes of row tiles through LDS stage 1
+    // only: stage 0 may already hold the first K-step of the next tile.  With one tile per
+    // workgroup the whole tile is staged at once.
+    // The per-lane addresses of the epilogue are recomputed from an opaque copy of the thread
+    // index for every tile: as loop invariants of the column walk they would be hoisted into
+    // registers that stay live across the K loop, which has none to spare.
+    int tid_e = tid;
+    asm volatile("" : "+v"(tid_e));
+    const int frag_row_e = tid_e & 31, frag_k_e = (tid_e >> 5) & 1;
+    float bv[NT][4][4];
 #pragma unroll
-          for (int q = 0; q < 4; ++q)
-            o[q] = static_cast<__bf16>(apply_act<ACT>(acc[i][j][4 * g + q] + bv[g][q]));
-          *reinterpret_cast<bf16x4*>(dst + 16 * g) = o;
+    for (int j = 0; j < NT; ++j) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int col = n0 + wave * WN + j * 32 + 8 * g + 4 * frag_k_e;
+        bf16x4 b4 = {};
+        if (a.bias != nullptr && col < a.N) b4 = *(global_bf16x4)(bias + col);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) bv[j][g][q] = static_cast<float>(b4[q]);
+      }
+    }
+    constexpr int OUT_CHUNKS = BN / 8;
+    constexpr int kPasses = WALKS ? 2 : 1;
+    constexpr int kPassTiles = (MT + kPasses - 1) / kPasses;
+    static_assert(!WALKS || kPassTiles * 32 * OUT_ROW <= STAGE, "half an output tile must fit one LDS stage");
+    char* const stage_out = WALKS ? smem + STAGE : smem;
+    // Scatter mode: row s of expert e goes to cell tags[s,e]-1 of out (the combine of a
+    // single-path route is folded into the store); rows without a tag are dropped.
+    __bf16* __restrict__ oc = a.out + (a.scatter ? 0 : static_cast<size_t>(row0) * a.N) + n0;
+#pragma unroll
+    for (int pass = 0; pass < kPasses; ++pass) {
+      const int i_lo = pass * kPassTiles, i_hi = pass + 1 < kPasses ? kPassTiles : MT;
+      if (pass == 1) __syncthreads();  // the first half has left LDS
+#pragma unroll
+      for (int i = 0; i < MT; ++i) {
+        if (i < i_lo || i >= i_hi) continue;
+        if (i < row_tiles) {
+#pragma unroll
+          for (int j = 0; j < NT; ++j) {
+            char* dst = stage_out + ((i - i_lo) * 32 + frag_row_e) * OUT_ROW + (wave * WN + j * 32 + 4 * frag_k_e) * 2;
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+              bf16x4 o;
+#pragma unroll
+              for (int q = 0; q < 4; ++q)
+                o[q] = static_cast<__bf16>(apply_act<ACT>(acc[i][j][4 * g + q] + bv[j][g][q]));
+              *reinterpret_cast<bf16x4*>(dst + 16 * g) = o;
+            }
+          }
         }
+      }
+      __syncthreads();
+      const int r_lo = i_lo * 32, r_hi = min(rows, i_hi * 32);
+      for (int q = tid_e; q < (r_hi - r_lo) * OUT_CHUNKS; q += THREADS) {
+        const int rl = q / OUT_CHUNKS, c = q - rl * OUT_CHUNKS;
+        const int r = r_lo + rl;
+        long to = r;
+        if (a.scatter) {
+          const int tag = a.tags[static_cast<size_t>(seat0 + r) * a.E + e];
+          to = (tag >= 1 && tag <= a.T) ? tag - 1 : -1;
+        }
+        if (to >= 0 && n0 + c * 8 < a.N)
+          *reinterpret_cast<u32x4*>(oc + static_cast<size_t>(to) * a.N + c * 8) =
+              *reinterpret_cast<const u32x4*>(stage_out + rl * OUT_ROW + c * 16);
+      }
+    }
+    if (nt + 1 < nt_end) {
+      __syncthreads();  // stage 1 is written again by the first K-step of the next tile
+      if (!ahead) {  // K does not allow the seamless tail: load the next tile's first K-step now
+        res_b = weight_rows(n0 + BN);
+#pragma unroll
+        for (int p = 0; p < kSteps; ++p) fetch_slice(s0, 0, p);
+#pragma unroll
+        for (int p = 0; p < kSteps; ++p) stash_slice(s0, 0, 0, p, Yes{});
+        __syncthreads();
       }
     }
   }
-  __syncthreads();
-  constexpr int OUT_CHUNKS = BN / 8;
-  // Scatter mode: row s of expert e goes to cell tags[s,e]-1 of out (the combine of a
-  // single-path route is folded into the store); rows without a tag are dropped.
-  __bf16* __restrict__ oc = a.out + (a.scatter ? 0 : static_cast<size_t>(row0) * a.N) + n0;
-  for (int q = tid; q < rows * OUT_CHUNKS; q += THREADS) {
-    const int r = q / OUT_CHUNKS, c = q - r * OUT_CHUNKS;
-    long to = r;
-    if (a.scatter) {
-      const int tag = a.tags[static_cast<size_t>(seat0 + r) * a.E + e];
-      to = (tag >= 1 && tag <= a.T) ? tag - 1 : -1;
-    }
-    if (to >= 0 && n0 + c * 8 < a.N)
-      *reinterpret_cast<u32x4*>(oc + static_cast<size_t>(to) * a.N + c * 8) =
-          *reinterpret_cast<const u32x4*>(smem + r * OUT_ROW + c * 16);
-  }
 }
+
+int device_cus() {
+  static const int cus = [] {
+    int dev = 0, n = 256;
+    if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
+    return std::max(n, 1);
+  }();
+  return cus;
+}
+
+// row blocks of 160 a capacity-filled route has; the loads themselves live on the device
+long estimated_row_blocks(int P, int E) { return std::max<long>((P + 159) / 160, std::min(E, P)); }
 
 template <int MT, int NT, int WAVES, int ACT>
 int launch_act(GemmArgs& a, hipStream_t st) {
   constexpr int BM = MT * 32, BN = WAVES * NT * 32;
   constexpr int STAGE = (BM + BN) * kRowBytes;
-  constexpr int OUT_BYTES = BM * (BN * 2 + 16);
+  constexpr int OUT_BYTES = BM * (BN * 2 + 16);  // the epilogue stages the output tile in the same memory
   const size_t lds = std::max(2 * STAGE, OUT_BYTES);
   a.tiles_n = (a.N + BN - 1) / BN;
   // sum over experts of ceil(M_e/BM) never exceeds P/BM + E; rounded up to whole XCD rounds
   a.tiles_m_max = ((a.P + BM - 1) / BM + a.E + kXcds - 1) / kXcds * kXcds;
-  const long grid = static_cast<long>(a.tiles_m_max) * a.tiles_n;
+  // Column tiles one workgroup walks: the largest number that neither leaves CUs without a
+  // workgroup nor adds a round of tiles to the busiest CU (estimated like the tile shape,
+  // from the row blocks a capacity-filled route has; the loads themselves live on the device).
+  static const int forced_walk = std::getenv("BRT_GEMM_WALK") ? std::atoi(std::getenv("BRT_GEMM_WALK")) : 0;
+  a.walk = 1;
+  if (WAVES == 4) {  // the narrower tiles stage more per thread and have no registers left for it
+    const long slots = static_cast<long>(device_cus()) * (WAVES == 2 ? 2 : 1);
+    const long row_blocks = estimated_row_blocks(a.P, a.E);
+    const long plain = (row_blocks * a.tiles_n + slots - 1) / slots;
+    for (int w = a.tiles_n; w > 1; --w) {
+      const long groups = (a.tiles_n + w - 1) / w;
+      if (row_blocks * groups >= slots && (row_blocks * groups + slots - 1) / slots * w <= plain) {
+        a.walk = w;
+        break;
+      }
+    }
+  }
+  if (forced_walk > 0) a.walk = std::min(forced_walk, a.tiles_n);
+  a.groups_n = (a.tiles_n + a.walk - 1) / a.walk;
+  const long grid = static_cast<long>(a.tiles_m_max) * a.groups_n;
   // more than 64 KB of dynamic LDS has to be allowed once per device and kernel
   static bool configured[64] = {};
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 63;
   if (!configured[dev] || dev == 63) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&grouped_gemm_kernel<MT, NT, WAVES, ACT>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)) != hipSuccess)
-      return fail(BRT_E_LAUNCH, "cannot reserve %zu bytes of LDS", lds);
+    for (const void* fn : {reinterpret_cast<const void*>(&grouped_gemm_kernel<MT, NT, WAVES, ACT, false>),
+                           reinterpret_cast<const void*>(&grouped_gemm_kernel<MT, NT, WAVES, ACT, true>)})
+      if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)) != hipSuccess)
+        return fail(BRT_E_LAUNCH, "cannot reserve %zu bytes of LDS", lds);
     configured[dev] = true;
   }
-  hipLaunchKernelGGL((grouped_gemm_kernel<MT, NT, WAVES, ACT>), dim3(static_cast<unsigned>(grid)),
-                     dim3(WAVES * 64), lds, st, a);
+  const dim3 blocks(static_cast<unsigned>(grid)), threads(WAVES * 64);
+  if (a.walk > 1) hipLaunchKernelGGL((grouped_gemm_kernel<MT, NT, WAVES, ACT, true>), blocks, threads, lds, st, a);
+  else hipLaunchKernelGGL((grouped_gemm_kernel<MT, NT, WAVES, ACT, false>), blocks, threads, lds, st, a);
   return check_launch("grouped_gemm_kernel");
 }
 
@@ -454,12 +555,8 @@ int grouped_gemm_impl(const void* x, const void* const* weights, const void* con
   static const int forced = std::getenv("BRT_GEMM_SHAPE") ? std::atoi(std::getenv("BRT_GEMM_SHAPE")) : 0;
   int shape = forced;
   if (shape == 0) {
-    static const int cus = [] {
-      int dev = 0, n = 256;
-      if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
-      return std::max(n, 1);
-    }();
-    const long row_blocks = std::max<long>((P + 159) / 160, std::min(E, P));  // estimate; loads live on the device
+    const int cus = device_cus();
+    const long row_blocks = estimated_row_blocks(P, E);
     double best = 0;
     for (int waves = 4; waves >= 2; --waves) {
       const long tiles = row_blocks * ((N + 64 * waves - 1) / (64 * waves));

@@ -268,3 +268,20 @@ def test_gelu_epilogue_on_every_bf16_value():
     assert (got != want)[~tiny].float().mean() < 0.02
     launch(bt.data_ptr())
     assert (out[:, 3].float() == float("inf")).all() and (out[:, 5].float() == 0).all()
+
+
+@pytest.mark.parametrize("K,N", [
+    (768, 3072),    # even number of whole K-steps: the load stream runs across tile boundaries
+    (832, 3072),    # odd number of K-steps: every tile of the walk is primed on its own
+    (776, 3072),    # K tail
+    (768, 2816),    # 11 column tiles: the last workgroup of a row block walks fewer
+    (768, 3000),    # last column tile is partial
+    (128, 3072),    # two K-steps: nothing but the seamless tail
+])
+def test_workgroups_walking_several_column_tiles(K, N):
+    """64 full row blocks and 11-12 column tiles are more tiles than the chip has CUs, so every
+    workgroup walks three column tiles of its row block."""
+    run([160] * 64, K, N, act="gelu", bias=True, seed=K + N)
+    loads = [160] * 64
+    loads[5], loads[17], loads[40] = 0, 3, 97
+    run(loads, K, N, act="none", bias=False, seed=K, slack=100)
