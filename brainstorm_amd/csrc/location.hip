@@ -29,7 +29,9 @@
 // as a kernel boundary costs, so a single-pass chained scan buys nothing at MoE
 // sizes (a few MiB) and adds a way to hang.  Up to 16 rows per wavefront stay in
 // registers between the two walks of pass 2; longer bands re-read their rows
-// (from cache).  The indices are written exactly once.
+// (from cache).  The indices are written exactly once.  Masks small enough for one workgroup of
+// eight wavefronts to hold in registers skip pass 1: that workgroup is the only band, and its
+// wavefronts' column sums meet in LDS (one launch).
 #include <algorithm>
 #include <cstdlib>
 
