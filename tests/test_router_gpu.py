@@ -340,3 +340,56 @@ def test_tag_index_gather_ops_run_native_and_match_the_oracle(brt_mod):
     far = torch.tensor([3, 2_000_000_000, 3, -5], dtype=torch.int64, device="cuda")
     _, u, inv = c_router.fuse_split_cells_from_paths([fused[:4]], is_tag_fuse=True, tags=[far])
     assert u.tolist() == [-5, 3, 2_000_000_000] and inv.tolist() == [1, 2, 1, 0]
+
+
+def test_capacity_padded_moe_layer_replays_from_a_hip_graph(brt_mod):
+    """Scatter router (capacity padding with a fixed per-path stride) -> grouped FFN -> gather
+    router has no host read on its way, so the whole layer can be captured once and replayed for
+    new inputs (the reference's binding copies the loads to the host, router.cc:181-187).  Every
+    replay is checked against the same layer run eagerly, with eager work in between."""
+    brt, _, _, GatherRouter = brt_mod
+    from brt.jit import grouped_linear
+    from brt.router import SwinMoEScatterRouter
+    from brt.runtime.grid_tensor import init_grid_tensor_from
+
+    T, E, d, dff = 4096, 8, 96, 384
+    gen = torch.Generator(device="cuda").manual_seed(3)
+    x = torch.randn(T, d, device="cuda", generator=gen).to(torch.bfloat16)
+    score = torch.softmax(torch.randn(T, E, device="cuda", generator=gen), dim=1)
+    w1 = (torch.randn(E, dff, d, device="cuda", generator=gen) * 0.05).to(torch.bfloat16)
+    w2 = (torch.randn(E, d, dff, device="cuda", generator=gen) * 0.05).to(torch.bfloat16)
+    t1 = torch.tensor([w1[e].data_ptr() for e in range(E)], dtype=torch.int64, device="cuda")
+    t2 = torch.tensor([w2[e].data_ptr() for e in range(E)], dtype=torch.int64, device="cuda")
+    scatter = SwinMoEScatterRouter(
+        protocol_kwargs={"top_k": 1, "capacity_factor": 1.25}, fabric_type="fused_dispatch",
+        fabric_kwargs={"capacity_padding": True, "max_path_padding": True}).cuda()
+    gather = GatherRouter(fabric_type="fused_combine", fabric_kwargs={"max_path_padding": True}).cuda()
+    annotate = brt.Annotator([0])
+
+    def layer(cells, scores):
+        routed, _ = scatter(annotate(cells), scores, None, None)
+        rows = routed.shape[0]
+        hidden = torch.empty(rows, dff, dtype=torch.bfloat16, device="cuda")
+        y = torch.empty(rows, d, dtype=torch.bfloat16, device="cuda")
+        grouped_linear(brt.to_torch_tensor(routed), hidden, t1, None, routed.load, d, dff, "gelu")
+        grouped_linear(hidden, y, t2, None, routed.load, dff, d, None)
+        return gather(init_grid_tensor_from(y, routed))
+
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        layer(x, score)  # allocations and lazy initialisation happen outside the capture
+        torch.cuda.synchronize()
+        with torch.cuda.graph(graph, stream=stream):
+            captured = layer(x, score)
+    torch.cuda.synchronize()
+    for _ in range(4):
+        x.copy_(torch.randn(T, d, device="cuda", generator=gen).to(torch.bfloat16))
+        score.copy_(torch.softmax(torch.randn(T, E, device="cuda", generator=gen), dim=1))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        want = layer(x, score)
+        torch.cuda.synchronize()
+        assert torch.equal(captured, want)
+        assert captured.abs().sum() > 0
