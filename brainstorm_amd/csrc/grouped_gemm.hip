@@ -16,9 +16,10 @@
 // rows of its own 32 columns.  Both operands are K-contiguous in memory, which is
 // the MFMA operand layout (a lane feeds 8 consecutive k of one row), so tiles
 // travel global -> registers -> LDS as 16-byte chunks without any transpose and
-// come back as ds_read_b128 fragments; chunk c of row r lives in slot c ^ (r & 7)
-// so that the 8 rows a read touches per cycle fall into distinct bank groups
-// without padding.  The loop is bound by memory latency, not by MFMA issue, so it
+// come back as ds_read_b128 fragments; chunk c of row r lives in slot
+// c ^ ((r >> 1) & 7), so that any 16 consecutive rows read at the same k cover all
+// 64 banks exactly once (a row is 32 banks wide: even and odd rows take the two
+// halves, and the 8 rows of one parity take 8 different slots) without padding.  The loop is bound by memory latency, not by MFMA issue, so it
 // keeps two K-steps in flight in registers on top of the two LDS stages (one
 // barrier per K-step of 64).  v_mfma_f32_32x32x16_bf16 is issued with the weight
 // fragment as its first operand: the accumulator then holds the transposed tile,
@@ -205,9 +206,12 @@ __global__ __launch_bounds__(WAVES * 64) void grouped_gemm_kernel(GemmArgs a) {
 #pragma unroll
   for (int i = 0; i < B_LOADS; ++i)
     off_b[i] = (static_cast<uint32_t>(lr + i * ROWS_PER_PASS) * K + lc * 8) * 2;
-  // LDS slot of chunk c of row r is c ^ (r & 7); ROWS_PER_PASS is a multiple of 8, so
-  // the swizzle is the same for every pass of this thread
-  const int slot = lr * kRowBytes + ((lc ^ (lr & 7)) << 4);
+  // LDS slot of chunk c of row r is c ^ ((r >> 1) & 7).  A thread's rows are ROWS_PER_PASS
+  // apart; the pass offset changes the swizzle term by a compile-time constant (0, or 4 for
+  // every other pass of the 3-wavefront tile), i.e. it flips one bit of the slot.
+  const int slot = lr * kRowBytes + ((lc ^ ((lr >> 1) & 7)) << 4);
+  auto pass_flip = [](int first_row) { return (((first_row >> 1) & 7) << 4); };  // xor on the byte offset
+  static_assert(ROWS_PER_PASS % 8 == 0 && BM % 16 == 0, "the pass offset must flip whole slot bits");
   const bool k_tail = (K % kBK) != 0;
 
   using Yes = std::integral_constant<bool, true>;
@@ -231,7 +235,7 @@ __global__ __launch_bounds__(WAVES * 64) void grouped_gemm_kernel(GemmArgs a) {
   };
   // the K tail (only ever in the last tile) is zeroed here, when the data is in registers
   auto stash_slice = [&](const Staged<LOADS>& s, int stage, int k0, int p, auto may_be_last) {
-    char* base = smem + stage * STAGE + slot;
+    char* stage_base = smem + stage * STAGE;
     const bool k_ok = !decltype(may_be_last)::value || !k_tail || k0 + lc * 8 < K;
     const u32x4 z = {};
 #pragma unroll
@@ -240,9 +244,11 @@ __global__ __launch_bounds__(WAVES * 64) void grouped_gemm_kernel(GemmArgs a) {
       const u32x4 v = k_ok ? s.v[i] : z;
       if (i < A_LOADS) {
         if (i + 1 < A_LOADS || a_last)
-          *reinterpret_cast<u32x4*>(base + i * ROWS_PER_PASS * kRowBytes) = v;
+          *reinterpret_cast<u32x4*>(stage_base + ((slot ^ pass_flip(i * ROWS_PER_PASS)) +
+                                                  i * ROWS_PER_PASS * kRowBytes)) = v;
       } else {
-        *reinterpret_cast<u32x4*>(base + (BM + (i - A_LOADS) * ROWS_PER_PASS) * kRowBytes) = v;
+        *reinterpret_cast<u32x4*>(stage_base + ((slot ^ pass_flip(BM + (i - A_LOADS) * ROWS_PER_PASS)) +
+                                                (BM + (i - A_LOADS) * ROWS_PER_PASS) * kRowBytes)) = v;
       }
     }
   };
@@ -266,7 +272,7 @@ __global__ __launch_bounds__(WAVES * 64) void grouped_gemm_kernel(GemmArgs a) {
     const char* sb = sa + (BM + wave * WN) * kRowBytes;
     bf16x8 fw[2][NT], fx[2][MT];
     auto read_frags = [&](int ks, int buf) {
-      const int phys = ((ks * 2 + frag_k) ^ (frag_row & 7)) << 4;
+      const int phys = ((ks * 2 + frag_k) ^ ((frag_row >> 1) & 7)) << 4;
 #pragma unroll
       for (int j = 0; j < NT; ++j)
         fw[buf][j] = *reinterpret_cast<const bf16x8*>(sb + j * 32 * kRowBytes + phys);
