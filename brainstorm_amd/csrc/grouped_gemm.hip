@@ -164,11 +164,11 @@ __global__ __launch_bounds__(WAVES * 64) void grouped_gemm_kernel(GemmArgs a) {
 
   // ---- global -> register staging ------------------------------------------------
   // Thread t owns 16-byte chunk t%8 of rows t/8 + i*ROWS_PER_PASS of the activation
-  // tile and of the weight tile.  Rows past the expert's last row or past N are
-  // clamped to a valid row (their products land in output rows/columns that are
-  // never stored, and all MT row tiles are always multiplied: the inner loop stays
-  // one branch-free block); only a K tail that is not a multiple of 64 needs real
-  // zeros.
+  // tile and of the weight tile.  Rows past the expert's last row or past N address
+  // past the buffer extent and read as zeros (their products land in output
+  // rows/columns that are never stored, and all MT row tiles are always multiplied:
+  // the inner loop stays one branch-free block); a K tail that is not a multiple of
+  // 64 is zeroed when it is written to LDS.
   const int lc = tid % kChunks, lr = tid / kChunks;
   // Buffer loads: a wave-uniform resource (base, byte extent) per operand, a 32-bit
   // per-lane byte offset and the K offset as the scalar offset, so the loop carries no
@@ -195,12 +195,15 @@ __global__ __launch_bounds__(WAVES * 64) void grouped_gemm_kernel(GemmArgs a) {
   uint32_t off_a[A_LOADS], off_b[B_LOADS];
 #pragma unroll
   for (int i = 0; i < A_LOADS; ++i) {
-    const int r = min(min(lr + i * ROWS_PER_PASS, BM - 1), rows - 1);
+    // rows past the expert's last one address past the extent: they read as zeros and cost no
+    // memory request (their products land in output rows that are never stored)
+    const int r = lr + i * ROWS_PER_PASS;
+    const bool in_tile = r < rows;
     if (gather) {
-      const int tag = a.tags[static_cast<size_t>(seat0 + r) * a.E + e];
+      const int tag = in_tile ? a.tags[static_cast<size_t>(seat0 + r) * a.E + e] : 0;
       off_a[i] = (tag >= 1 && tag <= a.T) ? (static_cast<uint32_t>(tag - 1) * K + lc * 8) * 2 : 0x80000000u;
     } else {
-      off_a[i] = (static_cast<uint32_t>(r) * K + lc * 8) * 2;
+      off_a[i] = in_tile ? (static_cast<uint32_t>(r) * K + lc * 8) * 2 : 0x80000000u;
     }
   }
 #pragma unroll
