@@ -363,13 +363,18 @@ def main():
     stream.synchronize()
     unique_torch_us = e0.elapsed_time(e1) * 1e3 / 20
 
+    # a plain device-to-device copy of as many rows as dispatch moves: what the same traffic
+    # costs without any routing, at this size
+    def k_copy_rows():
+        y.copy_(x[:P])
+
     # ---------------------------------------- per-kernel durations (same process)
     INNER = 20
     kernels = {"indexgen": k_indexgen, "dispatch": k_dispatch, "combine": k_combine,
                "combine_gather": k_combine_gather, "gate_topk_mask": k_gate,
                "gate_topk_mask_torch_ops": k_gate_torch,
                "tag_gather_unique": k_tag_unique, "tag_gather_sum": k_tag_sum,
-               "tag_gather_sum_torch_ops": k_tag_sum_torch}
+               "tag_gather_sum_torch_ops": k_tag_sum_torch, "plain_copy_of_the_rows": k_copy_rows}
     if have_ffn:
         kernels.update({"ffn_gemm1_gelu": k_gemm1, "ffn_gemm2": k_gemm2,
                         "indexgen_tags": k_indexgen_tags, "ffn_gemm1_gelu_gather": k_gemm1_gather,
@@ -404,6 +409,7 @@ def main():
     flops["ffn_gemm2_scatter"] = flops["ffn_gemm2"]
     bytes_["indexgen_tags"] = bytes_["indexgen"]
     bytes_["gate_topk_mask"] = 2 * idx_bytes  # fp32 scores in, int32 mask out
+    bytes_["plain_copy_of_the_rows"] = 2 * min(P, T) * D * es
     bytes_["tag_gather_sum"] = 2 * P * D * es + 8 * P + 4 * (2 * P)  # rows in/out, index, lists
     dc_bytes = bytes_["dispatch"] + bytes_["combine"]
     dc_us = us["dispatch"] + us["combine"]
