@@ -440,9 +440,11 @@ __global__ __launch_bounds__(WAVES * 64) void grouped_gemm_kernel(GemmArgs a) {
           const int tag = a.tags[static_cast<size_t>(seat0 + r) * a.E + e];
           to = (tag >= 1 && tag <= a.T) ? tag - 1 : -1;
         }
+        // streaming stores: the output is not read again by this kernel, and written through the
+        // L2 like ordinary stores it pushes the operand lines out that the column tiles share
         if (to >= 0 && n0 + c * 8 < a.N)
-          *reinterpret_cast<u32x4*>(oc + static_cast<size_t>(to) * a.N + c * 8) =
-              *reinterpret_cast<const u32x4*>(stage_out + rl * OUT_ROW + c * 16);
+          __builtin_nontemporal_store(*reinterpret_cast<const u32x4*>(stage_out + rl * OUT_ROW + c * 16),
+                                      reinterpret_cast<u32x4*>(oc + static_cast<size_t>(to) * a.N + c * 8));
       }
     }
     if (nt + 1 < nt_end) {
@@ -485,7 +487,7 @@ int launch_act(GemmArgs& a, hipStream_t st) {
   // from the row blocks a capacity-filled route has; the loads themselves live on the device).
   static const int forced_walk = std::getenv("BRT_GEMM_WALK") ? std::atoi(std::getenv("BRT_GEMM_WALK")) : 0;
   a.walk = 1;
-  if (WAVES == 4) {  // the narrower tiles stage more per thread and have no registers left for it
+  if (WAVES == 4 || WAVES == 8) {  // the narrower tiles stage more per thread and have no registers left for it
     const long slots = static_cast<long>(device_cus()) * (WAVES == 2 ? 2 : 1);
     const long row_blocks = estimated_row_blocks(a.P, a.E);
     const long plain = (row_blocks * a.tiles_n + slots - 1) / slots;
@@ -578,6 +580,8 @@ int grouped_gemm_impl(const void* x, const void* const* weights, const void* con
   if (shape == 24) return launch<5, 2, 4>(a, act, as_stream(stream));
   if (shape == 23) return launch<5, 2, 3>(a, act, as_stream(stream));
   if (shape == 22) return launch<5, 2, 2>(a, act, as_stream(stream));
+  if (shape == 18) return launch<5, 1, 8>(a, act, as_stream(stream));
+  if (shape == 16) return launch<5, 1, 6>(a, act, as_stream(stream));
   return launch<5, 1, 4>(a, act, as_stream(stream));
 }
 
