@@ -94,6 +94,11 @@ __device__ __forceinline__ float apply_act(float v) {
   return v;
 }
 
+// Cache policy of the weight loads (auxiliary operand of the buffer load: bit 1 = non-temporal on
+// gfx94x/gfx950).  Every weight byte is read exactly once per launch; loaded as a stream it does
+// not push the activation rows, which the column tiles of a row block share, out of the L2.
+constexpr int kStreamingLoad = 2;
+
 template <int N>
 struct Staged {
   u32x4 v[N];
@@ -232,7 +237,7 @@ __global__ __launch_bounds__(WAVES * 64) void grouped_gemm_kernel(GemmArgs a) {
           s.v[i] = __builtin_amdgcn_raw_buffer_load_b128(res_a, off_a[i < A_LOADS ? i : 0], k0 * 2, 0);
       } else {
         s.v[i] = __builtin_amdgcn_raw_buffer_load_b128(res_b, off_b[i >= A_LOADS ? i - A_LOADS : 0],
-                                                       k0 * 2, 0);
+                                                       k0 * 2, kStreamingLoad);
       }
     }
   };
