@@ -492,7 +492,7 @@ int launch_act(GemmArgs& a, hipStream_t st) {
   // from the row blocks a capacity-filled route has; the loads themselves live on the device).
   static const int forced_walk = std::getenv("BRT_GEMM_WALK") ? std::atoi(std::getenv("BRT_GEMM_WALK")) : 0;
   a.walk = 1;
-  if (WAVES == 4 || WAVES == 8) {  // the narrower tiles stage more per thread and have no registers left for it
+  if (WAVES == 4) {  // the narrower tiles stage more per thread and have no registers left for it
     const long slots = static_cast<long>(device_cus()) * (WAVES == 2 ? 2 : 1);
     const long row_blocks = estimated_row_blocks(a.P, a.E);
     const long plain = (row_blocks * a.tiles_n + slots - 1) / slots;
@@ -585,8 +585,6 @@ int grouped_gemm_impl(const void* x, const void* const* weights, const void* con
   if (shape == 24) return launch<5, 2, 4>(a, act, as_stream(stream));
   if (shape == 23) return launch<5, 2, 3>(a, act, as_stream(stream));
   if (shape == 22) return launch<5, 2, 2>(a, act, as_stream(stream));
-  if (shape == 18) return launch<5, 1, 8>(a, act, as_stream(stream));
-  if (shape == 16) return launch<5, 1, 6>(a, act, as_stream(stream));
   return launch<5, 1, 4>(a, act, as_stream(stream));
 }
 
