@@ -805,9 +805,11 @@ __global__ __launch_bounds__(kBlock, 8) void dispatch_lean_kernel(DispatchArgs a
                 unpack<DT, 16>(val[u], x);
 #pragma unroll
                 for (int q = 0; q < NE; ++q) x[q] = x[q] * g;
-                pack_store<DT, NE>(to, x);
+                pack_store<DT, NE, true>(to, x);
               } else {
-                *to = val[u];
+                // streaming store: the row is not read again by this kernel, and written through the
+                // L2 like an ordinary store it evicts source rows and index words still to be read
+                __builtin_nontemporal_store(val[u], to);
               }
             }
           }
@@ -925,7 +927,7 @@ __global__ __launch_bounds__(kBlock) void combine_lean_kernel(CombineArgs a) {
 #pragma unroll
           for (int u = 0; u < UPR; ++u) {
             const int off = off0 + u * LPR + glane;
-            if (off < cpr) pack_store<OUT_DT, NE>(dst + (to + off) * OUT_BYTES, acc[u]);
+            if (off < cpr) pack_store<OUT_DT, NE, true>(dst + (to + off) * OUT_BYTES, acc[u]);
           }
         }
       }
@@ -980,11 +982,12 @@ __global__ __launch_bounds__(kBlock) void combine_rows_kernel(CombineRowsArgs a)
           const int off = off0 + u * LPR + glane;
           if (off < cpr) {
             if constexpr (IN_DT == OUT_DT) {
-              *reinterpret_cast<U*>(dst + (to + off) * 16) = val[u];
+              // streaming store, as in dispatch: nothing here reads the row again
+              __builtin_nontemporal_store(val[u], reinterpret_cast<U*>(dst + (to + off) * 16));
             } else {
               float x[NE];
               unpack<IN_DT, 16>(val[u], x);
-              pack_store<OUT_DT, NE>(dst + (to + off) * OUT_BYTES, x);
+              pack_store<OUT_DT, NE, true>(dst + (to + off) * OUT_BYTES, x);
             }
           }
         }

@@ -46,25 +46,33 @@ __device__ __forceinline__ void unpack(const typename Unit<BYTES>::type& v,
   }
 }
 
+// One store of a native unit; STREAM marks it non-temporal (written past the L2: for rows that
+// the kernel does not read again, so that they do not evict data it still has to read).
+template <bool STREAM, typename V>
+__device__ __forceinline__ void store_unit(V* p, const V& v) {
+  if constexpr (STREAM) __builtin_nontemporal_store(v, p);
+  else *p = v;
+}
+
 // Packs N fp32 values to DT (round to nearest even) and stores them at p.
-template <int DT, int N>
+template <int DT, int N, bool STREAM = false>
 __device__ __forceinline__ void pack_store(void* p, const float (&x)[N]) {
   if constexpr (DT == BRT_F32) {
     if constexpr (N % 4 == 0) {
 #pragma unroll
       for (int i = 0; i < N / 4; ++i) {
         f32x4 o = {x[4 * i], x[4 * i + 1], x[4 * i + 2], x[4 * i + 3]};
-        static_cast<f32x4*>(p)[i] = o;
+        store_unit<STREAM>(static_cast<f32x4*>(p) + i, o);
       }
     } else if constexpr (N == 2) {
       f32x2 o = {x[0], x[1]};
-      *static_cast<f32x2*>(p) = o;
+      store_unit<STREAM>(static_cast<f32x2*>(p), o);
     } else {
-      *static_cast<float*>(p) = x[0];
+      store_unit<STREAM>(static_cast<float*>(p), x[0]);
     }
   } else {
     if constexpr (N == 1) {
-      *static_cast<uint16_t*>(p) = static_cast<uint16_t>(float_to_half_bits<DT>(x[0]));
+      store_unit<STREAM>(static_cast<uint16_t*>(p), static_cast<uint16_t>(float_to_half_bits<DT>(x[0])));
     } else {
       uint32_t w[N / 2];
 #pragma unroll
@@ -72,12 +80,12 @@ __device__ __forceinline__ void pack_store(void* p, const float (&x)[N]) {
         w[i] = float_to_half_bits<DT>(x[2 * i]) | (float_to_half_bits<DT>(x[2 * i + 1]) << 16);
       if constexpr (N == 8) {
         u32x4 o = {w[0], w[1], w[2], w[3]};
-        *static_cast<u32x4*>(p) = o;
+        store_unit<STREAM>(static_cast<u32x4*>(p), o);
       } else if constexpr (N == 4) {
         u32x2 o = {w[0], w[1]};
-        *static_cast<u32x2*>(p) = o;
+        store_unit<STREAM>(static_cast<u32x2*>(p), o);
       } else {
-        *static_cast<uint32_t*>(p) = w[0];
+        store_unit<STREAM>(static_cast<uint32_t*>(p), w[0]);
       }
     }
   }
