@@ -927,7 +927,9 @@ __global__ __launch_bounds__(kBlock) void combine_lean_kernel(CombineArgs a) {
 #pragma unroll
           for (int u = 0; u < UPR; ++u) {
             const int off = off0 + u * LPR + glane;
-            if (off < cpr) pack_store<OUT_DT, NE, true>(dst + (to + off) * OUT_BYTES, acc[u]);
+            // streamed only when a wavefront's store covers whole lines: a widening store writes two
+            // 16-byte halves per lane, which have to meet in the L2 first
+            if (off < cpr) pack_store<OUT_DT, NE, IN_DT == OUT_DT>(dst + (to + off) * OUT_BYTES, acc[u]);
           }
         }
       }
@@ -987,7 +989,7 @@ __global__ __launch_bounds__(kBlock) void combine_rows_kernel(CombineRowsArgs a)
             } else {
               float x[NE];
               unpack<IN_DT, 16>(val[u], x);
-              pack_store<OUT_DT, NE, true>(dst + (to + off) * OUT_BYTES, x);
+              pack_store<OUT_DT, NE>(dst + (to + off) * OUT_BYTES, x);
             }
           }
         }
