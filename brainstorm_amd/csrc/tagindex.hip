@@ -270,7 +270,7 @@ __global__ __launch_bounds__(256) void sum_rows_by_index_kernel(SumArgs a) {
         }
       }
     }
-    if (live) pack_store<OUT_DT, NE>(dst + static_cast<size_t>(off) * OUT_BYTES, acc);
+    if (live) pack_store<OUT_DT, NE, IN_DT == OUT_DT>(dst + static_cast<size_t>(off) * OUT_BYTES, acc);  // streamed when not widening
   }
 }
 
