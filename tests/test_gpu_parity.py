@@ -504,3 +504,24 @@ def test_config4_swin_small_rows_full_size(hip):
     assert same_bits(out, oracle.combine(y, idx, loads, max_path_padding=True, in_dtype="f16"))
     kept = thr.any(1)
     assert np.array_equal(out[kept], x[kept]) and not out[~kept].any()
+
+
+def test_tag_index_gather_full_size_properties(hip):
+    """At the largest configured size (100352 rows of 96 fp16 values) the CPU oracle is too slow to
+    be the checker, so the result is pinned by what the operation must satisfy: the unique tags of
+    a permutation are 1..n and the inverse is the permutation itself; summing rows by a permutation
+    moves every row unchanged; summing pairs (index p // 2) gives the fp32 sum of two rows rounded
+    once."""
+    n, cell = 100352, 96
+    rng = np.random.default_rng(8)
+    perm = rng.permutation(n).astype(np.int32)
+    unique, inverse = hip.unique_tags(perm + 1)
+    assert np.array_equal(unique, np.arange(1, n + 1, dtype=np.int32))
+    assert np.array_equal(inverse, perm.astype(np.int64))
+    x = rng.standard_normal((n, cell)).astype(np.float16)
+    bits = x.view(np.uint16)
+    moved = hip.combine_by_index(bits, inverse, n, "f16")
+    assert np.array_equal(moved[perm], bits)
+    pairs = hip.combine_by_index(bits, (np.arange(n) // 2).astype(np.int32), n // 2, "f16")
+    want = (x[0::2].astype(np.float32) + x[1::2].astype(np.float32)).astype(np.float16)
+    assert np.array_equal(pairs.view(np.float16), want)
