@@ -743,6 +743,13 @@ __global__ __launch_bounds__(kBlock, 8) void dispatch_lean_kernel(DispatchArgs a
   const U* __restrict__ src = static_cast<const U*>(a.src);
   U* __restrict__ dst = static_cast<U*>(a.dst);
 
+  // Rows of more than 128 bytes (lane groups of 16 and more) are written with streaming stores;
+  // shorter rows are scattered partial lines, which are faster merged in the L2 (measured: 16- and
+  // 32-byte rows lose 5-10 % when streamed, 80-byte rows 12 % in the combine; rows of 144 bytes and
+  // more gain 5-20 %).  The
+  // choice is a compile-time property of the shape: chosen by a branch at run time, the compiler
+  // merges the two stores into an ordinary one.
+  constexpr bool kStream = LS >= 4;
   int v_next = (n_steps > 0 && sub < nr && e < E) ? idx0[sub * E + e] : 0;
   const int my_count = (a.counts != nullptr && lane < E) ? a.counts[lane] : 0;
   const SmallTables tab = small_tables(a.loads, E, a.mpl, ep_shift, lane);
@@ -805,11 +812,11 @@ __global__ __launch_bounds__(kBlock, 8) void dispatch_lean_kernel(DispatchArgs a
                 unpack<DT, 16>(val[u], x);
 #pragma unroll
                 for (int q = 0; q < NE; ++q) x[q] = x[q] * g;
-                pack_store<DT, NE, true>(to, x);
+                pack_store<DT, NE, kStream>(to, x);
               } else {
                 // streaming store: the row is not read again by this kernel, and written through the
                 // L2 like an ordinary store it evicts source rows and index words still to be read
-                __builtin_nontemporal_store(val[u], to);
+                store_unit<kStream>(to, val[u]);
               }
             }
           }
@@ -928,8 +935,10 @@ __global__ __launch_bounds__(kBlock) void combine_lean_kernel(CombineArgs a) {
           for (int u = 0; u < UPR; ++u) {
             const int off = off0 + u * LPR + glane;
             // streamed only when a wavefront's store covers whole lines: a widening store writes two
-            // 16-byte halves per lane, which have to meet in the L2 first
-            if (off < cpr) pack_store<OUT_DT, NE, IN_DT == OUT_DT>(dst + (to + off) * OUT_BYTES, acc[u]);
+            // 16-byte halves per lane, which have to meet in the L2 first, and so do rows of up to 128 bytes
+            if (off < cpr) {
+              pack_store<OUT_DT, NE, IN_DT == OUT_DT && LS >= 4>(dst + (to + off) * OUT_BYTES, acc[u]);
+            }
           }
         }
       }
@@ -984,8 +993,8 @@ __global__ __launch_bounds__(kBlock) void combine_rows_kernel(CombineRowsArgs a)
           const int off = off0 + u * LPR + glane;
           if (off < cpr) {
             if constexpr (IN_DT == OUT_DT) {
-              // streaming store, as in dispatch: nothing here reads the row again
-              __builtin_nontemporal_store(val[u], reinterpret_cast<U*>(dst + (to + off) * 16));
+              // streaming store, as in dispatch (rows of more than 128 bytes): nothing here reads the row again
+              store_unit<LS >= 4>(reinterpret_cast<U*>(dst + (to + off) * 16), val[u]);
             } else {
               float x[NE];
               unpack<IN_DT, 16>(val[u], x);
@@ -1078,7 +1087,8 @@ bool launch_shape(long T, int rows_pw, int lds_pw_ints, LaunchShape* out) {
   else if (a.cpr > 32) { LAUNCH(6, 1) }                \
   else if (a.cpr > 16) { LAUNCH(5, 1) }                \
   else if (a.cpr > 8) { LAUNCH(4, 1) }                 \
-  else { LAUNCH(3, 1) }
+  else if (a.cpr > 4) { LAUNCH(3, 1) }                 \
+  else { LAUNCH(2, 1) }
 
 template <int BYTES, int DT>
 void launch_dispatch(const DispatchArgs& a, const LaunchShape& sh, hipStream_t st) {
@@ -1273,7 +1283,8 @@ extern "C" int brt_hip_combine_by_tags(const void* src, void* dst, const int32_t
     else if (a.cpr > 32) launch(integral_constant<int, 6>{}, integral_constant<int, 1>{});          \
     else if (a.cpr > 16) launch(integral_constant<int, 5>{}, integral_constant<int, 1>{});          \
     else if (a.cpr > 8) launch(integral_constant<int, 4>{}, integral_constant<int, 1>{});           \
-    else launch(integral_constant<int, 3>{}, integral_constant<int, 1>{});                          \
+    else if (a.cpr > 4) launch(integral_constant<int, 3>{}, integral_constant<int, 1>{});           \
+    else launch(integral_constant<int, 2>{}, integral_constant<int, 1>{});                          \
   }
   if (in_dtype == BRT_F32) BRT_ROWS_LAUNCH(BRT_F32, BRT_F32)
   else if (in_dtype == BRT_F16 && out_dtype == BRT_F16) BRT_ROWS_LAUNCH(BRT_F16, BRT_F16)

@@ -270,7 +270,9 @@ __global__ __launch_bounds__(256) void sum_rows_by_index_kernel(SumArgs a) {
         }
       }
     }
-    if (live) pack_store<OUT_DT, NE, IN_DT == OUT_DT>(dst + static_cast<size_t>(off) * OUT_BYTES, acc);  // streamed when not widening
+    // streamed when not widening and the rows are whole 16-byte units (the case of the expert
+    // outputs this op exists for); narrower units mean short or odd rows, better merged in the L2
+    if (live) pack_store<OUT_DT, NE, IN_DT == OUT_DT && BYTES == 16>(dst + static_cast<size_t>(off) * OUT_BYTES, acc);
   }
 }
 
