@@ -79,6 +79,24 @@ SIGNATURES = {
         [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_size, _c_int, _c_int,
          _c_ptr],
     ),
+    "brt_hip_gate_topk": (
+        _c_int,
+        [_c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
+    ),
+    "brt_hip_route_by_path": (
+        _c_int,
+        [_c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr,
+         _c_ptr, _c_int, _c_ptr],
+    ),
+    "brt_hip_dispatch_by_rows": (
+        _c_int,
+        [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    ),
+    "brt_hip_combine_by_rows": (
+        _c_int,
+        [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
+         _c_ptr],
+    ),
 }
 
 _lib = None

@@ -76,6 +76,20 @@ __device__ __forceinline__ float load_gate(const void* gates, int dtype, size_t 
   return dtype == BRT_F16 ? f16_to_float(h) : bf16_to_float(h);
 }
 
+// Load of a path from its real row count (src/router/location.cu:227-254): the path's own
+// capacity when padding path-wise (even for an empty path); 0 for an empty path; the count itself
+// without a capacity menu; else the smallest capacity that holds the count (the count itself when
+// not padding), and the last capacity when none does.
+__device__ __forceinline__ int finalize_load(int real, const int* caps, int C, int cap_pad,
+                                             int path_pad, int col) {
+  if (path_pad) return caps[col];  // unconditional, even for an empty path
+  if (real == 0) return 0;
+  if (C == 0) return real;
+  for (int i = 0; i < C; ++i)
+    if (real <= caps[i]) return cap_pad ? caps[i] : real;
+  return caps[C - 1];
+}
+
 // Fills s_val[e] = g[e] and s_start[e] = exclusive prefix of g (or e*stride when
 // stride != 0) for e < E, using the first wavefront of the block.  The caller
 // must __syncthreads() afterwards.

@@ -115,16 +115,6 @@ struct ScanArgs {
   int ep_shift, rows_pw, bands;
 };
 
-__device__ __forceinline__ int finalize_load(int real, const int* caps, int C, int cap_pad,
-                                             int path_pad, int col) {
-  if (path_pad) return caps[col];  // unconditional, even for an empty path
-  if (real == 0) return 0;
-  if (C == 0) return real;
-  for (int i = 0; i < C; ++i)
-    if (real <= caps[i]) return cap_pad ? caps[i] : real;
-  return caps[C - 1];
-}
-
 // Sum over the lanes that hold the same path (lanes e, e+ep, e+2ep, ...); every
 // lane ends up with the total.
 __device__ __forceinline__ int sum_over_rows_in_wave(int v, int ep_shift) {

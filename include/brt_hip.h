@@ -253,6 +253,58 @@ int brt_hip_combine_by_index(const void* in_data, void* out_data, const void* in
                              int P, int cell, int n_out, void* workspace, size_t workspace_bytes,
                              int in_dtype, int out_dtype, void* stream);
 
+/* ---------------------------------------------------------------------------
+ * Compact route format (no counterpart in the reference's extension; it replaces, for routes
+ * with k chosen paths per cell, the dense [T,E] hot mask and seat matrix that the reference
+ * passes from protocol to fabric: python/brt/router/protocol/topk.py:26-31,
+ * src/router/location.cu:212-257, src/router/route.cu:13-282).
+ *
+ *   path_ids    [T,k] int32  paths of a cell, all different; an id outside [0,E) is no route
+ *   weights     [T,k] fp32   gate value of each entry
+ *   seat_rows   [T,k] int32  1-based row of the dispatched buffer of entry (t,j); 0 = dropped
+ *   row_entries [P]   int32  1-based entry number t*k+j+1 of each dispatched row; 0 = padding
+ *                            (for k == 1 this is the new_tags output of brt_hip_dispatch)
+ *
+ * brt_hip_gate_topk: scores [T,E] (fp32/fp16/bf16) -> path_ids in the order of selection
+ *   (largest first, NaN above every number, lowest column among equals, as
+ *   brt_hip_topk_hot_mask), weights (or NULL) = the chosen scores as fp32, or with softmax != 0
+ *   their softmax over the row (fp32, exp(x - max) / sum: the Switch router's probabilities,
+ *   benchmark/switch_moe/switch_transformer.py:240-253), and optionally the dense hot_mask
+ *   (or NULL).  One launch; E <= 1024.
+ *
+ * brt_hip_route_by_path: what brt_hip_generate_indices_and_loads computes from the mask,
+ *   from path_ids: loads [E] by the same capacity rules, counts [E] (or NULL) the real row
+ *   counts, seat_rows and row_entries.  Seats of a path go to its cells in ascending cell
+ *   order; entry (t,j) of path e with seat s <= loads[e] owns row start[e] + s, start[e] = sum
+ *   of the loads before e, or e * max_path_load when max_path_load != 0 (seats beyond
+ *   max_path_load are dropped then).  Rows beyond P are dropped; row_entries is written whole
+ *   ([0,P)), it needs no zero fill.  One workgroup: E <= 512, T*k < 2^24, meant for routes of up
+ *   to a few 10^4 entries.  No workspace.
+ *
+ * brt_hip_dispatch_by_rows: dst[r] = src[(row_entries[r]-1) / k] (times weights[row_entries[r]-1]
+ *   when weights != NULL, rounded once to the data type), zero rows where row_entries[r] == 0.
+ *   dst [P,cell] is written whole.  Rows must be whole 16-byte units.
+ *
+ * brt_hip_combine_by_rows: dst[t] = sum over the entries j of cell t with seat_rows[t,j] != 0,
+ *   in ascending path id, of weights[t,j] * src[seat_rows[t,j]-1] (weights NULL = 1), in fp32 from 0
+ *   with product and sum rounded separately: the order and roundings of brt_hip_combine.  Cells
+ *   without a row keep dst when is_residual != 0 and are zeroed otherwise.  k <= 8; dtypes as
+ *   brt_hip_combine.
+ */
+int brt_hip_gate_topk(const void* scores, int T, int E, int k, int dtype, int softmax,
+                      int32_t* path_ids, float* weights, int32_t* hot_mask, void* stream);
+int brt_hip_route_by_path(const int32_t* path_ids, int T, int k, int E, const int32_t* caps, int C,
+                          int capacity_padding, int path_wise_padding, int max_path_load,
+                          int32_t* loads, int32_t* counts, int32_t* seat_rows,
+                          int32_t* row_entries, int P, void* stream);
+int brt_hip_dispatch_by_rows(const void* src, void* dst, const float* weights,
+                             const int32_t* row_entries, int P, int T, int k, int cell, int dtype,
+                             void* stream);
+int brt_hip_combine_by_rows(const void* src, void* dst, const float* weights,
+                            const int32_t* path_ids, const int32_t* seat_rows, int T, int k,
+                            int cell, int P, int is_residual, int in_dtype, int out_dtype,
+                            void* stream);
+
 #ifdef __cplusplus
 }
 #endif

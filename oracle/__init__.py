@@ -122,6 +122,80 @@ def topk_hot_mask(score, k: int) -> np.ndarray:
     return mask
 
 
+def gate_topk(score, k: int, softmax: bool = False) -> Tuple[np.ndarray, np.ndarray]:
+    """Compact form of the gate: the ``k`` chosen paths of every cell in the order of selection
+    (the order of ``torch.topk``: largest first, NaN on top, lowest column among equals) and
+    their weights: the scores, or their softmax over the row (evaluated in fp64, rounded to fp32)."""
+    score = np.ascontiguousarray(score, dtype=np.float32)
+    T, E = score.shape
+    assert 0 <= k <= E
+    ids = np.zeros((T, k), dtype=np.int32)
+    weights = np.zeros((T, k), dtype=np.float32)
+    lib().oracle_gate_topk(_p(score), T, E, int(k), int(softmax), _p(ids), _p(weights))
+    return ids, weights
+
+
+def route_by_path(path_ids, E: int, supported_capacities=None, capacity_padding: bool = False,
+                  path_wise_padding: bool = False, max_path_load: int = 0, P: Optional[int] = None):
+    """``generate_indices_and_loads`` on a route given as path ids ``[T, k]``.  Returns
+    ``(loads [E], counts [E], seat_rows [T, k], row_entries [P])``; ``P`` defaults to ``T * k``
+    (``E * max_path_load`` when padding to the largest path)."""
+    ids = _i32(path_ids)
+    T, k = ids.shape
+    caps = None if supported_capacities is None else _i32(supported_capacities)
+    if P is None:
+        P = E * max_path_load if max_path_load else T * k
+    loads = np.zeros((E,), dtype=np.int32)
+    counts = np.zeros((E,), dtype=np.int32)
+    seat_rows = np.zeros((T, k), dtype=np.int32)
+    row_entries = np.zeros((P,), dtype=np.int32)
+    lib().oracle_route_by_path(_p(ids), T, k, E, _p(caps), 0 if caps is None else caps.size,
+                               int(capacity_padding), int(path_wise_padding), int(max_path_load),
+                               _p(loads), _p(counts), _p(seat_rows), _p(row_entries), int(P))
+    return loads, counts, seat_rows, row_entries
+
+
+def dispatch_by_rows(in_data, row_entries, k: int, weights=None, dtype: str = "f32") -> np.ndarray:
+    """``out[r] = in_data[(row_entries[r]-1) // k]`` (times the entry's fp32 weight, rounded once),
+    zero rows where ``row_entries[r] == 0``."""
+    x = _data(in_data, dtype)
+    T = x.shape[0]
+    x = x.reshape(T, -1) if T > 0 else x.reshape(0, int(np.prod(x.shape[1:])))
+    cell = x.shape[1]
+    entries = _i32(row_entries).reshape(-1)
+    P = entries.size
+    w = None if weights is None else np.ascontiguousarray(weights, dtype=np.float32).reshape(-1)
+    out = np.zeros((P, cell), dtype=_NP[dtype])
+    if P > 0 and cell > 0:
+        lib().oracle_dispatch_by_rows(_p(x), _p(out), _p(w), _p(entries), P, T, int(k), cell, _DT[dtype])
+    return out
+
+
+def combine_by_rows(in_data, path_ids, seat_rows, weights=None, out_data=None,
+                    in_dtype: str = "f32", out_dtype: Optional[str] = None) -> np.ndarray:
+    """``out[t] = sum_j weights[t,j] * in_data[seat_rows[t,j]-1]`` over the entries that own a row,
+    in ascending path id, fp32 from 0; cells without a row keep ``out_data`` (or are zero)."""
+    out_dtype = out_dtype or in_dtype
+    ids = _i32(path_ids)
+    rows = _i32(seat_rows)
+    T, k = ids.shape
+    x = _data(in_data, in_dtype)
+    P = x.shape[0]
+    x = x.reshape(P, -1) if P > 0 else x.reshape(0, int(np.prod(x.shape[1:])))
+    cell = x.shape[1]
+    w = None if weights is None else np.ascontiguousarray(weights, dtype=np.float32).reshape(T, k)
+    if out_data is not None:
+        out = _data(out_data, out_dtype).reshape(T, cell).copy()
+        residual = 1
+    else:
+        out = np.zeros((T, cell), dtype=_NP[out_dtype])
+        residual = 0
+    if T > 0 and cell > 0:
+        lib().oracle_combine_by_rows(_p(x), _p(out), _p(w), _p(ids), _p(rows), T, k, cell, P, residual,
+                                     _DT[in_dtype], _DT[out_dtype])
+    return out
+
+
 def unique_tags(tags) -> Tuple[np.ndarray, np.ndarray]:
     """``_unique(tags, sorted=True, return_inverse=True)`` of ``fuse_split_cells_from_paths``
     (router.cc:362-366): ascending distinct tags and the position of every input tag in them

@@ -11,6 +11,7 @@
  *   src/backend/torch/router.cc   shape/dtype conventions around them
  *   python/brt/router/protocol/topk.py:26-31   top-k hot mask (torch.topk + scatter_)
  *   src/backend/torch/router.cc:348-369,449-472   tag-index gather (_unique + scatter_reduce)
+ *   the same route held as k path ids per cell (compact format; restated from the dense ops)
  *
  * Only tests, the smoke check and the bench's cpu_baseline leg may link or call
  * this file; the product path never does.
@@ -31,6 +32,7 @@
 #include <stddef.h>
 #include <string.h>
 #include <stdlib.h>
+#include <math.h>
 
 enum { ORACLE_F32 = 0, ORACLE_F16 = 1, ORACLE_BF16 = 2 };
 
@@ -400,6 +402,120 @@ void oracle_topk_hot_mask(const float* score, int32_t* mask, int T, int E, int k
       out[best] = 1;
     }
   }
+}
+
+/* ---------- compact route format ----------
+ * The same route as the dense mask / seat matrix, held as k path ids per cell.  No function of
+ * the reference has this signature; each restates what the reference computes on the dense
+ * form and is pinned by converting to and from that form (tests/test_oracle.py):
+ *   gate_topk       topk.py:26-31 (selection), switch_transformer.py:240-253 (softmax in fp32)
+ *   route_by_path   location.cu:132-257 (seats in ascending cell order, load rules :222-256)
+ *   dispatch_by_rows / combine_by_rows   route.cu:13-282 on rows named directly */
+void oracle_gate_topk(const float* score, int T, int E, int k, int softmax, int32_t* ids,
+                      float* weights) {
+  char* taken = (char*)malloc((size_t)(E > 0 ? E : 1));
+  for (int t = 0; t < T; ++t) {
+    const float* row = score + (size_t)t * E;
+    double top = -HUGE_VAL, sum = 0.0;
+    if (softmax) {
+      for (int e = 0; e < E; ++e) if (row[e] > top) top = row[e];
+      for (int e = 0; e < E; ++e) sum += exp((double)row[e] - top);
+    }
+    memset(taken, 0, (size_t)E);
+    for (int pass = 0; pass < k && pass < E; ++pass) {
+      int best = -1;
+      for (int e = 0; e < E; ++e) {
+        if (taken[e]) continue;
+        if (best < 0 || score_greater(row[e], row[best])) best = e;
+      }
+      taken[best] = 1;
+      ids[(size_t)t * k + pass] = best;
+      if (weights)
+        weights[(size_t)t * k + pass] =
+            softmax ? (float)(exp((double)row[best] - top) / sum) : row[best];
+    }
+  }
+  free(taken);
+}
+
+void oracle_route_by_path(const int32_t* ids, int T, int k, int E, const int32_t* caps, int C,
+                          int capacity_padding, int path_wise_padding, int max_path_load,
+                          int32_t* loads, int32_t* counts, int32_t* seat_rows,
+                          int32_t* row_entries, int P) {
+  /* the dense mask of the same route, then the dense scan (pinned above) on it */
+  int32_t* mask = (int32_t*)calloc((size_t)T * E + 1, sizeof(int32_t));
+  int32_t* seats = (int32_t*)calloc((size_t)T * E + 1, sizeof(int32_t));
+  for (int t = 0; t < T; ++t)
+    for (int j = 0; j < k; ++j) {
+      int e = ids[(size_t)t * k + j];
+      if (e >= 0 && e < E) mask[(size_t)t * E + e] = 1;
+    }
+  oracle_generate_indices_and_loads(mask, seats, loads, T, E, caps, C, capacity_padding,
+                                    path_wise_padding, 0);
+  for (int e = 0; e < E; ++e) {
+    int c = 0;
+    for (int t = 0; t < T; ++t) c += mask[(size_t)t * E + e];
+    if (counts) counts[e] = c;
+  }
+  for (int r = 0; r < P; ++r) row_entries[r] = 0;
+  for (int t = 0; t < T; ++t)
+    for (int j = 0; j < k; ++j) {
+      int e = ids[(size_t)t * k + j];
+      int32_t row = 0;
+      if (e >= 0 && e < E) {
+        long start = 0;
+        for (int q = 0; q < e; ++q) start += loads[q];
+        if (max_path_load != 0) start = (long)e * max_path_load;
+        int seat = seats[(size_t)t * E + e];
+        int limit = loads[e];
+        if (max_path_load != 0 && limit > max_path_load) limit = max_path_load;
+        if (seat >= 1 && seat <= limit && start + seat <= P) row = (int32_t)(start + seat);
+      }
+      seat_rows[(size_t)t * k + j] = row;
+      if (row != 0) row_entries[row - 1] = t * k + j + 1;
+    }
+  free(mask);
+  free(seats);
+}
+
+void oracle_dispatch_by_rows(const void* src, void* dst, const float* weights,
+                             const int32_t* row_entries, int P, int T, int k, int cell, int dtype) {
+  for (int r = 0; r < P; ++r) {
+    int entry = row_entries[r];
+    for (int j = 0; j < cell; ++j) {
+      float v = 0.0f;
+      if (entry >= 1 && entry <= T * k) {
+        v = load_elem(src, dtype, (size_t)((entry - 1) / k) * cell + j);
+        if (weights) v = v * weights[entry - 1];
+      }
+      store_elem(dst, dtype, (size_t)r * cell + j, v);
+    }
+  }
+}
+
+void oracle_combine_by_rows(const void* src, void* dst, const float* weights, const int32_t* ids,
+                            const int32_t* seat_rows, int T, int k, int cell, int P,
+                            int is_residual, int in_dtype, int out_dtype) {
+  for (int t = 0; t < T; ++t)
+    for (int j = 0; j < cell; ++j) {
+      float acc = 0.0f;
+      int any = 0, last = -1;
+      for (;;) { /* entries with a row, by ascending path id */
+        int pick = -1;
+        for (int q = 0; q < k; ++q) {
+          int row = seat_rows[(size_t)t * k + q], e = ids[(size_t)t * k + q];
+          if (row < 1 || row > P || e <= last) continue;
+          if (pick < 0 || e < ids[(size_t)t * k + pick]) pick = q;
+        }
+        if (pick < 0) break;
+        last = ids[(size_t)t * k + pick];
+        float v = load_elem(src, in_dtype, (size_t)(seat_rows[(size_t)t * k + pick] - 1) * cell + j);
+        if (weights) v = v * weights[(size_t)t * k + pick];
+        acc = acc + v;
+        any = 1;
+      }
+      if (any || !is_residual) store_elem(dst, out_dtype, (size_t)t * cell + j, acc);
+    }
 }
 
 /* ---------- tag-index gather (router.cc:348-369, 449-472) ----------

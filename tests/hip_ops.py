@@ -226,3 +226,83 @@ def combine_by_index(y_bits, index, n_out, in_dtype="f32", out_dtype=None):
         DT[in_dtype], DT[out_dtype], stream()))
     torch.cuda.synchronize()
     return host(d_out, True)
+
+
+def gate_topk(score_bits, k, dtype="f32", softmax=False, want_mask=False):
+    """-> (path_ids [T,k], weights [T,k] fp32[, hot_mask])."""
+    score_bits = np.ascontiguousarray(score_bits)
+    T, E = score_bits.shape
+    d_s = dev(score_bits)
+    d_ids = torch.full((T, k), -7, dtype=torch.int32, device="cuda")
+    d_w = torch.full((T, k), float("nan"), device="cuda")
+    d_m = torch.full((T, E), -7, dtype=torch.int32, device="cuda") if want_mask else None
+    _lib.check(_lib.lib().brt_hip_gate_topk(ptr(d_s), T, E, k, DT[dtype], int(softmax), ptr(d_ids),
+                                            ptr(d_w), ptr(d_m), stream()))
+    torch.cuda.synchronize()
+    out = (host(d_ids), host(d_w))
+    return out + (host(d_m),) if want_mask else out
+
+
+def route_by_path(path_ids, E, caps=None, capacity_padding=False, path_wise_padding=False,
+                  max_path_load=0, P=None):
+    """-> (loads, counts, seat_rows, row_entries)."""
+    ids = np.ascontiguousarray(path_ids, dtype=np.int32)
+    T, k = ids.shape
+    if P is None:
+        P = E * max_path_load if max_path_load else T * k
+    d_ids = dev(ids)
+    d_caps = None if caps is None else dev(np.asarray(caps, dtype=np.int32))
+    d_loads = torch.full((E,), -7, dtype=torch.int32, device="cuda")
+    d_counts = torch.full((E,), -7, dtype=torch.int32, device="cuda")
+    d_rows = torch.full((T, k), -7, dtype=torch.int32, device="cuda")
+    d_entries = torch.full((P,), -7, dtype=torch.int32, device="cuda")
+    _lib.check(_lib.lib().brt_hip_route_by_path(
+        ptr(d_ids), T, k, E, ptr(d_caps), 0 if caps is None else len(caps), int(capacity_padding),
+        int(path_wise_padding), int(max_path_load), ptr(d_loads), ptr(d_counts), ptr(d_rows),
+        ptr(d_entries), P, stream()))
+    torch.cuda.synchronize()
+    return host(d_loads), host(d_counts), host(d_rows), host(d_entries)
+
+
+def dispatch_by_rows(x_bits, row_entries, k, weights=None, dtype="f32"):
+    x_bits = np.ascontiguousarray(x_bits)
+    T = x_bits.shape[0]
+    cell = x_bits.size // max(T, 1)
+    entries = np.ascontiguousarray(row_entries, dtype=np.int32).reshape(-1)
+    P = entries.size
+    d_x = dev(x_bits.reshape(T, -1))
+    d_e = dev(entries)
+    d_w = None if weights is None else dev(np.ascontiguousarray(weights, dtype=np.float32))
+    if dtype == "f32":
+        d_out = torch.full((P, cell), float("nan"), device="cuda")
+    else:
+        d_out = torch.full((P, cell), 0x55, dtype=torch.int16, device="cuda")
+    _lib.check(_lib.lib().brt_hip_dispatch_by_rows(ptr(d_x), ptr(d_out), ptr(d_w), ptr(d_e), P, T, k,
+                                                   cell, DT[dtype], stream()))
+    torch.cuda.synchronize()
+    return host(d_out, True)
+
+
+def combine_by_rows(y_bits, path_ids, seat_rows, weights=None, out_bits=None, in_dtype="f32",
+                    out_dtype=None):
+    out_dtype = out_dtype or in_dtype
+    y_bits = np.ascontiguousarray(y_bits)
+    ids = np.ascontiguousarray(path_ids, dtype=np.int32)
+    rows = np.ascontiguousarray(seat_rows, dtype=np.int32)
+    T, k = ids.shape
+    P = y_bits.shape[0]
+    cell = y_bits.size // max(P, 1)
+    d_y = dev(y_bits.reshape(P, -1))
+    d_w = None if weights is None else dev(np.ascontiguousarray(weights, dtype=np.float32))
+    if out_bits is not None:
+        d_out = dev(np.ascontiguousarray(out_bits).reshape(T, cell))
+    elif out_dtype == "f32":
+        d_out = torch.full((T, cell), float("nan"), device="cuda")
+    else:
+        d_out = torch.full((T, cell), 0x55, dtype=torch.int16, device="cuda")
+    d_ids, d_rows = dev(ids), dev(rows)
+    _lib.check(_lib.lib().brt_hip_combine_by_rows(
+        ptr(d_y), ptr(d_out), ptr(d_w), ptr(d_ids), ptr(d_rows), T, k, cell, P,
+        int(out_bits is not None), DT[in_dtype], DT[out_dtype], stream()))
+    torch.cuda.synchronize()
+    return host(d_out, True)

@@ -525,3 +525,135 @@ def test_tag_index_gather_full_size_properties(hip):
     pairs = hip.combine_by_index(bits, (np.arange(n) // 2).astype(np.int32), n // 2, "f16")
     want = (x[0::2].astype(np.float32) + x[1::2].astype(np.float32)).astype(np.float16)
     assert np.array_equal(pairs.view(np.float16), want)
+
+
+# ------------------------------------------------------------- compact route format
+def _compact_route(T, E, k, seed, hole=0.0, bias=None):
+    rng = np.random.default_rng(seed)
+    score = rng.random((T, E)) + (0 if bias is None else bias)
+    ids = np.argsort(-score, axis=1)[:, :k].astype(np.int32)
+    if hole:
+        ids[rng.random((T, k)) < hole] = -1
+    return ids
+
+
+@pytest.mark.parametrize("T,E,k,dtype", [
+    (8192, 64, 1, "f32"), (16384, 32, 2, "f32"), (100352, 8, 1, "f16"), (1000, 5, 3, "bf16"),
+    (777, 64, 8, "f32"), (513, 100, 7, "f32"), (300, 128, 2, "bf16"), (40, 1000, 9, "f32"), (7, 1, 1, "f32"),
+])
+def test_gate_topk_ids_bit_exact_weights_within_tolerance(hip, T, E, k, dtype):
+    rng = np.random.default_rng(T + E + k)
+    bits = as_dtype_bits((3 * rng.standard_normal((T, E))).astype(np.float32), dtype)
+    score = bits_to_f32(bits, dtype)
+    ids, w, mask = hip.gate_topk(bits, k, dtype, softmax=False, want_mask=True)
+    want_ids, want_w = oracle.gate_topk(score, k)
+    assert np.array_equal(ids, want_ids)
+    assert np.array_equal(w, want_w)                          # the scores themselves: exact
+    assert np.array_equal(mask, oracle.topk_hot_mask(score, k))
+    ids, p = hip.gate_topk(bits, k, dtype, softmax=True)
+    _, want_p = oracle.gate_topk(score, k, softmax=True)
+    assert np.array_equal(ids, want_ids)
+    # fp32 softmax against the fp64 one: tolerance 2e-6 relative (exp and the sum of E terms in fp32)
+    assert np.allclose(p, want_p, rtol=2e-6, atol=1e-30)
+
+
+@pytest.mark.parametrize("T,E,k,hole", [
+    (8192, 64, 1, 0.0), (16384, 32, 2, 0.0), (100352, 8, 1, 0.0), (1000, 5, 3, 0.2), (1, 4, 1, 0.0),
+    (63, 300, 4, 0.1), (5000, 512, 2, 0.0), (1025, 17, 8, 0.3),
+])
+@pytest.mark.parametrize("mode", ["plain", "clip", "pad", "pad_max", "short"])
+def test_route_by_path_bit_exact(hip, T, E, k, hole, mode):
+    ids = _compact_route(T, E, k, seed=T + k, hole=hole, bias=zipf_bias(E, 1.2, 3) if E == 32 else None)
+    cap = max(1, (T * k) // (2 * E))
+    caps = {"plain": None, "short": None, "clip": [cap], "pad": [cap, 4 * cap, T], "pad_max": [cap, 4 * cap, T]}[mode]
+    pad = mode in ("pad", "pad_max")
+    loads0 = oracle.route_by_path(ids, E, caps, pad)[0]
+    mpl = int(loads0.max()) if mode == "pad_max" else 0
+    P = E * mpl if mpl else int(loads0.sum()) + 5
+    if mode == "short":
+        P = max(1, P // 2)                                    # rows beyond P are dropped
+    want = oracle.route_by_path(ids, E, caps, pad, False, mpl, P)
+    got = hip.route_by_path(ids, E, caps, pad, False, mpl, P)
+    for g, w, name in zip(got, want, ("loads", "counts", "seat_rows", "row_entries")):
+        assert np.array_equal(g, w), name
+
+
+def test_route_by_path_path_wise_padding_and_bad_arguments(hip):
+    ids = _compact_route(500, 8, 2, seed=1)
+    ids[ids == 3] = -1                                        # nobody takes path 3
+    caps = [100, 200, 300, 400, 150, 250, 350, 450]
+    want = oracle.route_by_path(ids, 8, caps, True, True, 0, 2300)
+    got = hip.route_by_path(ids, 8, caps, True, True, 0, 2300)
+    assert want[0][3] == 400 and want[1][3] == 0              # an empty path still gets its capacity
+    for g, w in zip(got, want):
+        assert np.array_equal(g, w)
+    with pytest.raises(RuntimeError):
+        hip.route_by_path(ids, 513)
+    with pytest.raises(RuntimeError):
+        hip.route_by_path(ids, 8, None, True)
+
+
+@pytest.mark.parametrize("T,E,k,cell,dtype", [
+    (8192, 64, 1, 768, "bf16"),        # the Switch layer shape
+    (16384, 32, 2, 1024, "bf16"),
+    (3000, 8, 1, 96, "f16"),
+    (1024, 16, 2, 512, "f32"),
+    (777, 5, 3, 8, "f16"),             # one 16-byte unit per row
+    (513, 64, 4, 1100, "f32"),         # rows wider than one pass of a wavefront
+    (300, 6, 2, 20, "f32"),            # 80-byte rows
+])
+@pytest.mark.parametrize("weighted", [False, True])
+def test_rows_ops_bit_exact_and_equal_to_the_dense_ops(hip, T, E, k, cell, dtype, weighted):
+    rng = np.random.default_rng(T + cell)
+    ids = _compact_route(T, E, k, seed=cell, hole=0.03)
+    cap = max(1, int(0.9 * T * k / E))
+    loads, _, seat_rows, row_entries = oracle.route_by_path(ids, E, [cap])
+    P = int(loads.sum())
+    row_entries = row_entries[:P]
+    w = rng.random((T, k)).astype(np.float32)
+    if dtype != "f32":
+        w = bits_to_f32(as_dtype_bits(w, dtype), dtype)       # representable as dense gates too
+    x = as_dtype_bits(rng.standard_normal((T, cell)).astype(np.float32), dtype)
+    got = hip.dispatch_by_rows(x, row_entries, k, w if weighted else None, dtype)
+    assert np.array_equal(got, oracle.dispatch_by_rows(x, row_entries, k, w if weighted else None, dtype))
+    # the dense ops on the same route
+    mask = np.zeros((T, E), dtype=np.int32)
+    gates = np.zeros((T, E), dtype=np.float32)
+    t, j = np.nonzero(ids >= 0)
+    mask[t, ids[t, j]] = 1
+    gates[t, ids[t, j]] = w[t, j]
+    seats, loads_d = oracle.generate_indices_and_loads(mask, [cap])
+    assert np.array_equal(loads_d, loads)
+    g_bits = as_dtype_bits(gates, dtype) if weighted else None
+    dense, _ = hip.dispatch(x, seats, loads, gates_bits=g_bits, dtype=dtype)
+    assert np.array_equal(got, dense)
+
+    y = as_dtype_bits(rng.standard_normal((P, cell)).astype(np.float32), dtype)
+    res = as_dtype_bits(rng.standard_normal((T, cell)).astype(np.float32), dtype)
+    for out_bits in (None, res):
+        for out_dtype in ((dtype, "f32") if dtype != "f32" and out_bits is None else (dtype,)):
+            got = hip.combine_by_rows(y, ids, seat_rows, w if weighted else None, out_bits, dtype, out_dtype)
+            want = oracle.combine_by_rows(y, ids, seat_rows, w if weighted else None, out_bits, dtype, out_dtype)
+            assert np.array_equal(got, want)
+            dense = hip.combine(y, seats, loads, gates_bits=g_bits, residual_bits=out_bits, in_dtype=dtype,
+                                out_dtype=out_dtype)
+            assert np.array_equal(got, dense)
+
+
+def test_combine_by_rows_order_and_bad_rows(hip):
+    y = np.zeros((3, 4), dtype=np.float32)
+    y[:, 0] = [1e8, 1.0, -1e8]
+    rows = np.array([[1, 2, 3], [0, 9, -4]], dtype=np.int32)   # second cell: no valid row
+    for ids, first in (([0, 1, 2], 0.0), ([0, 2, 1], 1.0), ([5, 9, 7], 1.0)):
+        path_ids = np.array([ids, ids], dtype=np.int32)
+        got = hip.combine_by_rows(y, path_ids, rows)
+        assert got[0, 0] == first and np.array_equal(got, oracle.combine_by_rows(y, path_ids, rows))
+        assert not got[1].any()
+    # a cell that names one path twice: the second entry is left out, as in the oracle
+    twice = np.array([[4, 4, 6], [1, 2, 3]], dtype=np.int32)
+    assert np.array_equal(hip.combine_by_rows(y, twice, rows), oracle.combine_by_rows(y, twice, rows))
+    entries = np.array([0, 7, -3, 2], dtype=np.int32)          # 7 and -3 name no entry of 3 x 1
+    x = np.arange(12, dtype=np.float32).reshape(3, 4)
+    got = hip.dispatch_by_rows(x, entries, 1)
+    assert np.array_equal(got, oracle.dispatch_by_rows(x, entries, 1))
+    assert np.array_equal(got[3], x[1]) and not got[:3].any()

@@ -526,3 +526,121 @@ def test_combine_by_index_against_float64_accumulation(dtype, tol):
     np.add.at(want, index, bits_to_f32(bits, dtype).astype(np.float64))
     got = bits_to_f32(oracle.combine_by_index(bits, index, n_out, dtype), dtype)
     assert np.abs(got - want).max() <= tol * max(1.0, np.abs(want).max())
+
+
+# ------------------------------------------------------------- compact route format
+def _compact_route(T, E, k, seed, hole=0.0):
+    """k distinct random paths per cell; a fraction `hole` of the entries is no route (-1)."""
+    rng = np.random.default_rng(seed)
+    ids = np.argsort(rng.random((T, E)), axis=1)[:, :k].astype(np.int32)
+    if hole:
+        ids[rng.random((T, k)) < hole] = -1
+    return ids
+
+
+def _dense_of(ids, E, weights=None):
+    """The dense mask (and gate matrix) of a compact route, by numpy fancy indexing."""
+    T, k = ids.shape
+    mask = np.zeros((T, E), dtype=np.int32)
+    gates = np.zeros((T, E), dtype=np.float32)
+    t, j = np.nonzero((ids >= 0) & (ids < E))
+    mask[t, ids[t, j]] = 1
+    if weights is not None:
+        gates[t, ids[t, j]] = weights[t, j]
+    return mask, gates
+
+
+@pytest.mark.parametrize("T,E,k", [(64, 4, 1), (200, 16, 2), (50, 64, 4), (33, 100, 7), (5, 3, 3)])
+def test_gate_topk_matches_torch_topk_and_softmax(T, E, k):
+    import torch
+
+    rng = np.random.default_rng(T + E + k)
+    score = (3 * rng.standard_normal((T, E))).astype(np.float32)
+    want = torch.topk(torch.from_numpy(score), k, dim=1)            # topk.py:26
+    ids, w = oracle.gate_topk(score, k)
+    assert np.array_equal(ids, want.indices.numpy().astype(np.int32))
+    assert np.array_equal(w, want.values.numpy())
+    ids2, p = oracle.gate_topk(score, k, softmax=True)
+    assert np.array_equal(ids2, ids)
+    probs = torch.softmax(torch.from_numpy(score).double(), dim=1)  # switch_transformer.py:243
+    assert np.allclose(p, probs.gather(1, want.indices).numpy(), rtol=1e-6, atol=0)
+    mask, _ = _dense_of(ids, E)
+    assert np.array_equal(mask, oracle.topk_hot_mask(score, k))
+
+
+def test_gate_topk_top1_is_the_switch_router():
+    # switch_transformer.py:240-253: probs = softmax(logits.float()); index = argmax; weight = max
+    import torch
+
+    rng = np.random.default_rng(5)
+    logits = rng.standard_normal((300, 64)).astype(np.float32)
+    ids, w = oracle.gate_topk(logits, 1, softmax=True)
+    probs = torch.softmax(torch.from_numpy(logits), dim=-1)
+    assert np.array_equal(ids[:, 0], torch.argmax(probs, dim=-1).numpy())
+    assert np.allclose(w[:, 0], probs.max(dim=-1).values.numpy(), rtol=2e-6, atol=0)
+
+
+@pytest.mark.parametrize("T,E,k,hole", [(512, 8, 1, 0.0), (1000, 16, 2, 0.1), (77, 64, 4, 0.0), (1, 5, 2, 0.0)])
+@pytest.mark.parametrize("mode", ["plain", "clip", "pad", "pad_max"])
+def test_route_by_path_matches_the_dense_closed_form(T, E, k, hole, mode):
+    ids = _compact_route(T, E, k, seed=T + k, hole=hole)
+    mask, _ = _dense_of(ids, E)
+    cap = max(1, (T * k) // (2 * E))
+    caps = {"plain": None, "clip": [cap], "pad": [cap, 4 * cap, T], "pad_max": [cap, 4 * cap, T]}[mode]
+    pad = mode in ("pad", "pad_max")
+    seats, loads_want = fabric_test_closed_form(mask, caps, capacity_padding=pad)
+    mpl = int(loads_want.max()) if mode == "pad_max" else 0
+    P = E * mpl if mpl else int(loads_want.sum()) + 3  # three rows behind the last path: padding
+    loads, counts, seat_rows, row_entries = oracle.route_by_path(ids, E, caps, pad, False, mpl, P)
+    assert np.array_equal(loads, loads_want)
+    assert np.array_equal(counts, mask.sum(0))
+    start = np.arange(E) * mpl if mpl else np.cumsum(loads_want) - loads_want
+    want_rows = np.zeros((T, k), dtype=np.int32)
+    for t in range(T):
+        for j in range(k):
+            e = ids[t, j]
+            if 0 <= e < E and seats[t, e] <= loads_want[e]:
+                want_rows[t, j] = start[e] + seats[t, e]
+    assert np.array_equal(seat_rows, want_rows)
+    # row_entries is the inverse of seat_rows, zero elsewhere
+    want_entries = np.zeros_like(row_entries)
+    t, j = np.nonzero(want_rows)
+    want_entries[want_rows[t, j] - 1] = t * k + j + 1
+    assert np.array_equal(row_entries, want_entries)
+    assert np.count_nonzero(row_entries) == np.count_nonzero(want_rows)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16", "f16"])
+@pytest.mark.parametrize("weighted", [False, True])
+def test_rows_ops_equal_the_dense_ops_on_the_same_route(dtype, weighted):
+    T, E, k, d = 300, 16, 2, 24
+    rng = np.random.default_rng(11)
+    ids = _compact_route(T, E, k, seed=3, hole=0.05)
+    w = rng.random((T, k)).astype(np.float32)
+    if dtype != "f32":  # gates travel in the data type in the dense ops: use representable ones
+        w = bits_to_f32(as_dtype_bits(w, dtype), dtype)
+    mask, gates = _dense_of(ids, E, w)
+    caps = [30]
+    seats, loads = oracle.generate_indices_and_loads(mask, caps)
+    loads_c, _, seat_rows, row_entries = oracle.route_by_path(ids, E, caps, P=int(loads.sum()))
+    assert np.array_equal(loads_c, loads)
+    x = as_dtype_bits(rng.standard_normal((T, d)).astype(np.float32), dtype)
+    g_bits = as_dtype_bits(gates, dtype) if weighted else None
+    want, _ = oracle.dispatch(x, seats, loads, gates=g_bits, dtype=dtype)
+    got = oracle.dispatch_by_rows(x, row_entries, k, w if weighted else None, dtype)
+    assert np.array_equal(got, want)
+    y = as_dtype_bits(rng.standard_normal((int(loads.sum()), d)).astype(np.float32), dtype)
+    res = as_dtype_bits(rng.standard_normal((T, d)).astype(np.float32), dtype)
+    for out_data in (None, res):
+        want = oracle.combine(y, seats, loads, gates=g_bits, out_data=out_data, in_dtype=dtype)
+        got = oracle.combine_by_rows(y, ids, seat_rows, w if weighted else None, out_data, dtype)
+        assert np.array_equal(got, want)
+
+
+def test_combine_by_rows_adds_in_ascending_path_order():
+    # three rows for one cell: (1e8 + 1) - 1e8 is 0 in fp32, 1e8 - 1e8 + 1 is 1
+    y = np.array([[1e8], [1.0], [-1e8]], dtype=np.float32)
+    rows = np.array([[1, 2, 3]], dtype=np.int32)
+    assert oracle.combine_by_rows(y, np.array([[0, 1, 2]], dtype=np.int32), rows)[0, 0] == 0.0
+    assert oracle.combine_by_rows(y, np.array([[0, 2, 1]], dtype=np.int32), rows)[0, 0] == 1.0
+    assert oracle.combine_by_rows(y, np.array([[5, 9, 7]], dtype=np.int32), rows)[0, 0] == 1.0
