@@ -301,6 +301,78 @@ def main():
     if not torch.equal(gate_mask, mask):
         sys.exit("bench.py: the gate kernel does not reproduce the argmax mask")
 
+    # the same route in the compact format (k path ids per cell instead of the [T,E] mask):
+    # fused softmax + top-1 gate, route from the ids, dispatch by row entries, the same FFN, combine
+    # by the row entries (for one path per cell they are the row tags); reported beside the dense
+    # path and checked against it bit for bit, not part of `value`
+    logits_d = logits.to(dev)
+    c_ids = torch.empty(T, 1, dtype=torch.int32, device=dev)
+    c_w = torch.empty(T, 1, dtype=torch.float32, device=dev)
+    c_loads_counts = torch.empty(2, E, dtype=torch.int32, device=dev)
+    c_seat_rows = torch.empty(T, 1, dtype=torch.int32, device=dev)
+    c_entries = torch.empty(P, dtype=torch.int32, device=dev)
+    c_y = torch.empty(P, D, dtype=torch.bfloat16, device=dev)
+    c_h = torch.empty(P, DFF, dtype=torch.bfloat16, device=dev)
+    c_y2 = torch.empty(P, D, dtype=torch.bfloat16, device=dev)
+    c_out = x.clone()
+    c_out_gather = x.clone()
+    c_ws = torch.empty(max(4, L.brt_hip_route_by_path_workspace_bytes(T, 1, E)), dtype=torch.uint8, device=dev)
+
+    def k_gate_compact():
+        _lib.check(L.brt_hip_gate_topk(logits_d.data_ptr(), T, E, 1, _lib.F32, 1, c_ids.data_ptr(),
+                                       c_w.data_ptr(), None, sptr()))
+
+    def k_gate_switch_torch():  # switch_transformer.py:240-253
+        p = torch.softmax(logits_d, dim=-1)
+        torch.nn.functional.one_hot(torch.argmax(p, dim=-1), num_classes=E)
+        torch.max(p, dim=-1)
+
+    def k_route_compact():
+        _lib.check(L.brt_hip_route_by_path(
+            c_ids.data_ptr(), T, 1, E, caps.data_ptr(), 1, 0, 0, 0, c_loads_counts[0].data_ptr(),
+            c_loads_counts[1].data_ptr(), c_seat_rows.data_ptr(), c_entries.data_ptr(), P,
+            c_ws.data_ptr(), c_ws.numel(), sptr()))
+
+    def k_dispatch_rows():
+        _lib.check(L.brt_hip_dispatch_by_rows(x.data_ptr(), c_y.data_ptr(), None, c_entries.data_ptr(),
+                                              P, T, 1, D, _lib.BF16, sptr()))
+
+    def k_combine_rows():
+        _lib.check(L.brt_hip_combine_by_rows(
+            (c_y2 if have_ffn else c_y).data_ptr(), c_out_gather.data_ptr(), None, c_ids.data_ptr(),
+            c_seat_rows.data_ptr(), T, 1, D, P, 1, _lib.BF16, _lib.BF16, sptr()))
+
+    def step_compact():
+        k_route_compact()
+        k_dispatch_rows()
+        if have_ffn:
+            _lib.check(L.brt_hip_grouped_gemm(
+                c_y.data_ptr(), wi_tab.data_ptr(), None, c_h.data_ptr(), c_loads_counts[0].data_ptr(),
+                E, P, D, DFF, _lib.ACT_GELU, sptr()))
+            _lib.check(L.brt_hip_grouped_gemm(
+                c_h.data_ptr(), wo_tab.data_ptr(), None, c_y2.data_ptr(), c_loads_counts[0].data_ptr(),
+                E, P, DFF, D, _lib.ACT_NONE, sptr()))
+        _lib.check(L.brt_hip_combine_by_tags(
+            (c_y2 if have_ffn else c_y).data_ptr(), c_out.data_ptr(), c_entries.data_ptr(), P, D, T,
+            _lib.BF16, _lib.BF16, sptr()))
+
+    with torch.cuda.stream(stream):
+        k_gate_compact()
+        step_compact()
+        k_combine_rows()
+    stream.synchronize()
+    if not torch.equal(c_ids.view(-1).long(), expert.to(dev)):
+        sys.exit("bench.py: the compact gate does not reproduce the argmax")
+    if not torch.allclose(c_w.view(-1).cpu(), probs.max(dim=1).values, rtol=2e-6, atol=0):
+        sys.exit("bench.py: the compact gate's softmax weight is off")
+    if not (torch.equal(c_out.view(torch.int16), out.view(torch.int16))
+            and torch.equal(c_out_gather.view(torch.int16), out.view(torch.int16))
+            and torch.equal(c_loads_counts, loads_counts)):
+        sys.exit("bench.py: the layer on the compact route disagrees with the dense one")
+    g_compact = capture(step_compact, args.steps)
+    timed(g_compact, 1)
+    compact_layer_us = timed(g_compact, 1) / args.steps * 1e3
+
     # the library's batched GEMM on the same FFN, every expert padded to the full capacity (the
     # only shape a batched routine takes), GELU as its own elementwise launch: reported beside
     # the grouped kernel, not part of the step
@@ -374,7 +446,11 @@ def main():
                "combine_gather": k_combine_gather, "gate_topk_mask": k_gate,
                "gate_topk_mask_torch_ops": k_gate_torch,
                "tag_gather_unique": k_tag_unique, "tag_gather_sum": k_tag_sum,
-               "tag_gather_sum_torch_ops": k_tag_sum_torch, "plain_copy_of_the_rows": k_copy_rows}
+               "tag_gather_sum_torch_ops": k_tag_sum_torch, "plain_copy_of_the_rows": k_copy_rows,
+               "compact_gate_softmax_top1": k_gate_compact,
+               "compact_gate_switch_torch_ops": k_gate_switch_torch,
+               "compact_route_by_path": k_route_compact, "compact_dispatch_by_rows": k_dispatch_rows,
+               "compact_combine_by_rows": k_combine_rows}
     if have_ffn:
         kernels.update({"ffn_gemm1_gelu": k_gemm1, "ffn_gemm2": k_gemm2,
                         "indexgen_tags": k_indexgen_tags, "ffn_gemm1_gelu_gather": k_gemm1_gather,
@@ -410,6 +486,10 @@ def main():
     bytes_["indexgen_tags"] = bytes_["indexgen"]
     bytes_["gate_topk_mask"] = 2 * idx_bytes  # fp32 scores in, int32 mask out
     bytes_["plain_copy_of_the_rows"] = 2 * min(P, T) * D * es
+    bytes_["compact_gate_softmax_top1"] = idx_bytes + 8 * T          # fp32 scores in, id + weight out
+    bytes_["compact_route_by_path"] = 2 * 4 * T + 4 * T + 4 * P + 8 * E  # ids twice, seat rows, entries
+    bytes_["compact_dispatch_by_rows"] = R * D * es + P * D * es + 4 * P
+    bytes_["compact_combine_by_rows"] = R * D * es + T * D * es + 8 * T
     bytes_["tag_gather_sum"] = 2 * P * D * es + 8 * P + 4 * (2 * P)  # rows in/out, index, lists
     dc_bytes = bytes_["dispatch"] + bytes_["combine"]
     dc_us = us["dispatch"] + us["combine"]
@@ -507,6 +587,8 @@ def main():
         },
         "layer_us": round(ms_per_step * 1e3, 2),
         "layer_us_one_graph_launch_per_step": round(per_graph_launch_us, 2),
+        "layer_compact_us": round(compact_layer_us, 2),
+        "layer_compact_step": "route from path ids+dispatch by rows+ffn+combine by row tags; K steps in one HIP graph",
         "layer_fused_us": None if fused_layer_us is None else round(fused_layer_us, 2),
         "layer_fused_step": "indexgen(tag indices)+GEMM1 gathering cells+GEMM2 scattering to cells; K steps in one HIP graph",
         "wall_ms_timed_region": round(wall_ms, 3),

@@ -83,10 +83,11 @@ SIGNATURES = {
         _c_int,
         [_c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
     ),
+    "brt_hip_route_by_path_workspace_bytes": (_c_size, [_c_int, _c_int, _c_int]),
     "brt_hip_route_by_path": (
         _c_int,
         [_c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr,
-         _c_ptr, _c_int, _c_ptr],
+         _c_ptr, _c_int, _c_ptr, _c_size, _c_ptr],
     ),
     "brt_hip_dispatch_by_rows": (
         _c_int,

@@ -33,6 +33,28 @@ __device__ __forceinline__ int wave_inclusive_scan(int v) {
   return v;
 }
 
+// All-reduce of a commutative `op` over aligned segments of `width` lanes (a power of two; the
+// same for the whole wavefront): the xor butterfly, with its first four steps on the DPP network
+// instead of the LDS crossbar.  Step d pairs lane i with lane i ^ d; quad_perm does that for
+// d = 1, 2, and because the values are uniform over aligned groups of d lanes once step d is
+// reached, row_half_mirror (i -> 7 - i) and row_mirror (i -> 15 - i) do it for d = 4, 8.
+template <typename Op>
+__device__ __forceinline__ int segment_all_reduce(int v, int width, Op op) {
+  if (width > 1) v = op(v, __builtin_amdgcn_mov_dpp(v, 0xB1, 0xf, 0xf, true));   // quad_perm:[1,0,3,2]
+  if (width > 2) v = op(v, __builtin_amdgcn_mov_dpp(v, 0x4E, 0xf, 0xf, true));   // quad_perm:[2,3,0,1]
+  if (width > 4) v = op(v, __builtin_amdgcn_mov_dpp(v, 0x141, 0xf, 0xf, true));  // row_half_mirror
+  if (width > 8) v = op(v, __builtin_amdgcn_mov_dpp(v, 0x140, 0xf, 0xf, true));  // row_mirror
+  if (width > 16) v = op(v, __shfl_xor(v, 16, kWave));
+  if (width > 32) v = op(v, __shfl_xor(v, 32, kWave));
+  return v;
+}
+template <typename Op>
+__device__ __forceinline__ float segment_all_reduce(float v, int width, Op op) {
+  return __int_as_float(segment_all_reduce(__float_as_int(v), width, [&](int x, int y) {
+    return __float_as_int(op(__int_as_float(x), __int_as_float(y)));
+  }));
+}
+
 // Value of `v` held by lane `src_lane`; src_lane must be wave-uniform.
 __device__ __forceinline__ int read_lane(int v, int src_lane) {
   return __builtin_amdgcn_readlane(v, src_lane);

@@ -25,11 +25,15 @@ namespace brt {
 namespace {
 
 constexpr int kBlock = 256;
-constexpr int kRouteWaves = 16;  // one workgroup of 16 wavefronts computes a whole route
-constexpr int kRouteBlock = kRouteWaves * kWave;
-constexpr int kBatch = 8;        // chunks of 64 entries a wavefront keeps in flight
+constexpr int kWholeWaves = 8;    // a small route: one workgroup of 8 wavefronts, one launch
+constexpr int kWholeChunks = 32;  // ... up to this many chunks of 64 entries
+constexpr int kSplitWaves = 4;    // larger routes: workgroups of 4 wavefronts, two launches
+constexpr int kSplitGroups = 32;  // ... in at most this many workgroups
+constexpr int kSplitUnits = kSplitGroups * kSplitWaves;
+constexpr int kBatch = 4;        // chunks of 64 entries a wavefront keeps in flight
 constexpr int kMaxK = 8;         // paths per cell in combine_by_rows
-constexpr int kMaxRoutePaths = 512;  // (kRouteWaves + 3) * E words of LDS
+constexpr int kMaxRoutePaths = 512;  // (2 * kWholeWaves + 3) * E words of LDS
+constexpr int kMaxCapsInLds = 1024;
 
 struct RouteArgs {
   const int* ids;
@@ -38,7 +42,10 @@ struct RouteArgs {
   int* counts;
   int* seat_rows;
   int* row_entries;
+  int* ws;  // [groups][E] + [units][E] counters of the two-launch form
+  int units;
   int n, E, C, P, bits, per_wave;
+  int caps_in_lds;  // number of capacities staged in LDS (all of them, or 0)
   int capacity_padding, path_wise_padding, max_path_load;
 };
 
@@ -55,109 +62,204 @@ __device__ __forceinline__ unsigned long long same_path_lanes(int e, bool valid,
 
 __device__ __forceinline__ unsigned long long lanes_below(int lane) { return (1ull << lane) - 1ull; }
 
-// One workgroup.  Wavefront w owns the entries [w * per_wave, (w+1) * per_wave), in chunks of 64
-// (one entry per lane).  Pass 1 counts entries per (wavefront, path) in LDS: the lanes of a chunk
-// that hold the same path are found with one ballot per id bit, and the lowest of them adds their
-// number to the wavefront's counter -- no atomics, every counter has one writer.  A column scan
-// over the 16 wavefronts turns the counters into each wavefront's first seat per path and gives
-// the real count of every path, from which the loads and the first row of every path follow.
+// Wavefront (unit) u owns the entries [u * per_wave, (u+1) * per_wave), in chunks of 64
+// (one entry per lane), kBatch chunks in flight.  Pass 1 counts entries per (wavefront, path) in
+// LDS: the lanes of a chunk that hold the same path are found with one ballot per id bit, and the
+// lowest of them adds their number to the wavefront's counter -- no atomics, every counter has
+// one writer.  Then every wavefront sums the counters of the units before it (its first
+// seat per path) while the first wavefront turns the column totals into loads and first rows.
 // Pass 2 walks the entries again: seat = wavefront's running count + rank among the lanes of the
-// chunk with the same path.
-__global__ __launch_bounds__(kRouteBlock) void route_by_path_kernel(RouteArgs a) {
+// chunk with the same path.  The first batch of ids stays in registers between the passes; the
+// capacities are staged in LDS at the start, off the critical path.  The kernels are kept small
+// (loops over batches and path columns are not unrolled): at a few microseconds per launch,
+// fetching the code is part of the run time.
+struct Batch {
+  int id[kBatch];
+};
+
+__device__ __forceinline__ Batch load_batch(const int* __restrict__ ids, int c0, int hi, int lane) {
+  Batch b;
+#pragma unroll
+  for (int q = 0; q < kBatch; ++q) {
+    const int i = c0 + q * kWave + lane;
+    b.id[q] = i < hi ? ids[i] : -1;
+  }
+  return b;
+}
+
+__device__ __forceinline__ void count_batch(const Batch& b, int c0, int hi, int lane, int E, int bits,
+                                            int* mine) {
+#pragma unroll
+  for (int q = 0; q < kBatch; ++q) {
+    if (c0 + q * kWave < hi) {  // same for the whole wavefront
+      const int e = b.id[q];
+      const bool valid = e >= 0 && e < E;
+      const unsigned long long same = same_path_lanes(e, valid, bits);
+      if (valid && (same & lanes_below(lane)) == 0) mine[e] += __popcll(same);
+    }
+  }
+}
+
+__device__ __forceinline__ void emit_batch(const Batch& b, int c0, int hi, int lane, const RouteArgs& a,
+                                           int* mine, const int* s_kept, const int* s_start) {
+#pragma unroll
+  for (int q = 0; q < kBatch; ++q) {
+    if (c0 + q * kWave < hi) {
+      const int i = c0 + q * kWave + lane;
+      const int e = b.id[q];
+      const bool valid = e >= 0 && e < a.E;
+      const unsigned long long same = same_path_lanes(e, valid, a.bits);
+      const int rank = __popcll(same & lanes_below(lane));
+      const int before = valid ? mine[e] : 0;  // read by every lane before the first of them updates it
+      if (valid && rank == 0) mine[e] = before + __popcll(same);
+      const int seat = before + rank + 1;
+      int row = 0;
+      if (valid && seat <= s_kept[e]) row = s_start[e] + seat;
+      if (row > a.P) row = 0;
+      if (i < hi) a.seat_rows[i] = row;
+      if (row != 0) a.row_entries[row - 1] = i + 1;
+    }
+  }
+}
+
+// Sums, for the paths e = c * 64 + lane, `rows` rows of counters ([rows][E], in LDS or in
+// global memory): all of them into total, those before row `mine` into before.  At most MAX rows,
+// all loaded before the first is used: one memory round trip.
+template <int MAX, typename Ptr>
+__device__ __forceinline__ void sum_rows(Ptr cnt, int rows, int mine, int E, int e, int* before,
+                                         int* total) {
+  // every load is unconditional (row and path clamped into the table, the value dropped
+  // afterwards): a load under a condition of its own becomes a branch, and the loads of
+  // consecutive branches wait for each other
+  const int col = min(e, E - 1);
+  int n[MAX];
+#pragma unroll
+  for (int v = 0; v < MAX; ++v) n[v] = cnt[min(v, rows - 1) * E + col];
+#pragma unroll
+  for (int v = 0; v < MAX; ++v) {
+    const int add = (v < rows && e < E) ? n[v] : 0;
+    *before += v < mine ? add : 0;
+    *total += add;
+  }
+}
+
+// kWhole: one workgroup computes the route (small routes: one launch).  kCount + kEmit: the
+// same work spread over up to kSplitGroups workgroups in two launches; a unit is a wavefront and
+// its contiguous range of entries.  The counters travel through `ws`: [groups][E] sums per
+// workgroup, then [units][E] per unit, so that a unit finds its first seats with one round of
+// loads: the sums of the workgroups before its own plus the units before it in its own.
+enum RouteMode { kWhole = 0, kCount = 1, kEmit = 2 };
+
+template <int MODE, int WAVES>
+__global__ __launch_bounds__(WAVES * kWave) void route_kernel(RouteArgs a) {
   extern __shared__ int lds[];
   const int E = a.E;
-  int* s_base = lds;                     // [kRouteWaves][E]
-  int* s_load = lds + kRouteWaves * E;   // [E]
-  int* s_start = s_load + E;             // [E]
-  int* s_kept = s_start + E;             // [E] rows a path really fills
+  int* s_cnt = lds;                                         // [WAVES][E] counters
+  int* s_seat = MODE == kWhole ? lds + WAVES * E : lds;     // [WAVES][E] running seats of pass 2
+  int* s_load = s_seat + WAVES * E;                         // [E]
+  int* s_start = s_load + E;                                // [E]
+  int* s_kept = s_start + E;                                // [E] rows a path really fills
+  int* s_caps = s_kept + E;                                 // [caps_in_lds]
   const int lane = threadIdx.x & (kWave - 1), w = threadIdx.x >> 6;
-  for (int i = threadIdx.x; i < kRouteWaves * E; i += kRouteBlock) s_base[i] = 0;
+  const int unit = blockIdx.x * WAVES + w;
+  constexpr int kStep = kWave * kBatch;
+
+  const int lo = static_cast<int>(min(static_cast<long>(a.n), static_cast<long>(unit) * a.per_wave));
+  const int hi = min(a.n, lo + a.per_wave);
+  // the first batch of ids is fetched once, ahead of everything else, and serves both passes
+  const Batch first = load_batch(a.ids, lo, hi, lane);
+  int* unit_rows = a.ws + static_cast<size_t>(gridDim.x) * E;  // behind the workgroup sums
+  // kEmit: the counters of the first 64 paths are fetched in the same round trip as the ids and
+  // the capacities
+  int before0 = 0, total0 = 0;
+  if constexpr (MODE == kEmit) {
+    int own = 0;  // this workgroup's total is part of the workgroup sums already
+    sum_rows<kSplitGroups>(a.ws, static_cast<int>(gridDim.x), static_cast<int>(blockIdx.x), E, lane, &before0, &total0);
+    sum_rows<WAVES>(unit_rows + static_cast<size_t>(blockIdx.x) * WAVES * E, WAVES, w, E, lane, &before0, &own);
+  }
+  if (MODE != kCount)
+    for (int i = threadIdx.x; i < a.caps_in_lds; i += WAVES * kWave) s_caps[i] = a.caps[i];
+  if (MODE != kEmit)
+    for (int i = threadIdx.x; i < WAVES * E; i += WAVES * kWave) s_cnt[i] = 0;
   __syncthreads();
+  const int* caps = a.caps_in_lds != 0 ? s_caps : a.caps;
 
-  const int lo = min(a.n, w * a.per_wave), hi = min(a.n, lo + a.per_wave);
-  int* mine = s_base + w * E;
-
-  for (int c0 = lo; c0 < hi; c0 += kWave * kBatch) {
-    int id[kBatch];
-#pragma unroll
-    for (int b = 0; b < kBatch; ++b) {
-      const int i = c0 + b * kWave + lane;
-      id[b] = i < hi ? a.ids[i] : -1;
+  if (MODE != kEmit) {
+    int* mine = s_cnt + w * E;
+#pragma unroll 1
+    for (int c0 = lo; c0 < hi; c0 += kStep) {
+      Batch b = first;
+      if (c0 != lo) b = load_batch(a.ids, c0, hi, lane);
+      count_batch(b, c0, hi, lane, E, a.bits, mine);
     }
+  }
+  if (MODE == kCount) {
+    const int* mine = s_cnt + w * E;
+    for (int e = lane; e < E; e += kWave) unit_rows[static_cast<size_t>(unit) * E + e] = mine[e];
+    __syncthreads();
+    for (int e = threadIdx.x; e < E; e += WAVES * kWave) {
+      int sum = 0;
 #pragma unroll
-    for (int b = 0; b < kBatch; ++b) {
-      if (c0 + b * kWave < hi) {  // same for the whole wavefront
-        const int e = id[b];
-        const bool valid = e >= 0 && e < E;
-        const unsigned long long same = same_path_lanes(e, valid, a.bits);
-        if (valid && (same & lanes_below(lane)) == 0) mine[e] += __popcll(same);
+      for (int v = 0; v < WAVES; ++v) sum += s_cnt[v * E + e];
+      a.ws[static_cast<size_t>(blockIdx.x) * E + e] = sum;
+    }
+    return;
+  }
+  if (MODE == kWhole) __syncthreads();
+
+  // first seat of this unit in every path; the first wavefront also finishes the columns
+  int* mine = s_seat + w * E;
+  int carry = 0;
+#pragma unroll 1
+  for (int e0 = 0; e0 < E; e0 += kWave) {
+    const int e = e0 + lane;
+    int before = 0, total = 0;
+    if constexpr (MODE == kWhole) {
+      sum_rows<WAVES>(s_cnt, WAVES, w, E, e, &before, &total);
+    } else if (e0 == 0) {
+      before = before0;
+      total = total0;
+    } else {
+      int own = 0;
+      sum_rows<kSplitGroups>(a.ws, static_cast<int>(gridDim.x), static_cast<int>(blockIdx.x), E, e, &before, &total);
+      sum_rows<WAVES>(unit_rows + static_cast<size_t>(blockIdx.x) * WAVES * E, WAVES, w, E, e, &before, &own);
+    }
+    if (e < E) mine[e] = before;
+    if (w == 0) {
+      const int load = e < E ? finalize_load(total, caps, a.C, a.capacity_padding, a.path_wise_padding, e) : 0;
+      const int incl = wave_inclusive_scan(load);
+      if (e < E) {
+        s_load[e] = load;
+        s_kept[e] = min(total, a.max_path_load != 0 ? min(load, a.max_path_load) : load);
+        s_start[e] = a.max_path_load != 0 ? e * a.max_path_load : carry + incl - load;
+        if (blockIdx.x == 0) {
+          a.loads[e] = load;
+          if (a.counts) a.counts[e] = total;
+        }
       }
-    }
-  }
-  __syncthreads();
-
-  for (int e = threadIdx.x; e < E; e += kRouteBlock) {
-    int run = 0;
-    for (int v = 0; v < kRouteWaves; ++v) {
-      const int c = s_base[v * E + e];
-      s_base[v * E + e] = run;
-      run += c;
-    }
-    const int load = finalize_load(run, a.caps, a.C, a.capacity_padding, a.path_wise_padding, e);
-    s_load[e] = load;
-    s_kept[e] = min(run, a.max_path_load != 0 ? min(load, a.max_path_load) : load);
-    a.loads[e] = load;
-    if (a.counts) a.counts[e] = run;
-  }
-  __syncthreads();
-  if (w == 0) {  // first row of every path
-    int carry = 0;
-    for (int e0 = 0; e0 < E; e0 += kWave) {
-      const int e = e0 + lane;
-      const int v = e < E ? s_load[e] : 0;
-      const int incl = wave_inclusive_scan(v);
-      if (e < E) s_start[e] = a.max_path_load != 0 ? e * a.max_path_load : carry + incl - v;
       carry += __shfl(incl, kWave - 1, kWave);
     }
   }
-  __syncthreads();
+  __syncthreads();  // loads and first rows are in place
 
-  for (int c0 = lo; c0 < hi; c0 += kWave * kBatch) {
-    int id[kBatch];
-#pragma unroll
-    for (int b = 0; b < kBatch; ++b) {
-      const int i = c0 + b * kWave + lane;
-      id[b] = i < hi ? a.ids[i] : -1;
-    }
-#pragma unroll
-    for (int b = 0; b < kBatch; ++b) {
-      if (c0 + b * kWave < hi) {
-        const int i = c0 + b * kWave + lane;
-        const int e = id[b];
-        const bool valid = e >= 0 && e < E;
-        const unsigned long long same = same_path_lanes(e, valid, a.bits);
-        const int rank = __popcll(same & lanes_below(lane));
-        const int before = valid ? mine[e] : 0;  // read by every lane before the first of them updates it
-        if (valid && rank == 0) mine[e] = before + __popcll(same);
-        const int seat = before + rank + 1;
-        int row = 0;
-        if (valid && seat <= s_kept[e]) row = s_start[e] + seat;
-        if (row > a.P) row = 0;
-        if (i < hi) a.seat_rows[i] = row;
-        if (row != 0) a.row_entries[row - 1] = i + 1;
-      }
-    }
+#pragma unroll 1
+  for (int c0 = lo; c0 < hi; c0 += kStep) {
+    Batch b = first;
+    if (c0 != lo) b = load_batch(a.ids, c0, hi, lane);
+    emit_batch(b, c0, hi, lane, a, mine, s_kept, s_start);
   }
 
   // padding rows: between the rows a path filled and the first row of the next path, and
   // behind the last path
-  for (int e = w; e < E; e += kRouteWaves) {
-    const int first = s_start[e] + s_kept[e];
+  const int all_units = gridDim.x * WAVES;
+  for (int e = unit; e < E; e += all_units) {
+    const int from = s_start[e] + s_kept[e];
     const int end = min(a.P, a.max_path_load != 0 ? s_start[e] + a.max_path_load : s_start[e] + s_load[e]);
-    for (int r = first + lane; r < end; r += kWave) a.row_entries[r] = 0;
+    for (int r = from + lane; r < end; r += kWave) a.row_entries[r] = 0;
   }
-  const int total = a.max_path_load != 0 ? E * a.max_path_load : s_start[E - 1] + s_load[E - 1];
-  for (int r = total + threadIdx.x; r < a.P; r += kRouteBlock) a.row_entries[r] = 0;
+  const int rows = a.max_path_load != 0 ? E * a.max_path_load : s_start[E - 1] + s_load[E - 1];
+  for (long r = static_cast<long>(rows) + unit * kWave + lane; r < a.P; r += static_cast<long>(all_units) * kWave)
+    a.row_entries[r] = 0;
 }
 
 // ---------------------------------------------------------------- rows by entry
@@ -246,17 +348,31 @@ __global__ __launch_bounds__(kBlock) void combine_by_rows_kernel(RowsArgs a) {
   for (int tb = 0; tb < nt; tb += GROUPS) {
     const int i = tb + gidx;
     const bool live = i < nt;
-    const size_t slot0 = static_cast<size_t>(t0 + i) * k;
+    // Entries of the cell: three independent sets of loads, one memory round trip before the
+    // rows can be fetched.  Every load is unconditional (cell and entry clamped into the tables,
+    // the value dropped afterwards): loads under conditions of their own become branches that
+    // wait for each other.
+    const size_t slot0 = static_cast<size_t>(min(t0 + i, static_cast<long>(a.T) - 1)) * k;
     int id[kMaxK], row[kMaxK];
     float g[kMaxK];
+#pragma unroll
+    for (int j = 0; j < kMaxK; ++j) {
+      const int jj = min(j, k - 1);
+      row[j] = a.seat_rows[slot0 + jj];
+      id[j] = a.ids[slot0 + jj];
+    }
+    if (a.weights != nullptr) {
+#pragma unroll
+      for (int j = 0; j < kMaxK; ++j) g[j] = a.weights[slot0 + min(j, k - 1)];
+    } else {
+#pragma unroll
+      for (int j = 0; j < kMaxK; ++j) g[j] = 1.0f;
+    }
     int owned = 0;
 #pragma unroll
     for (int j = 0; j < kMaxK; ++j) {
-      const bool has = live && j < k;
-      row[j] = has ? a.seat_rows[slot0 + j] : 0;
-      if (row[j] < 0 || row[j] > a.P) row[j] = 0;
-      id[j] = row[j] != 0 ? a.ids[slot0 + j] : 0x7fffffff;
-      g[j] = (row[j] != 0 && a.weights) ? a.weights[slot0 + j] : 1.0f;
+      if (!live || j >= k || row[j] < 0 || row[j] > a.P) row[j] = 0;
+      if (row[j] == 0) id[j] = 0x7fffffff;
       owned += row[j] != 0;
     }
     const size_t to = static_cast<size_t>(t0 + i) * cpr;
@@ -319,16 +435,35 @@ int rows_per_wavefront(int cpr, long rows) {
 
 using namespace brt;
 
+namespace {
+
+// Units and entries per unit of the two-launch form.
+void split_geometry(int n, int* units, int* per_wave) {
+  const int chunks = (n + kWave - 1) / kWave;
+  const int chunks_pw = std::max(1, (chunks + kSplitUnits - 1) / kSplitUnits);
+  const int used = (chunks + chunks_pw - 1) / chunks_pw;
+  *units = (used + kSplitWaves - 1) / kSplitWaves * kSplitWaves;
+  *per_wave = chunks_pw * kWave;
+}
+
+}  // namespace
+
+extern "C" size_t brt_hip_route_by_path_workspace_bytes(int T, int k, int E) {
+  if (T <= 0 || k <= 0 || E <= 0 || static_cast<long>(T) * k >= (1l << 31)) return 0;
+  int units, per_wave;
+  split_geometry(T * k, &units, &per_wave);
+  return static_cast<size_t>(units / kSplitWaves + units) * E * sizeof(int);
+}
+
 extern "C" int brt_hip_route_by_path(const int32_t* path_ids, int T, int k, int E, const int32_t* caps,
                                      int C, int capacity_padding, int path_wise_padding,
                                      int max_path_load, int32_t* loads, int32_t* counts,
-                                     int32_t* seat_rows, int32_t* row_entries, int P, void* stream) {
+                                     int32_t* seat_rows, int32_t* row_entries, int P,
+                                     void* workspace, size_t workspace_bytes, void* stream) {
   if (T < 0 || k < 0 || E <= 0 || P < 0 || max_path_load < 0)
     return fail(BRT_E_INVALID, "bad shape T=%d k=%d E=%d P=%d", T, k, E, P);
   if (E > kMaxRoutePaths) return fail(BRT_E_UNSUPPORTED, "more than %d paths", kMaxRoutePaths);
-  if (static_cast<long>(T) * k >= (1l << 24))
-    return fail(BRT_E_UNSUPPORTED, "T*k = %ld: the single-workgroup route is limited to 2^24 entries",
-                static_cast<long>(T) * k);
+  if (static_cast<long>(T) * k >= (1l << 31)) return fail(BRT_E_UNSUPPORTED, "T*k >= 2^31");
   if (caps == nullptr) C = 0;
   if (capacity_padding && C < 1)
     return fail(BRT_E_INVALID, "capacity_padding needs at least one supported capacity");
@@ -347,11 +482,25 @@ extern "C" int brt_hip_route_by_path(const int32_t* path_ids, int T, int k, int 
   a.capacity_padding = capacity_padding; a.path_wise_padding = path_wise_padding;
   a.max_path_load = max_path_load;
   while ((1 << a.bits) < E) ++a.bits;
+  a.caps_in_lds = C <= kMaxCapsInLds ? C : 0;
+  hipStream_t st = as_stream(stream);
   const int chunks = (n + kWave - 1) / kWave;
-  a.per_wave = (chunks + kRouteWaves - 1) / kRouteWaves * kWave;
-  const size_t lds_bytes = static_cast<size_t>(kRouteWaves + 3) * E * sizeof(int);
-  hipLaunchKernelGGL(route_by_path_kernel, dim3(1), dim3(kRouteBlock), lds_bytes, as_stream(stream), a);
-  return check_launch("route_by_path_kernel");
+  if (chunks <= kWholeChunks) {
+    a.per_wave = (chunks + kWholeWaves - 1) / kWholeWaves * kWave;
+    const size_t lds_bytes = (static_cast<size_t>(2 * kWholeWaves + 3) * E + a.caps_in_lds) * sizeof(int);
+    hipLaunchKernelGGL((route_kernel<kWhole, kWholeWaves>), dim3(1), dim3(kWholeWaves * kWave), lds_bytes, st, a);
+    return check_launch("route_kernel");
+  }
+  split_geometry(n, &a.units, &a.per_wave);
+  const size_t need = static_cast<size_t>(a.units / kSplitWaves + a.units) * E * sizeof(int);
+  if (workspace == nullptr || workspace_bytes < need || !aligned(workspace, 4))
+    return fail(BRT_E_WORKSPACE, "route_by_path needs %zu bytes of workspace, got %zu", need, workspace_bytes);
+  a.ws = static_cast<int*>(workspace);
+  const dim3 grid(a.units / kSplitWaves), block(kSplitWaves * kWave);
+  const size_t lds_bytes = (static_cast<size_t>(kSplitWaves + 3) * E + a.caps_in_lds) * sizeof(int);
+  hipLaunchKernelGGL((route_kernel<kCount, kSplitWaves>), grid, block, lds_bytes, st, a);
+  hipLaunchKernelGGL((route_kernel<kEmit, kSplitWaves>), grid, block, lds_bytes, st, a);
+  return check_launch("route_kernel");
 }
 
 namespace {

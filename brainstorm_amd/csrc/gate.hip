@@ -50,14 +50,19 @@ __device__ __forceinline__ float load_score(const void* p, size_t i) {
   return half_bits_to_float<DT>(static_cast<const uint16_t*>(p)[i]);
 }
 
-// Sum of v over the aligned lane segments of `width` lanes; every lane gets its segment's total.
 __device__ __forceinline__ float segment_sum(float v, int width) {
-  for (int d = 1; d < width; d <<= 1) v += __shfl_xor(v, d, kWave);
-  return v;
+  return segment_all_reduce(v, width, [](float x, float y) { return x + y; });
 }
 __device__ __forceinline__ float segment_max(float v, int width) {
-  for (int d = 1; d < width; d <<= 1) v = fmaxf(v, __shfl_xor(v, d, kWave));
-  return v;
+  return segment_all_reduce(v, width, [](float x, float y) { return fmaxf(x, y); });
+}
+__device__ __forceinline__ uint32_t segment_max(uint32_t v, int width) {
+  return static_cast<uint32_t>(segment_all_reduce(static_cast<int>(v), width, [](int x, int y) {
+    return static_cast<int>(max(static_cast<uint32_t>(x), static_cast<uint32_t>(y)));
+  }));
+}
+__device__ __forceinline__ int segment_min(int v, int width) {
+  return segment_all_reduce(v, width, [](int x, int y) { return min(x, y); });
 }
 
 template <int DT, bool COMPACT>
@@ -82,8 +87,7 @@ __global__ __launch_bounds__(kBlock) void topk_mask_kernel(GateArgs a) {
     }
     int taken = 0;
     for (int pass = 0; pass < a.k; ++pass) {
-      uint32_t best = key;
-      for (int d = 1; d < ep; d <<= 1) best = max(best, static_cast<uint32_t>(__shfl_xor(static_cast<int>(best), d, kWave)));
+      const uint32_t best = segment_max(key, ep);
       const unsigned long long tied = __ballot(key == best && key != 0) & seg;
       if (tied != 0 && lane == __builtin_ctzll(tied)) {
         taken = 1;
@@ -137,15 +141,13 @@ __global__ __launch_bounds__(kBlock) void topk_mask_wide_kernel(GateArgs a) {
       uint32_t mine = 0;
 #pragma unroll
       for (int c = 0; c < kMaxPerLane; ++c) mine = max(mine, key[c]);
-      uint32_t best = mine;
-      for (int d = 1; d < kWave; d <<= 1) best = max(best, static_cast<uint32_t>(__shfl_xor(static_cast<int>(best), d, kWave)));
+      const uint32_t best = segment_max(mine, kWave);
       // lowest column holding the maximum: lowest c first, then lowest lane
       int my_c = kMaxPerLane;
 #pragma unroll
       for (int c = kMaxPerLane - 1; c >= 0; --c)
         if (key[c] == best && best != 0) my_c = c;
-      int low_c = my_c;
-      for (int d = 1; d < kWave; d <<= 1) low_c = min(low_c, __shfl_xor(low_c, d, kWave));
+      const int low_c = segment_min(my_c, kWave);
       const unsigned long long tied = __ballot(my_c == low_c && my_c < kMaxPerLane);
       if (tied != 0 && lane == __builtin_ctzll(tied)) {
 #pragma unroll

@@ -278,8 +278,10 @@ int brt_hip_combine_by_index(const void* in_data, void* out_data, const void* in
  *   order; entry (t,j) of path e with seat s <= loads[e] owns row start[e] + s, start[e] = sum
  *   of the loads before e, or e * max_path_load when max_path_load != 0 (seats beyond
  *   max_path_load are dropped then).  Rows beyond P are dropped; row_entries is written whole
- *   ([0,P)), it needs no zero fill.  One workgroup: E <= 512, T*k < 2^24, meant for routes of up
- *   to a few 10^4 entries.  No workspace.
+ *   ([0,P)), it needs no zero fill.  E <= 512.  Routes of up to 2048 entries take one launch of
+ *   one workgroup; larger ones two launches that pass per-wavefront counters through the
+ *   workspace (size from brt_hip_route_by_path_workspace_bytes, 4-byte aligned, uninitialised,
+ *   not shared between calls that run at the same time).
  *
  * brt_hip_dispatch_by_rows: dst[r] = src[(row_entries[r]-1) / k] (times weights[row_entries[r]-1]
  *   when weights != NULL, rounded once to the data type), zero rows where row_entries[r] == 0.
@@ -293,10 +295,12 @@ int brt_hip_combine_by_index(const void* in_data, void* out_data, const void* in
  */
 int brt_hip_gate_topk(const void* scores, int T, int E, int k, int dtype, int softmax,
                       int32_t* path_ids, float* weights, int32_t* hot_mask, void* stream);
+size_t brt_hip_route_by_path_workspace_bytes(int T, int k, int E);
 int brt_hip_route_by_path(const int32_t* path_ids, int T, int k, int E, const int32_t* caps, int C,
                           int capacity_padding, int path_wise_padding, int max_path_load,
                           int32_t* loads, int32_t* counts, int32_t* seat_rows,
-                          int32_t* row_entries, int P, void* stream);
+                          int32_t* row_entries, int P, void* workspace, size_t workspace_bytes,
+                          void* stream);
 int brt_hip_dispatch_by_rows(const void* src, void* dst, const float* weights,
                              const int32_t* row_entries, int P, int T, int k, int cell, int dtype,
                              void* stream);

@@ -256,10 +256,12 @@ def route_by_path(path_ids, E, caps=None, capacity_padding=False, path_wise_padd
     d_counts = torch.full((E,), -7, dtype=torch.int32, device="cuda")
     d_rows = torch.full((T, k), -7, dtype=torch.int32, device="cuda")
     d_entries = torch.full((P,), -7, dtype=torch.int32, device="cuda")
+    need = _lib.lib().brt_hip_route_by_path_workspace_bytes(T, k, E)
+    ws = torch.full((max(need, 4),), 0xA5, dtype=torch.uint8, device="cuda")  # content must not matter
     _lib.check(_lib.lib().brt_hip_route_by_path(
         ptr(d_ids), T, k, E, ptr(d_caps), 0 if caps is None else len(caps), int(capacity_padding),
         int(path_wise_padding), int(max_path_load), ptr(d_loads), ptr(d_counts), ptr(d_rows),
-        ptr(d_entries), P, stream()))
+        ptr(d_entries), P, ptr(ws), need, stream()))
     torch.cuda.synchronize()
     return host(d_loads), host(d_counts), host(d_rows), host(d_entries)
 
