@@ -28,6 +28,10 @@ __all__ = [
     "fuse_split_cells_from_paths",
     "combine_with_indices_and_loads",
     "combine_with_src_indices",
+    "gate_topk",
+    "route_by_path",
+    "dispatch_by_rows",
+    "combine_by_rows",
 ]
 
 
@@ -578,3 +582,151 @@ def _sum_rows_by_index(in_data, index, n, shape):
 
 # legacy name (sample/cpp/router.ipynb:258-266) of the seat-index combine
 combine_with_src_indices = combine_with_indices_and_loads
+
+
+# ------------------------------------------------------- compact route format
+# Not in the reference's extension.  The same route as hot mask + seat indices, held as k path
+# ids per cell: ``path_ids [T, k]``, ``weights [T, k]`` (fp32), ``seat_rows [T, k]`` (1-based row of
+# the dispatched buffer, 0 = dropped) and ``row_entries [P]`` (1-based entry ``t*k + j + 1`` of
+# every dispatched row, 0 = padding; for ``k == 1`` these are the row tags of dispatch).
+def gate_topk(score: torch.Tensor, top_k: int, softmax: bool = False,
+              hot_mask: bool = False) -> Tuple[torch.Tensor, ...]:
+    """``(path_ids, weights[, hot_mask])``: the ``top_k`` largest scores of every row in the order
+    of ``torch.topk`` (NaN highest, lowest path among equals) and their weights -- the scores as
+    fp32, or with ``softmax`` their softmax over the row (the router probabilities of
+    benchmark/switch_moe/switch_transformer.py:240-253).  One kernel for what the reference does
+    with ``softmax`` + ``topk`` / ``argmax`` + ``zeros`` + ``scatter_`` (protocol/topk.py:26-31)."""
+    _check_on_device(score, "score")
+    if score.dim() != 2:
+        raise RuntimeError("score must be [cells, paths]")
+    if score.dtype not in _DT:
+        raise NotImplementedError("score data type is not supported")
+    T, E = score.shape
+    if not 0 <= top_k <= E:
+        raise RuntimeError("selected index k out of range")
+    score = score.contiguous()
+    with _device_guard(score.device):
+        ids = torch.empty((T, top_k), dtype=torch.int32, device=score.device)
+        weights = torch.empty((T, top_k), dtype=torch.float32, device=score.device)
+        mask = torch.empty((T, E), dtype=torch.int32, device=score.device) if hot_mask else None
+        if top_k > 0 or hot_mask:
+            _lib.check(_lib.lib().brt_hip_gate_topk(
+                _ptr(score), T, E, int(top_k), _DT[score.dtype], int(bool(softmax)), _ptr(ids),
+                _ptr(weights), _ptr(mask), _stream()))
+    return (ids, weights, mask) if hot_mask else (ids, weights)
+
+
+_route_workspaces = {}
+
+
+def route_by_path(
+    path_ids: torch.Tensor,
+    path_num: int,
+    supported_capacities: Optional[torch.Tensor] = None,
+    capacity_padding: bool = False,
+    path_wise_padding: bool = False,
+    max_path_load: int = 0,
+    rows: Optional[int] = None,
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """``generate_indices_and_loads`` (router.cc:48-80) on path ids instead of a hot mask:
+    ``(loads, counts, seat_rows, row_entries)``.  ``loads`` follow the same capacity rules,
+    ``counts`` are the real rows per path.  ``rows`` is the length of the dispatched buffer:
+    ``path_num * max_path_load`` when padding every path to ``max_path_load``, else by default
+    ``cells * k``, which always holds the ``sum(loads)`` rows of a route without capacity padding
+    (no read-back of the loads is needed to size it; rows behind the last path are padding)."""
+    _check_on_device(path_ids, "path_ids")
+    _check_int32(path_ids, "path_ids")
+    if path_ids.dim() != 2:
+        raise RuntimeError("path_ids must be [cells, k]")
+    path_ids = path_ids.contiguous()
+    T, k = path_ids.shape
+    E = int(path_num)
+    caps = None
+    if supported_capacities is not None:
+        _check_int32(supported_capacities, "supported_capacities")
+        caps = supported_capacities.to(path_ids.device).contiguous()
+    if rows is None:
+        rows = E * int(max_path_load) if max_path_load else T * k
+    with _device_guard(path_ids.device):
+        dev = path_ids.device
+        loads_counts = torch.empty((2, E), dtype=torch.int32, device=dev)
+        seat_rows = torch.empty((T, k), dtype=torch.int32, device=dev)
+        row_entries = torch.empty((rows,), dtype=torch.int32, device=dev)
+        need = _lib.lib().brt_hip_route_by_path_workspace_bytes(T, k, E)
+        key = (dev.index, _stream())
+        ws = _route_workspaces.get(key)
+        if ws is None or ws.numel() < need:
+            ws = torch.empty(max(need, 1 << 16), dtype=torch.uint8, device=dev)
+            _route_workspaces[key] = ws
+        _lib.check(_lib.lib().brt_hip_route_by_path(
+            _ptr(path_ids), T, k, E, _ptr(caps), 0 if caps is None else caps.numel(),
+            int(capacity_padding), int(path_wise_padding), int(max_path_load),
+            _ptr(loads_counts[0]), _ptr(loads_counts[1]), _ptr(seat_rows), _ptr(row_entries),
+            int(rows), _ptr(ws), ws.numel(), _stream()))
+    return loads_counts[0], loads_counts[1], seat_rows, row_entries
+
+
+def dispatch_by_rows(in_data: torch.Tensor, row_entries: torch.Tensor, k: int,
+                     weights: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``out[r] = in_data[(row_entries[r]-1) // k]`` (times ``weights.view(-1)[row_entries[r]-1]``,
+    rounded once), zero rows where ``row_entries[r] == 0``: what ``dispatch_with_indices_and_loads``
+    (router.cc:131-273) writes for the same route, every row written by the kernel."""
+    _check_on_device(in_data, "in_data")
+    _check_on_device(row_entries, "row_entries")
+    _check_int32(row_entries, "row_entries")
+    if in_data.dtype not in _DT:
+        raise NotImplementedError("in_data data type is not supported")
+    in_data = in_data.contiguous()
+    T = in_data.size(0)
+    cell = in_data.numel() // T if T > 0 else 0
+    P = row_entries.numel()
+    if weights is not None:
+        if weights.dtype != torch.float32 or weights.numel() != T * k:
+            raise RuntimeError("weights must be fp32 [cells, k]")
+        weights = weights.contiguous()
+    with _device_guard(in_data.device):
+        out = torch.empty((P,) + tuple(in_data.shape[1:]), dtype=in_data.dtype, device=in_data.device)
+        _lib.check(_lib.lib().brt_hip_dispatch_by_rows(
+            _ptr(in_data), _ptr(out), _ptr(weights), _ptr(row_entries.contiguous()), P, T, int(k),
+            cell, _DT[in_data.dtype], _stream()))
+    return out
+
+
+def combine_by_rows(in_data: torch.Tensor, path_ids: torch.Tensor, seat_rows: torch.Tensor,
+                    weights: Optional[torch.Tensor] = None, out_data: Optional[torch.Tensor] = None,
+                    out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """``out[t] = sum_j weights[t,j] * in_data[seat_rows[t,j]-1]`` over the entries that own a row,
+    in ascending path id, fp32 from zero: the result of ``combine_with_indices_and_loads``
+    (router.cc:372-473) for the same route, bit for bit.  With ``out_data`` the result is
+    written in place and cells without a row keep their value (the residual convention)."""
+    _check_on_device(in_data, "in_data")
+    for t, n in ((path_ids, "path_ids"), (seat_rows, "seat_rows")):
+        _check_on_device(t, n)
+        _check_int32(t, n)
+    if in_data.dtype not in _DT:
+        raise NotImplementedError("in_data data type is not supported")
+    if path_ids.shape != seat_rows.shape or path_ids.dim() != 2:
+        raise RuntimeError("path_ids and seat_rows must both be [cells, k]")
+    in_data = in_data.contiguous()
+    T, k = path_ids.shape
+    P = in_data.size(0)
+    cell = in_data.numel() // P if P > 0 else (out_data.numel() // T if out_data is not None and T > 0 else 0)
+    if weights is not None:
+        if weights.dtype != torch.float32 or weights.numel() != T * k:
+            raise RuntimeError("weights must be fp32 [cells, k]")
+        weights = weights.contiguous()
+    with _device_guard(in_data.device):
+        if out_data is not None:
+            if not out_data.is_contiguous() or out_data.numel() != T * cell:
+                raise RuntimeError("out_data must be a contiguous [cells, ...] tensor")
+            out = out_data
+        else:
+            out = torch.empty((T,) + tuple(in_data.shape[1:]), dtype=out_dtype or in_data.dtype,
+                              device=in_data.device)
+        if out.dtype not in _DT or (out.dtype != in_data.dtype and out.dtype != torch.float32):
+            raise NotImplementedError("output data type is not supported")
+        _lib.check(_lib.lib().brt_hip_combine_by_rows(
+            _ptr(in_data), _ptr(out), _ptr(weights), _ptr(path_ids.contiguous()),
+            _ptr(seat_rows.contiguous()), T, k, cell, P, int(out_data is not None),
+            _DT[in_data.dtype], _DT[out.dtype], _stream()))
+    return out

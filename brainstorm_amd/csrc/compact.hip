@@ -29,7 +29,7 @@ constexpr int kWholeWaves = 8;    // a small route: one workgroup of 8 wavefront
 constexpr int kWholeChunks = 32;  // ... up to this many chunks of 64 entries
 constexpr int kSplitWaves = 4;    // larger routes: workgroups of 4 wavefronts, two launches
 constexpr int kSplitGroups = 32;  // ... in at most this many workgroups
-constexpr int kSplitUnits = kSplitGroups * kSplitWaves;
+constexpr int kSplitWavesLarge = 16;  // ... of 16 wavefronts for routes beyond 32768 entries
 constexpr int kBatch = 4;        // chunks of 64 entries a wavefront keeps in flight
 constexpr int kMaxK = 8;         // paths per cell in combine_by_rows
 constexpr int kMaxRoutePaths = 512;  // (2 * kWholeWaves + 3) * E words of LDS
@@ -330,13 +330,16 @@ __global__ __launch_bounds__(kBlock) void dispatch_by_rows_kernel(RowsArgs a) {
 // dst[t] = sum over the entries of cell t that own a row, in ascending path order, of
 // weight * src[row] (fp32, product and sum rounded separately, starting from 0): the order and
 // the roundings of the dense combine.  Cells without a row keep dst (is_residual) or get zeros.
-template <int IN_DT, int OUT_DT, int LS, int UPR>
+// KMAX >= k entries per cell are held in registers and sorted by path id (entries without a row
+// last), so the row loads of a cell do not depend on each other.
+template <int IN_DT, int OUT_DT, int LS, int UPR, int KMAX>
 __global__ __launch_bounds__(kBlock) void combine_by_rows_kernel(RowsArgs a) {
   using U = u32x4;
   constexpr int NE = 16 / elem_bytes(IN_DT);
   constexpr int OUT_BYTES = NE * elem_bytes(OUT_DT);
   constexpr int LPR = 1 << LS;
   constexpr int GROUPS = kWave >> LS;
+  constexpr int kNone = 0x7fffffff;
   const int lane = threadIdx.x & (kWave - 1);
   const long wave = static_cast<long>(blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6);
   const int gidx = lane >> LS, glane = lane & (LPR - 1);
@@ -348,33 +351,50 @@ __global__ __launch_bounds__(kBlock) void combine_by_rows_kernel(RowsArgs a) {
   for (int tb = 0; tb < nt; tb += GROUPS) {
     const int i = tb + gidx;
     const bool live = i < nt;
-    // Entries of the cell: three independent sets of loads, one memory round trip before the
-    // rows can be fetched.  Every load is unconditional (cell and entry clamped into the tables,
-    // the value dropped afterwards): loads under conditions of their own become branches that
-    // wait for each other.
+    // Entries of the cell: independent loads, one memory round trip before the rows can be
+    // fetched.  Every load is unconditional (cell and entry clamped into the tables, the value
+    // dropped afterwards): loads under conditions of their own become branches that wait for
+    // each other.
     const size_t slot0 = static_cast<size_t>(min(t0 + i, static_cast<long>(a.T) - 1)) * k;
-    int id[kMaxK], row[kMaxK];
-    float g[kMaxK];
+    int id[KMAX], row[KMAX];
+    float g[KMAX];
 #pragma unroll
-    for (int j = 0; j < kMaxK; ++j) {
+    for (int j = 0; j < KMAX; ++j) {
       const int jj = min(j, k - 1);
       row[j] = a.seat_rows[slot0 + jj];
       id[j] = a.ids[slot0 + jj];
     }
     if (a.weights != nullptr) {
 #pragma unroll
-      for (int j = 0; j < kMaxK; ++j) g[j] = a.weights[slot0 + min(j, k - 1)];
+      for (int j = 0; j < KMAX; ++j) g[j] = a.weights[slot0 + min(j, k - 1)];
     } else {
 #pragma unroll
-      for (int j = 0; j < kMaxK; ++j) g[j] = 1.0f;
+      for (int j = 0; j < KMAX; ++j) g[j] = 1.0f;
     }
-    int owned = 0;
 #pragma unroll
-    for (int j = 0; j < kMaxK; ++j) {
-      if (!live || j >= k || row[j] < 0 || row[j] > a.P) row[j] = 0;
-      if (row[j] == 0) id[j] = 0x7fffffff;
-      owned += row[j] != 0;
+    for (int j = 0; j < KMAX; ++j) {
+      if (!live || j >= k || row[j] < 1 || row[j] > a.P) id[j] = kNone;
     }
+    // ascending path id by odd-even transposition (stable: of two entries that name the same
+    // path the first stays first, and only it is used)
+#pragma unroll
+    for (int round = 0; round < KMAX; ++round) {
+#pragma unroll
+      for (int j = round & 1; j + 1 < KMAX; j += 2) {
+        const bool swap = id[j] > id[j + 1];
+        const int ti = id[j], tr = row[j];
+        const float tg = g[j];
+        id[j] = swap ? id[j + 1] : ti;
+        row[j] = swap ? row[j + 1] : tr;
+        g[j] = swap ? g[j + 1] : tg;
+        id[j + 1] = swap ? ti : id[j + 1];
+        row[j + 1] = swap ? tr : row[j + 1];
+        g[j + 1] = swap ? tg : g[j + 1];
+      }
+    }
+    bool use[KMAX];
+#pragma unroll
+    for (int j = 0; j < KMAX; ++j) use[j] = id[j] != kNone && (j == 0 || id[j] != id[j - 1]);
     const size_t to = static_cast<size_t>(t0 + i) * cpr;
     for (int off0 = 0; off0 < cpr; off0 += LPR * UPR) {
       float acc[UPR][NE];
@@ -382,38 +402,26 @@ __global__ __launch_bounds__(kBlock) void combine_by_rows_kernel(RowsArgs a) {
       for (int u = 0; u < UPR; ++u)
 #pragma unroll
         for (int q = 0; q < NE; ++q) acc[u][q] = 0.0f;
-      int last = -1;
-      for (int pass = 0; pass < owned; ++pass) {
-        // the entry with the lowest path id above the last one taken
-        int best = 0x7fffffff, sr = 0;
-        float gg = 1.0f;
 #pragma unroll
-        for (int j = 0; j < kMaxK; ++j) {
-          const bool better = id[j] > last && id[j] < best;
-          best = better ? id[j] : best;
-          sr = better ? row[j] : sr;
-          gg = better ? g[j] : gg;
-        }
-        const bool has = best != 0x7fffffff;  // false only for a cell that names a path twice
-        last = best;
+      for (int j = 0; j < KMAX; ++j) {
         U val[UPR];
 #pragma unroll
         for (int u = 0; u < UPR; ++u) {
           const int off = off0 + u * LPR + glane;
-          if (has && off < cpr) val[u] = src[static_cast<size_t>(sr - 1) * cpr + off];
+          if (use[j] && off < cpr) val[u] = src[static_cast<size_t>(row[j] - 1) * cpr + off];
         }
 #pragma unroll
         for (int u = 0; u < UPR; ++u) {
           const int off = off0 + u * LPR + glane;
-          if (has && off < cpr) {
+          if (use[j] && off < cpr) {
             float x[NE];
             unpack<IN_DT, 16>(val[u], x);
 #pragma unroll
-            for (int q = 0; q < NE; ++q) acc[u][q] = acc[u][q] + x[q] * gg;
+            for (int q = 0; q < NE; ++q) acc[u][q] = acc[u][q] + x[q] * g[j];
           }
         }
       }
-      if (live && (owned != 0 || !a.is_residual)) {
+      if (live && (use[0] || !a.is_residual)) {
 #pragma unroll
         for (int u = 0; u < UPR; ++u) {
           const int off = off0 + u * LPR + glane;
@@ -437,12 +445,16 @@ using namespace brt;
 
 namespace {
 
-// Units and entries per unit of the two-launch form.
-void split_geometry(int n, int* units, int* per_wave) {
+// Wavefronts per workgroup, units and entries per unit of the two-launch form: at most
+// kSplitGroups workgroups, of 4 wavefronts while that keeps a unit within one batch of chunks, of
+// 16 beyond.
+void split_geometry(int n, int* waves, int* units, int* per_wave) {
   const int chunks = (n + kWave - 1) / kWave;
-  const int chunks_pw = std::max(1, (chunks + kSplitUnits - 1) / kSplitUnits);
+  *waves = chunks <= kSplitGroups * kSplitWaves * kBatch ? kSplitWaves : kSplitWavesLarge;
+  const int most = kSplitGroups * *waves;
+  const int chunks_pw = std::max(1, (chunks + most - 1) / most);
   const int used = (chunks + chunks_pw - 1) / chunks_pw;
-  *units = (used + kSplitWaves - 1) / kSplitWaves * kSplitWaves;
+  *units = (used + *waves - 1) / *waves * *waves;
   *per_wave = chunks_pw * kWave;
 }
 
@@ -450,9 +462,9 @@ void split_geometry(int n, int* units, int* per_wave) {
 
 extern "C" size_t brt_hip_route_by_path_workspace_bytes(int T, int k, int E) {
   if (T <= 0 || k <= 0 || E <= 0 || static_cast<long>(T) * k >= (1l << 31)) return 0;
-  int units, per_wave;
-  split_geometry(T * k, &units, &per_wave);
-  return static_cast<size_t>(units / kSplitWaves + units) * E * sizeof(int);
+  int waves, units, per_wave;
+  split_geometry(T * k, &waves, &units, &per_wave);
+  return static_cast<size_t>(units / waves + units) * E * sizeof(int);
 }
 
 extern "C" int brt_hip_route_by_path(const int32_t* path_ids, int T, int k, int E, const int32_t* caps,
@@ -491,15 +503,21 @@ extern "C" int brt_hip_route_by_path(const int32_t* path_ids, int T, int k, int 
     hipLaunchKernelGGL((route_kernel<kWhole, kWholeWaves>), dim3(1), dim3(kWholeWaves * kWave), lds_bytes, st, a);
     return check_launch("route_kernel");
   }
-  split_geometry(n, &a.units, &a.per_wave);
-  const size_t need = static_cast<size_t>(a.units / kSplitWaves + a.units) * E * sizeof(int);
+  int waves;
+  split_geometry(n, &waves, &a.units, &a.per_wave);
+  const size_t need = static_cast<size_t>(a.units / waves + a.units) * E * sizeof(int);
   if (workspace == nullptr || workspace_bytes < need || !aligned(workspace, 4))
     return fail(BRT_E_WORKSPACE, "route_by_path needs %zu bytes of workspace, got %zu", need, workspace_bytes);
   a.ws = static_cast<int*>(workspace);
-  const dim3 grid(a.units / kSplitWaves), block(kSplitWaves * kWave);
-  const size_t lds_bytes = (static_cast<size_t>(kSplitWaves + 3) * E + a.caps_in_lds) * sizeof(int);
-  hipLaunchKernelGGL((route_kernel<kCount, kSplitWaves>), grid, block, lds_bytes, st, a);
-  hipLaunchKernelGGL((route_kernel<kEmit, kSplitWaves>), grid, block, lds_bytes, st, a);
+  const dim3 grid(a.units / waves), block(waves * kWave);
+  const size_t lds_bytes = (static_cast<size_t>(waves + 3) * E + a.caps_in_lds) * sizeof(int);
+  if (waves == kSplitWaves) {
+    hipLaunchKernelGGL((route_kernel<kCount, kSplitWaves>), grid, block, lds_bytes, st, a);
+    hipLaunchKernelGGL((route_kernel<kEmit, kSplitWaves>), grid, block, lds_bytes, st, a);
+  } else {
+    hipLaunchKernelGGL((route_kernel<kCount, kSplitWavesLarge>), grid, block, lds_bytes, st, a);
+    hipLaunchKernelGGL((route_kernel<kEmit, kSplitWavesLarge>), grid, block, lds_bytes, st, a);
+  }
   return check_launch("route_kernel");
 }
 
@@ -577,16 +595,21 @@ extern "C" int brt_hip_combine_by_rows(const void* src, void* dst, const float* 
   const int waves_pb = kBlock / kWave;
   const dim3 grid(static_cast<unsigned>((n_waves + waves_pb - 1) / waves_pb)), block(kBlock);
   hipStream_t st = as_stream(stream);
-#define BRT_LAUNCH(IN, OUT)                                                                              \
-  with_row_shape(a.cpr, [&](auto ls, auto upr) {                                                         \
-    hipLaunchKernelGGL((combine_by_rows_kernel<IN, OUT, decltype(ls)::value, decltype(upr)::value>),     \
-                       grid, block, 0, st, a);                                                           \
+#define BRT_LAUNCH_K(IN, OUT, KMAX)                                                                          \
+  with_row_shape(a.cpr, [&](auto ls, auto upr) {                                                             \
+    hipLaunchKernelGGL((combine_by_rows_kernel<IN, OUT, decltype(ls)::value, decltype(upr)::value, KMAX>),   \
+                       grid, block, 0, st, a);                                                               \
   });
+#define BRT_LAUNCH(IN, OUT)                 \
+  if (k == 1) BRT_LAUNCH_K(IN, OUT, 1)      \
+  else if (k == 2) BRT_LAUNCH_K(IN, OUT, 2) \
+  else BRT_LAUNCH_K(IN, OUT, kMaxK)
   if (in_dtype == BRT_F32) BRT_LAUNCH(BRT_F32, BRT_F32)
   else if (in_dtype == BRT_F16 && out_dtype == BRT_F16) BRT_LAUNCH(BRT_F16, BRT_F16)
   else if (in_dtype == BRT_F16) BRT_LAUNCH(BRT_F16, BRT_F32)
   else if (out_dtype == BRT_BF16) BRT_LAUNCH(BRT_BF16, BRT_BF16)
   else BRT_LAUNCH(BRT_BF16, BRT_F32)
 #undef BRT_LAUNCH
+#undef BRT_LAUNCH_K
   return check_launch("combine_by_rows_kernel");
 }

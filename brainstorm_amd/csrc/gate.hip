@@ -193,9 +193,10 @@ int launch_gate(GateArgs a, int dtype, bool compact, void* stream) {
   while ((1 << shift) < std::min(E, kWave)) ++shift;
   a.ep_shift = shift;
   const int rps = E <= kWave ? kWave >> shift : 1;
-  // enough wavefronts to cover the chip a few times over, whole steps per wavefront
-  long rows = std::max<long>(rps, (T + 8191) / 8192 * rps);
-  rows = std::min<long>(rows, 16l * rps);
+  // about 8192 wavefronts (the chip a few times over), whole steps per wavefront: a wavefront's
+  // steps run one after the other, each a full memory round trip
+  long rows = ((T + 8191) / 8192 + rps - 1) / rps * rps;
+  rows = std::min<long>(std::max<long>(rows, rps), 16l * rps);
   a.rows_pw = static_cast<int>(rows);
   const long n_waves = (T + a.rows_pw - 1) / a.rows_pw;
   const int waves_pb = kBlock / kWave;

@@ -393,3 +393,51 @@ def test_capacity_padded_moe_layer_replays_from_a_hip_graph(brt_mod):
         torch.cuda.synchronize()
         assert torch.equal(captured, want)
         assert captured.abs().sum() > 0
+
+
+@pytest.mark.parametrize("top_k,dtype", [(1, torch.bfloat16), (2, torch.float32)])
+def test_compact_route_ops_equal_the_routers(brt_mod, top_k, dtype):
+    """gate_topk -> route_by_path -> dispatch_by_rows -> experts -> combine_by_rows gives, bit for
+    bit, what ScatterRouter(topk, fused_dispatch) -> experts -> GatherRouter(fused_combine) gives."""
+    brt, c_router, ScatterRouter, GatherRouter = brt_mod
+    T, E, d, cap = 3000, 16, 256, 200
+    rng = np.random.default_rng(21 + top_k)
+    logits = torch.from_numpy(rng.standard_normal((T, E)).astype(np.float32)).cuda()
+    x = torch.from_numpy(rng.standard_normal((T, d)).astype(np.float32)).cuda().to(dtype)
+    caps = torch.tensor([cap], dtype=torch.int32)
+
+    scatter = ScatterRouter(protocol_type="topk", fabric_type="fused_dispatch",
+                            protocol_kwargs={"top_k": top_k},
+                            fabric_kwargs={"supported_capacities": [cap]}).cuda()
+    gather = GatherRouter(fabric_type="fused_combine").cuda()
+    routed = scatter(brt.Annotator([0])(x), logits)
+    dense_rows = brt.to_torch_tensor(routed)
+    dense_idx, dense_loads = routed.tag, routed.load    # the gather pops them from the stacks
+    dense_out = gather(routed * 2, x.clone())
+
+    ids, weights, mask = c_router.gate_topk(logits, top_k, softmax=True, hot_mask=True)
+    want = torch.topk(logits, top_k, dim=1)
+    assert torch.equal(ids.long(), want.indices)
+    probs = torch.softmax(logits, dim=1).gather(1, want.indices)
+    assert torch.allclose(weights, probs, rtol=2e-6, atol=0)
+    assert torch.equal(mask, c_router.topk_hot_mask(logits, top_k))
+    loads, counts, seat_rows, row_entries = c_router.route_by_path(ids, E, caps)
+    assert torch.equal(loads, dense_loads) and torch.equal(counts, mask.sum(0).int())
+    P = int(loads.sum())
+    assert row_entries.numel() == T * top_k and not row_entries[P:].any()
+    y = c_router.dispatch_by_rows(x, row_entries, top_k)
+    assert torch.equal(y[:P].view(torch.int16 if dtype == torch.bfloat16 else torch.int32),
+                       dense_rows.view(torch.int16 if dtype == torch.bfloat16 else torch.int32))
+    out = c_router.combine_by_rows(y * 2, ids, seat_rows, out_data=x.clone())
+    assert torch.equal(out, torch.as_tensor(dense_out))
+    # weighted, no residual, fp32 result: against the dense op with the gates scattered to [T, E]
+    gates = torch.zeros(T, E, device="cuda").scatter_(1, ids.long(), weights)
+    w_out = c_router.combine_by_rows(y, ids, seat_rows, weights=weights, out_dtype=torch.float32)
+    d_out = c_router.combine_with_indices_and_loads(
+        y[:P], dense_idx, dense_loads, gates.to(dtype) if dtype != torch.float32 else gates)[0]
+    if dtype == torch.float32:
+        assert torch.equal(w_out, d_out)
+    with pytest.raises(RuntimeError):
+        c_router.route_by_path(ids.long(), E)
+    with pytest.raises(RuntimeError):
+        c_router.dispatch_by_rows(x, row_entries, top_k, weights=weights.half())
