@@ -293,8 +293,8 @@ def combine_by_rows(y_bits, path_ids, seat_rows, weights=None, out_bits=None, in
     rows = np.ascontiguousarray(seat_rows, dtype=np.int32)
     T, k = ids.shape
     P = y_bits.shape[0]
-    cell = y_bits.size // max(P, 1)
-    d_y = dev(y_bits.reshape(P, -1))
+    cell = int(np.prod(y_bits.shape[1:]))
+    d_y = dev(y_bits.reshape(P, cell))
     d_w = None if weights is None else dev(np.ascontiguousarray(weights, dtype=np.float32))
     if out_bits is not None:
         d_out = dev(np.ascontiguousarray(out_bits).reshape(T, cell))

@@ -657,3 +657,27 @@ def test_combine_by_rows_order_and_bad_rows(hip):
     got = hip.dispatch_by_rows(x, entries, 1)
     assert np.array_equal(got, oracle.dispatch_by_rows(x, entries, 1))
     assert np.array_equal(got[3], x[1]) and not got[:3].any()
+
+
+def test_compact_route_empty_and_tiny_inputs(hip):
+    # no cells: loads follow the rules for empty paths, every row is padding
+    ids = np.zeros((0, 2), dtype=np.int32)
+    for caps, pad, pw in ((None, False, False), ([4, 8], True, False), ([3, 5, 7], True, True)):
+        want = oracle.route_by_path(ids, 3, caps, pad, pw, 0, 6)
+        got = hip.route_by_path(ids, 3, caps, pad, pw, 0, 6)
+        for g, w in zip(got, want):
+            assert np.array_equal(g, w)
+        assert not got[3].any()
+    # one cell, one path; k = 0 entries per cell
+    got = hip.route_by_path(np.array([[0]], dtype=np.int32), 1)
+    assert got[0].tolist() == [1] and got[2].tolist() == [[1]] and got[3].tolist() == [1]
+    got = hip.route_by_path(np.zeros((5, 0), dtype=np.int32), 4, P=3)
+    assert not got[0].any() and not got[3].any()
+    ids0, w0 = hip.gate_topk(np.zeros((4, 6), dtype=np.float32), 0)
+    assert ids0.shape == (4, 0) and w0.shape == (4, 0)
+    # empty row sets
+    x = np.ones((3, 8), dtype=np.float32)
+    assert hip.dispatch_by_rows(x, np.zeros((0,), dtype=np.int32), 1).shape == (0, 8)
+    out = hip.combine_by_rows(np.zeros((0, 8), dtype=np.float32), np.zeros((3, 1), dtype=np.int32),
+                              np.zeros((3, 1), dtype=np.int32), out_bits=x)
+    assert np.array_equal(out, x)                              # nothing routed: the residual stays
