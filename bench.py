@@ -356,11 +356,28 @@ def main():
             (c_y2 if have_ffn else c_y).data_ptr(), c_out.data_ptr(), c_entries.data_ptr(), P, D, T,
             _lib.BF16, _lib.BF16, sptr()))
 
+    # ... and with dispatch and combine folded into the GEMMs as well (rows named by the entries)
+    c_out_fused = x.clone()
+
+    def step_compact_fused():
+        k_route_compact()
+        _lib.check(L.brt_hip_grouped_gemm_by_rows(
+            x.data_ptr(), wi_tab.data_ptr(), None, c_h.data_ptr(), c_loads_counts[0].data_ptr(),
+            c_entries.data_ptr(), 1, E, P, T, D, DFF, _lib.ACT_GELU, 1, 0, sptr()))
+        _lib.check(L.brt_hip_grouped_gemm_by_rows(
+            c_h.data_ptr(), wo_tab.data_ptr(), None, c_out_fused.data_ptr(),
+            c_loads_counts[0].data_ptr(), c_entries.data_ptr(), 1, E, P, T, DFF, D, _lib.ACT_NONE,
+            0, 1, sptr()))
+
     with torch.cuda.stream(stream):
         k_gate_compact()
         step_compact()
         k_combine_rows()
+        if have_ffn:
+            step_compact_fused()
     stream.synchronize()
+    if have_ffn and not torch.equal(c_out_fused.view(torch.int16), out.view(torch.int16)):
+        sys.exit("bench.py: the compact layer with routing folded into the GEMMs disagrees")
     if not torch.equal(c_ids.view(-1).long(), expert.to(dev)):
         sys.exit("bench.py: the compact gate does not reproduce the argmax")
     if not torch.allclose(c_w.view(-1).cpu(), probs.max(dim=1).values, rtol=2e-6, atol=0):
@@ -372,6 +389,11 @@ def main():
     g_compact = capture(step_compact, args.steps)
     timed(g_compact, 1)
     compact_layer_us = timed(g_compact, 1) / args.steps * 1e3
+    compact_fused_layer_us = None
+    if have_ffn:
+        g_compact_fused = capture(step_compact_fused, args.steps)
+        timed(g_compact_fused, 1)
+        compact_fused_layer_us = timed(g_compact_fused, 1) / args.steps * 1e3
 
     # the library's batched GEMM on the same FFN, every expert padded to the full capacity (the
     # only shape a batched routine takes), GELU as its own elementwise launch: reported beside
@@ -589,6 +611,8 @@ def main():
         "layer_us_one_graph_launch_per_step": round(per_graph_launch_us, 2),
         "layer_compact_us": round(compact_layer_us, 2),
         "layer_compact_step": "route from path ids+dispatch by rows+ffn+combine by row tags; K steps in one HIP graph",
+        "layer_compact_fused_us": None if compact_fused_layer_us is None else round(compact_fused_layer_us, 2),
+        "layer_compact_fused_step": "route from path ids+GEMM1 gathering cells+GEMM2 scattering to cells, rows named by the row entries; K steps in one HIP graph",
         "layer_fused_us": None if fused_layer_us is None else round(fused_layer_us, 2),
         "layer_fused_step": "indexgen(tag indices)+GEMM1 gathering cells+GEMM2 scattering to cells; K steps in one HIP graph",
         "wall_ms_timed_region": round(wall_ms, 3),

@@ -67,6 +67,11 @@ SIGNATURES = {
         [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int,
          _c_int, _c_int, _c_int, _c_ptr],
     ),
+    "brt_hip_grouped_gemm_by_rows": (
+        _c_int,
+        [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
+         _c_int, _c_int, _c_int, _c_ptr],
+    ),
     "brt_hip_unique_tags_workspace_bytes": (_c_size, [ctypes.c_long, ctypes.c_long]),
     "brt_hip_unique_tags": (
         _c_int,

@@ -61,7 +61,10 @@ struct GemmArgs {
   const __bf16* const* bias;
   __bf16* out;
   const int* loads;
-  const int* tags;  // [T,E] tag matrix (column e: 1-based cells of path e in seat order) or null
+  const int* tags;  // [T,E] tag matrix (column e: 1-based cells of path e in seat order), or the
+                    // row-entry vector [P] of the compact route (1-based entry t*k+j+1 per row), or null
+  int tag_vector;   // tags is the row-entry vector
+  int tag_div;      // entries per cell (k) of the row-entry vector
   int E, P, K, N, T;
   int gather, scatter;  // rows of x / of out are addressed through the tags
   int tiles_n, tiles_m_max;
@@ -182,6 +185,18 @@ __global__ __launch_bounds__(WAVES * 64) void grouped_gemm_kernel(GemmArgs a) {
   // operand load); an empty tag addresses past the extent and so reads a row of zeros, which
   // is what dispatch writes for a padding row.
   const bool gather = a.gather != 0;
+  // 0-based cell behind row r of this tile, -1 for an empty slot: from the tag matrix (seat
+  // seat0 + r of column e), or from the row-entry vector of the compact route (entry t*k+j+1 of
+  // row row0 + r of the dispatched layout)
+  auto cell_of_row = [&](int r) {
+    if (a.tag_vector) {
+      const int entry = a.tags[static_cast<size_t>(row0) + r];
+      const int cell = a.tag_div > 1 ? (entry - 1) / a.tag_div : entry - 1;
+      return (entry >= 1 && cell < a.T) ? cell : -1;
+    }
+    const int tag = a.tags[static_cast<size_t>(seat0 + r) * a.E + e];
+    return (tag >= 1 && tag <= a.T) ? tag - 1 : -1;
+  };
   const char* xa = reinterpret_cast<const char*>(gather ? a.x : a.x + static_cast<size_t>(row0) * K);
   const __bf16* const w_e = a.w[e];
   const size_t xa_bytes = static_cast<size_t>(gather ? a.T : a.P - row0) * K * 2;
@@ -205,8 +220,8 @@ __global__ __launch_bounds__(WAVES * 64) void grouped_gemm_kernel(GemmArgs a) {
     const int r = lr + i * ROWS_PER_PASS;
     const bool in_tile = r < rows;
     if (gather) {
-      const int tag = in_tile ? a.tags[static_cast<size_t>(seat0 + r) * a.E + e] : 0;
-      off_a[i] = (tag >= 1 && tag <= a.T) ? (static_cast<uint32_t>(tag - 1) * K + lc * 8) * 2 : 0x80000000u;
+      const int cell = in_tile ? cell_of_row(r) : -1;
+      off_a[i] = cell >= 0 ? (static_cast<uint32_t>(cell) * K + lc * 8) * 2 : 0x80000000u;
     } else {
       off_a[i] = in_tile ? (static_cast<uint32_t>(r) * K + lc * 8) * 2 : 0x80000000u;
     }
@@ -441,10 +456,7 @@ __global__ __launch_bounds__(WAVES * 64) void grouped_gemm_kernel(GemmArgs a) {
         const int rl = q / OUT_CHUNKS, c = q - rl * OUT_CHUNKS;
         const int r = r_lo + rl;
         long to = r;
-        if (a.scatter) {
-          const int tag = a.tags[static_cast<size_t>(seat0 + r) * a.E + e];
-          to = (tag >= 1 && tag <= a.T) ? tag - 1 : -1;
-        }
+        if (a.scatter) to = cell_of_row(r);
         // streaming stores: the output is not read again by this kernel, and written through the
         // L2 like ordinary stores it pushes the operand lines out that the column tiles share
         if (to >= 0 && n0 + c * 8 < a.N)
@@ -539,8 +551,8 @@ using namespace brt;
 namespace {
 
 int grouped_gemm_impl(const void* x, const void* const* weights, const void* const* biases, void* out,
-                      const int32_t* loads, const int32_t* tags, int E, int P, int T, int K, int N,
-                      int act, int gather_in, int scatter_out, void* stream) {
+                      const int32_t* loads, const int32_t* tags, int entries_per_cell, int E, int P,
+                      int T, int K, int N, int act, int gather_in, int scatter_out, void* stream) {
   if (E <= 0 || P < 0 || K <= 0 || N <= 0 || T < 0)
     return fail(BRT_E_INVALID, "bad shape E=%d P=%d T=%d K=%d N=%d", E, P, T, K, N);
   if (K % 8 != 0 || N % 8 != 0)
@@ -561,6 +573,8 @@ int grouped_gemm_impl(const void* x, const void* const* weights, const void* con
   a.out = static_cast<__bf16*>(out);
   a.loads = loads;
   a.tags = tags;
+  a.tag_vector = entries_per_cell > 0;
+  a.tag_div = entries_per_cell;
   a.E = E; a.P = P; a.K = K; a.N = N; a.T = T;
   a.gather = gather_in != 0; a.scatter = scatter_out != 0;
   // Tile choice.  A wavefront owns 160 x 64 outputs (7 LDS fragment reads feed 10 MFMAs); a
@@ -593,7 +607,7 @@ int grouped_gemm_impl(const void* x, const void* const* weights, const void* con
 extern "C" int brt_hip_grouped_gemm(const void* x, const void* const* weights,
                                     const void* const* biases, void* out, const int32_t* loads,
                                     int E, int P, int K, int N, int act, void* stream) {
-  return grouped_gemm_impl(x, weights, biases, out, loads, nullptr, E, P, 0, K, N, act, 0, 0, stream);
+  return grouped_gemm_impl(x, weights, biases, out, loads, nullptr, 0, E, P, 0, K, N, act, 0, 0, stream);
 }
 
 extern "C" int brt_hip_grouped_gemm_routed(const void* x, const void* const* weights,
@@ -601,6 +615,18 @@ extern "C" int brt_hip_grouped_gemm_routed(const void* x, const void* const* wei
                                            const int32_t* loads, const int32_t* tags, int E, int P,
                                            int T, int K, int N, int act, int gather_in,
                                            int scatter_out, void* stream) {
-  return grouped_gemm_impl(x, weights, biases, out, loads, tags, E, P, T, K, N, act, gather_in,
+  return grouped_gemm_impl(x, weights, biases, out, loads, tags, 0, E, P, T, K, N, act, gather_in,
                            scatter_out, stream);
+}
+
+extern "C" int brt_hip_grouped_gemm_by_rows(const void* x, const void* const* weights,
+                                            const void* const* biases, void* out,
+                                            const int32_t* loads, const int32_t* row_entries, int k,
+                                            int E, int P, int T, int K, int N, int act,
+                                            int gather_in, int scatter_out, void* stream) {
+  if (k <= 0) return fail(BRT_E_INVALID, "entries per cell must be positive, got %d", k);
+  if (scatter_out && k != 1)
+    return fail(BRT_E_UNSUPPORTED, "scatter_out needs one path per cell (k = %d)", k);
+  return grouped_gemm_impl(x, weights, biases, out, loads, row_entries, k, E, P, T, K, N, act,
+                           gather_in, scatter_out, stream);
 }

@@ -45,7 +45,8 @@ def grouped_linear(x: torch.Tensor, out: torch.Tensor, weight_table: torch.Tenso
                    bias_table: Optional[torch.Tensor], loads: torch.Tensor, in_features: int,
                    out_features: int, activation: Optional[str] = None, *,
                    tags: Optional[torch.Tensor] = None, gather: bool = False,
-                   scatter: bool = False, rows: Optional[int] = None) -> torch.Tensor:
+                   scatter: bool = False, rows: Optional[int] = None,
+                   row_entries: Optional[torch.Tensor] = None, entries_per_cell: int = 1) -> torch.Tensor:
     """``out[s_e : s_e + loads[e]] = act(x[s_e : s_e + loads[e]] @ W_e^T + b_e)`` for every
     branch e, ``s_e = sum(loads[:e])``, in one launch.  ``weight_table`` /
     ``bias_table`` are int64 device tensors holding the branch pointers.
@@ -55,7 +56,11 @@ def grouped_linear(x: torch.Tensor, out: torch.Tensor, weight_table: torch.Tenso
     GEMM: ``gather=True`` reads row s of branch e from ``x[tags[s, e] - 1]`` (``x`` is the
     cell-major tensor, no dispatch needed), ``scatter=True`` stores it to
     ``out[tags[s, e] - 1]`` (``out`` is cell-major and doubles as the residual; single-path
-    routes only).  ``rows`` bounds ``sum(loads)`` when neither side is path-major."""
+    routes only).  ``rows`` bounds ``sum(loads)`` when neither side is path-major.
+
+    ``row_entries`` (the vector ``route_by_path`` writes: 1-based entry ``t * k + j + 1`` of every
+    row of the dispatched layout, ``k = entries_per_cell``) names the rows instead of ``tags``:
+    row r is cell ``(row_entries[r] - 1) // k``."""
     if x.dtype != torch.bfloat16 or out.dtype != torch.bfloat16:
         raise NotImplementedError("the grouped GEMM computes in bf16 (fp32 accumulation)")
     if not (x.is_cuda and out.is_cuda and loads.is_cuda):
@@ -68,7 +73,17 @@ def grouped_linear(x: torch.Tensor, out: torch.Tensor, weight_table: torch.Tenso
         raise RuntimeError("shared inputs do not match [rows, in_features] / [rows, out_features]")
     routed = gather or scatter
     cells = 0
-    if routed:
+    if routed and row_entries is not None:
+        if not row_entries.is_cuda or row_entries.dtype != torch.int32 or not row_entries.is_contiguous():
+            raise RuntimeError("row_entries must be a contiguous int32 vector on the device")
+        if gather and scatter and x.shape[0] != out.shape[0]:
+            raise RuntimeError("a gathered input / scattered output has one row per cell")
+        cells = x.shape[0] if gather else out.shape[0]
+        if rows is None:
+            rows = row_entries.numel()
+        elif rows > row_entries.numel():
+            raise RuntimeError("rows exceeds the row-entry vector")
+    elif routed:
         if tags is None or not tags.is_cuda or tags.dtype != torch.int32 or not tags.is_contiguous():
             raise RuntimeError("gather/scatter need the contiguous int32 tag-index matrix on the device")
         cells = tags.shape[0]
@@ -86,7 +101,12 @@ def grouped_linear(x: torch.Tensor, out: torch.Tensor, weight_table: torch.Tenso
         lib = _lib.lib()
         stream = torch._C._cuda_getCurrentRawStream(torch._C._cuda_getDevice())
         bias_ptr = None if bias_table is None else bias_table.data_ptr()
-        if routed:
+        if routed and row_entries is not None:
+            _lib.check(lib.brt_hip_grouped_gemm_by_rows(
+                x.data_ptr(), weight_table.data_ptr(), bias_ptr, out.data_ptr(), loads.data_ptr(),
+                row_entries.data_ptr(), int(entries_per_cell), loads.numel(), rows, cells,
+                in_features, out_features, _ACT[activation], int(gather), int(scatter), stream))
+        elif routed:
             _lib.check(lib.brt_hip_grouped_gemm_routed(
                 x.data_ptr(), weight_table.data_ptr(), bias_ptr, out.data_ptr(), loads.data_ptr(),
                 tags.data_ptr(), loads.numel(), rows, cells, in_features, out_features,

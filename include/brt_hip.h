@@ -220,6 +220,19 @@ int brt_hip_grouped_gemm_routed(const void* x, const void* const* weights,
                                 const int32_t* tags, int E, int P, int T, int K, int N, int act,
                                 int gather_in, int scatter_out, void* stream);
 
+/*
+ * The routed grouped GEMM on the compact route (no counterpart in the reference): as
+ * brt_hip_grouped_gemm_routed, with the rows named by the row_entries vector [P] that
+ * brt_hip_route_by_path writes (1-based entry t*k+j+1 of each row of the dispatched layout,
+ * 0 = padding row) instead of the [T,E] tag matrix.  Row r of the layout is cell
+ * (row_entries[r]-1)/k of x (gather_in) or of out (scatter_out; k must be 1).  Rows of path e
+ * start at sum(loads[:e]) (no max_path_load layout).
+ */
+int brt_hip_grouped_gemm_by_rows(const void* x, const void* const* weights,
+                                 const void* const* biases, void* out, const int32_t* loads,
+                                 const int32_t* row_entries, int k, int E, int P, int T, int K,
+                                 int N, int act, int gather_in, int scatter_out, void* stream);
+
 /* ---------------------------------------------------------------------------
  * Tag-index gather (the default GatherRouter path of the reference).
  *

@@ -160,6 +160,18 @@ def test_ffn_with_gather_and_scatter_equals_dispatch_ffn_combine(T, E, d, dff, c
     grouped_linear(hf, out, t2, None, loads, dff, d, tags=tags, scatter=True, rows=P)
     assert torch.equal(out.view(torch.int16), want.view(torch.int16))
 
+    # the same with the rows named by the row-entry vector of the compact route
+    ids = torch.from_numpy(mask.argmax(1).astype(np.int32)).cuda().view(T, 1)
+    loads_c, _, _, row_entries = c_router.route_by_path(ids, E, caps, pad, rows=P)
+    assert torch.equal(loads_c, loads)
+    hr = torch.full((P + 7, dff), float("nan"), dtype=torch.bfloat16, device="cuda")
+    out_r = x.clone()
+    grouped_linear(x, hr, t1, None, loads, d, dff, "gelu", row_entries=row_entries, gather=True, rows=P)
+    assert torch.equal(hr[:P].view(torch.int16), h.view(torch.int16))
+    assert torch.isnan(hr[P:].float()).all()
+    grouped_linear(hr, out_r, t2, None, loads, dff, d, row_entries=row_entries, scatter=True, rows=P)
+    assert torch.equal(out_r.view(torch.int16), want.view(torch.int16))
+
     # and both agree with per-expert torch matmuls on the cells each expert kept
     lh = loads.cpu().tolist()
     ref = x.float().clone()
@@ -170,6 +182,30 @@ def test_ffn_with_gather_and_scatter_equals_dispatch_ffn_combine(T, E, d, dff, c
             ref[cells] = hid.float() @ w2[e].float().t()
     scale = ref.abs().max()
     assert (out.float() - ref).abs().max() / scale < 1e-2
+
+
+def test_gathering_gemm_on_a_top2_compact_route():
+    """Two entries per cell: the GEMM that reads its rows through row_entries gives what
+    dispatch_by_rows followed by the plain grouped GEMM gives, bit for bit."""
+    from brainstorm_amd._C import router as c_router
+    from brainstorm_amd.jit import grouped_linear
+
+    T, E, d, dff, k = 1500, 12, 128, 256, 2
+    g = torch.Generator().manual_seed(9)
+    x = torch.randn(T, d, generator=g).to(torch.bfloat16).cuda()
+    ids, _ = c_router.gate_topk(torch.randn(T, E, generator=g).cuda(), k)
+    caps = torch.tensor([220], dtype=torch.int32, device="cuda")
+    loads, counts, seat_rows, row_entries = c_router.route_by_path(ids, E, caps)
+    P = int(loads.sum())
+    assert int(counts.max()) > 220                      # some entries are dropped
+    _, t1 = _expert_tables(E, d, dff, 4)
+    y = c_router.dispatch_by_rows(x, row_entries, k)
+    want = torch.empty(P, dff, dtype=torch.bfloat16, device="cuda")
+    grouped_linear(y[:P].contiguous(), want, t1, None, loads, d, dff, "gelu")
+    got = torch.empty(P, dff, dtype=torch.bfloat16, device="cuda")
+    grouped_linear(x, got, t1, None, loads, d, dff, "gelu", row_entries=row_entries,
+                   entries_per_cell=k, gather=True, rows=P)
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
 
 
 def test_routed_gemm_argument_checks():
@@ -185,6 +221,13 @@ def test_routed_gemm_argument_checks():
     with pytest.raises(RuntimeError):
         grouped_linear(x[:4], out, table, None, loads, 64, 64, tags=tags, gather=True)  # x not cell-major
     grouped_linear(x, out, table, None, loads, 64, 64, tags=tags, gather=True, scatter=True)
+    entries = torch.arange(1, 17, dtype=torch.int32, device="cuda")        # 8 cells x 2 entries
+    with pytest.raises(NotImplementedError):                              # scatter needs one path per cell
+        grouped_linear(x, out, table, None, loads, 64, 64, row_entries=entries, entries_per_cell=2,
+                       scatter=True, rows=8)
+    two = torch.tensor([16], dtype=torch.int32, device="cuda")
+    wide = torch.zeros(16, 64, dtype=torch.bfloat16, device="cuda")
+    grouped_linear(x, wide, table, None, two, 64, 64, row_entries=entries, entries_per_cell=2, gather=True)
 
 
 def test_full_size_switch_layer_fused_equals_unfused():
