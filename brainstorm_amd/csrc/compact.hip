@@ -168,7 +168,8 @@ __global__ __launch_bounds__(WAVES * kWave) void route_kernel(RouteArgs a) {
   const int hi = min(a.n, lo + a.per_wave);
   // the first batch of ids is fetched once, ahead of everything else, and serves both passes
   const Batch first = load_batch(a.ids, lo, hi, lane);
-  int* unit_rows = a.ws + static_cast<size_t>(gridDim.x) * E;  // behind the workgroup sums
+  // per-unit counters lie behind the workgroup sums (two-launch form only)
+  int* unit_rows = MODE == kWhole ? nullptr : a.ws + static_cast<size_t>(gridDim.x) * E;
   // kEmit: the counters of the first 64 paths are fetched in the same round trip as the ids and
   // the capacities
   int before0 = 0, total0 = 0;
