@@ -977,7 +977,7 @@ __global__ __launch_bounds__(kBlock) void combine_rows_kernel(CombineRowsArgs a)
   for (int rb = 0; rb < np; rb += GROUPS) {
     const int i = rb + gidx;
     const bool live = i < np;
-    const int tag = live ? a.row_tags[p0 + i] : 0;
+    const int tag_loaded = live ? a.row_tags[p0 + i] : 0;
     const size_t from = static_cast<size_t>(p0 + i) * cpr;
     for (int off0 = 0; off0 < cpr; off0 += LPR * UPR) {
       U val[UPR];
@@ -986,6 +986,11 @@ __global__ __launch_bounds__(kBlock) void combine_rows_kernel(CombineRowsArgs a)
         const int off = off0 + u * LPR + glane;
         if (live && off < cpr) val[u] = src[from + off];
       }
+      // The tag is first used here, behind the row loads: left alone, the compiler computes the
+      // destination address ahead of the loop and so waits for the tag before it issues the row
+      // loads -- two memory round trips instead of one.
+      int tag = tag_loaded;
+      asm volatile("" : "+v"(tag) : : "memory");
       if (tag >= 1 && tag <= a.T) {
         const size_t to = static_cast<size_t>(tag - 1) * cpr;
 #pragma unroll
