@@ -113,6 +113,7 @@ struct ScanArgs {
   int T, E, C;
   int capacity_padding, path_wise_padding;
   int ep_shift, rows_pw, bands;
+  int n_ins;  // loads per lane that cover a wavefront's rows: rows_pw / (rows one load covers)
 };
 
 // Sum over the lanes that hold the same path (lanes e, e+ep, e+2ep, ...); every
@@ -146,35 +147,48 @@ __device__ __forceinline__ void walk_batch(const int (&m)[kBatch], int i0, int n
       tot[u] = __shfl(x, (rps - 1) * ep + e, kWave);
     }
   }
+  // rows of this wavefront through one 64-bit base and 32-bit offsets: the address of every
+  // store is one instruction instead of a 64-bit multiply-add chain
+  int* __restrict__ out_w = a.out + row_w * a.E;
+  const int rows_here = static_cast<int>(max(0l, min(static_cast<long>(a.rows_pw), a.T - row_w)));
 #pragma unroll
   for (int u = 0; u < kBatch; ++u) {
     const int run = carry + incl[u];
     carry += tot[u];
-    const long r = row_w + static_cast<long>(i0 + u) * rps + sub;
-    if (i0 + u < n_ins && col_ok && r < a.T) {
+    const int rl = (i0 + u) * rps + sub;  // row within the wavefront's rows
+    if (i0 + u < n_ins && col_ok && rl < rows_here) {
+      const unsigned at = static_cast<unsigned>(rl) * a.E + col;
       if (MODE == kSeat) {
-        a.out[r * a.E + col] = run * m[u];  // location * mask, location.cu:177-178
+        out_w[at] = run * m[u];  // location * mask, location.cu:177-178
       } else if (MODE == kThrottle) {
-        a.out[r * a.E + col] = (m[u] == 1 && run <= thr) ? 1 : 0;
+        out_w[at] = (m[u] == 1 && run <= thr) ? 1 : 0;
       } else {
         const int index = run * m[u];
         if (index >= 1 && index <= a.T)
-          a.out[static_cast<size_t>(index - 1) * a.E + col] = static_cast<int>(r) + 1;
+          a.out[static_cast<size_t>(index - 1) * a.E + col] = static_cast<int>(row_w) + rl + 1;
         // slots past the path's last tag are nobody's to write but this row's owner
-        if (r >= total) a.out[r * a.E + col] = 0;
+        if (row_w + rl >= total) out_w[at] = 0;
       }
     }
   }
 }
 
-// Loads one batch of row words (zero beyond the band / the matrix).
+// Loads one batch of row words (zero beyond the band / the matrix).  One 64-bit base per
+// wavefront and 32-bit offsets; the loads are unconditional (a word outside the wavefront's rows
+// is read from its first row and dropped), so that they issue back to back.
 __device__ __forceinline__ void load_batch(int (&v)[kBatch], int i0, int n_ins, long row_w, int rps,
                                            int sub, int col, bool col_ok, const ScanArgs& a) {
+  const int* __restrict__ mask_w = a.mask + min(row_w, a.T - 1l) * a.E;
+  const int rows_here = static_cast<int>(max(0l, min(static_cast<long>(a.rows_pw), a.T - row_w)));
+  bool ok[kBatch];
 #pragma unroll
   for (int u = 0; u < kBatch; ++u) {
-    const long r = row_w + static_cast<long>(i0 + u) * rps + sub;
-    v[u] = (i0 + u < n_ins && col_ok && r < a.T) ? a.mask[r * a.E + col] : 0;
+    const int rl = (i0 + u) * rps + sub;
+    ok[u] = i0 + u < n_ins && col_ok && rl < rows_here;
+    v[u] = mask_w[ok[u] ? static_cast<unsigned>(rl) * a.E + col : 0u];
   }
+#pragma unroll
+  for (int u = 0; u < kBatch; ++u) v[u] = ok[u] ? v[u] : 0;
 }
 
 // pass 1: column sums of one band
@@ -185,18 +199,14 @@ __global__ __launch_bounds__(kBlock) void band_count_kernel(ScanArgs a) {
   const int ep = 1 << a.ep_shift, rps = kWave >> a.ep_shift;
   const int e = lane & (ep - 1), sub = lane >> a.ep_shift;
   const long row_w = (static_cast<long>(blockIdx.x) * kWavesPB + wave) * a.rows_pw;
-  const int n_ins = a.rows_pw / rps;
+  const int n_ins = a.n_ins;
   for (int c0 = 0; c0 < E; c0 += kWave) {
     const int col = c0 + e;
     const bool col_ok = col < E;
     int sum = 0;
     for (int i0 = 0; i0 < n_ins; i0 += kBatch) {
       int v[kBatch];
-#pragma unroll
-      for (int u = 0; u < kBatch; ++u) {
-        const long r = row_w + static_cast<long>(i0 + u) * rps + sub;
-        v[u] = (i0 + u < n_ins && col_ok && r < a.T) ? a.mask[r * E + col] : 0;
-      }
+      load_batch(v, i0, n_ins, row_w, rps, sub, col, col_ok, a);
 #pragma unroll
       for (int u = 0; u < kBatch; ++u) sum += v[u];
     }
@@ -226,7 +236,7 @@ __global__ __launch_bounds__(kWavesPB * kWave) void band_apply_kernel(ScanArgs a
   const int ep = 1 << a.ep_shift, rps = kWave >> a.ep_shift;
   const int e = lane & (ep - 1), sub = lane >> a.ep_shift;
   const long row_w = (static_cast<long>(band) * kWavesPB + wave) * a.rows_pw;
-  const int n_ins = a.rows_pw / rps;
+  const int n_ins = a.n_ins;
 
   for (int c0 = 0; c0 < E; c0 += kWave) {
     const int col = c0 + e;
@@ -237,25 +247,31 @@ __global__ __launch_bounds__(kWavesPB * kWave) void band_apply_kernel(ScanArgs a
     // ---- this wave's share of the offset: bands wave, wave+4, ... above this one ----
     int above = 0, below = 0;
     for (int j0 = wave + sub * kWavesPB; j0 < band; j0 += kWavesPB * rps * kPartialBatch) {
+      // unconditional loads through 32-bit offsets (an entry that does not count is read from
+      // the head of the table and dropped), so that they issue back to back
       int v[kPartialBatch];
+      bool ok[kPartialBatch];
 #pragma unroll
       for (int u = 0; u < kPartialBatch; ++u) {
         const int j = j0 + u * kWavesPB * rps;
-        v[u] = (j < band && col_ok) ? a.partial[static_cast<size_t>(j) * E + col] : 0;
+        ok[u] = j < band && col_ok;
+        v[u] = a.partial[ok[u] ? static_cast<unsigned>(j) * E + col : 0u];
       }
 #pragma unroll
-      for (int u = 0; u < kPartialBatch; ++u) above += v[u];
+      for (int u = 0; u < kPartialBatch; ++u) above += ok[u] ? v[u] : 0;
     }
     if (MODE == kTag) {  // the tag list of a path ends at its total: the later bands count too
       for (int j0 = band + 1 + wave + sub * kWavesPB; j0 < a.bands; j0 += kWavesPB * rps * kPartialBatch) {
         int v[kPartialBatch];
+        bool ok[kPartialBatch];
 #pragma unroll
         for (int u = 0; u < kPartialBatch; ++u) {
           const int j = j0 + u * kWavesPB * rps;
-          v[u] = (j < a.bands && col_ok) ? a.partial[static_cast<size_t>(j) * E + col] : 0;
+          ok[u] = j < a.bands && col_ok;
+          v[u] = a.partial[ok[u] ? static_cast<unsigned>(j) * E + col : 0u];
         }
 #pragma unroll
-        for (int u = 0; u < kPartialBatch; ++u) below += v[u];
+        for (int u = 0; u < kPartialBatch; ++u) below += ok[u] ? v[u] : 0;
       }
       below = sum_over_rows_in_wave(below, a.ep_shift);
     }
@@ -372,6 +388,7 @@ int launch_scan(int mode, ScanArgs& a, void* workspace, size_t workspace_bytes, 
   a.prefix_in = a.partial + static_cast<size_t>(g.bands) * a.E;
   a.ep_shift = g.ep_shift;
   a.rows_pw = g.rows_pw;
+  a.n_ins = g.rows_pw >> (6 - g.ep_shift);
   a.bands = g.bands;
   const dim3 grid(g.bands);
   hipStream_t st = as_stream(stream);
