@@ -750,29 +750,26 @@ __global__ __launch_bounds__(kBlock, 8) void dispatch_lean_kernel(DispatchArgs a
   // choice is a compile-time property of the shape: chosen by a branch at run time, the compiler
   // merges the two stores into an ordinary one.
   constexpr bool kStream = LS >= 4;
-  // In seat mode the source row of a token is the token itself, so its units are
-  // fetched before the index words have even arrived and are reused for every
-  // path the token is routed to (a top-k token is read once and stored k times).
-  // The loads are unconditional (row and unit clamped into the tensor, the value unused where
-  // the lane has nothing to move): a load under a condition of its own becomes a branch, and
-  // the loads of consecutive branches wait for each other.
-  auto load_units = [&](int i, int tokens, int step, int off0, U (&val)[UPR]) {
-    const size_t from = static_cast<size_t>(min(r0 + step * rps + min(i, tokens - 1), a.T - 1l)) * cpr;
-#pragma unroll
-    for (int u = 0; u < UPR; ++u) val[u] = src[from + min(off0 + u * LPR + glane, cpr - 1)];
-  };
-
-  // Everything the first step needs is requested before anything is waited for: index words,
-  // the rows themselves, counts, and the loads whose prefix sums give the destination rows.
   int v_next = (n_steps > 0 && sub < nr && e < E) ? idx0[sub * E + e] : 0;
-  U val[UPR];
-  if (n_steps > 0) load_units(gidx, min(rps, nr), 0, 0, val);
   const int my_count = (a.counts != nullptr && lane < E) ? a.counts[lane] : 0;
   const SmallTables tab = small_tables(a.loads, E, a.mpl, ep_shift, lane);
 
+// In seat mode the source row of a token is the token itself, so its units are
+  // fetched before the index words have even arrived and are reused for every
+  // path the token is routed to (a top-k token is read once and stored k times).
+  auto load_units = [&](int i, int tokens, int step, int off0, U (&val)[UPR]) {
+    const size_t from = static_cast<size_t>(r0 + step * rps + i) * cpr;
+#pragma unroll
+    for (int u = 0; u < UPR; ++u) {
+      const int off = off0 + u * LPR + glane;
+      if (i < tokens && off < cpr) val[u] = src[from + off];
+    }
+  };
+
   for (int step = 0; step < n_steps; ++step) {
     const int tokens = min(rps, nr - step * rps);
-    if (step > 0) load_units(gidx, tokens, step, 0, val);
+    U val[UPR];
+    load_units(gidx, tokens, step, 0, val);
     const int v = v_next;
     const int row = step * rps + sub;
     {
