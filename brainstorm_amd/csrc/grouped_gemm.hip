@@ -121,6 +121,7 @@ __global__ __launch_bounds__(WAVES * 64) void grouped_gemm_kernel(GemmArgs a) {
   constexpr int OUT_ROW = BN * 2 + 16;
   extern __shared__ __attribute__((aligned(16))) char smem[];
   __shared__ int s_tile[4];  // expert, first row, valid rows, first row counted inside the expert
+  __shared__ int s_cell[BM];  // routed forms: 0-based cell behind each row of the tile, -1 = empty slot
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -185,18 +186,26 @@ __global__ __launch_bounds__(WAVES * 64) void grouped_gemm_kernel(GemmArgs a) {
   // operand load); an empty tag addresses past the extent and so reads a row of zeros, which
   // is what dispatch writes for a padding row.
   const bool gather = a.gather != 0;
-  // 0-based cell behind row r of this tile, -1 for an empty slot: from the tag matrix (seat
-  // seat0 + r of column e), or from the row-entry vector of the compact route (entry t*k+j+1 of
-  // row row0 + r of the dispatched layout)
-  auto cell_of_row = [&](int r) {
-    if (a.tag_vector) {
-      const int entry = a.tags[static_cast<size_t>(row0) + r];
-      const int cell = a.tag_div > 1 ? (entry - 1) / a.tag_div : entry - 1;
-      return (entry >= 1 && cell < a.T) ? cell : -1;
+  // Routed forms: the 0-based cell behind every row of this tile (-1 for an empty slot), from
+  // the tag matrix (seat seat0 + r of column e) or from the row-entry vector of the compact route
+  // (entry t*k+j+1 of row row0 + r of the dispatched layout).  One load per row, all of them in
+  // one memory round trip, kept in LDS for the operand offsets below and for the store loop of
+  // the epilogue.
+  if (a.tags != nullptr) {
+    for (int r = tid; r < rows; r += THREADS) {
+      int cell;
+      if (a.tag_vector) {
+        const int entry = a.tags[static_cast<size_t>(row0) + r];
+        cell = a.tag_div > 1 ? (entry - 1) / a.tag_div : entry - 1;
+        cell = (entry >= 1 && cell < a.T) ? cell : -1;
+      } else {
+        const int tag = a.tags[static_cast<size_t>(seat0 + r) * a.E + e];
+        cell = (tag >= 1 && tag <= a.T) ? tag - 1 : -1;
+      }
+      s_cell[r] = cell;
     }
-    const int tag = a.tags[static_cast<size_t>(seat0 + r) * a.E + e];
-    return (tag >= 1 && tag <= a.T) ? tag - 1 : -1;
-  };
+    __syncthreads();
+  }
   const char* xa = reinterpret_cast<const char*>(gather ? a.x : a.x + static_cast<size_t>(row0) * K);
   const __bf16* const w_e = a.w[e];
   const size_t xa_bytes = static_cast<size_t>(gather ? a.T : a.P - row0) * K * 2;
@@ -220,7 +229,7 @@ __global__ __launch_bounds__(WAVES * 64) void grouped_gemm_kernel(GemmArgs a) {
     const int r = lr + i * ROWS_PER_PASS;
     const bool in_tile = r < rows;
     if (gather) {
-      const int cell = in_tile ? cell_of_row(r) : -1;
+      const int cell = in_tile ? s_cell[r] : -1;
       off_a[i] = cell >= 0 ? (static_cast<uint32_t>(cell) * K + lc * 8) * 2 : 0x80000000u;
     } else {
       off_a[i] = in_tile ? (static_cast<uint32_t>(r) * K + lc * 8) * 2 : 0x80000000u;
@@ -456,7 +465,7 @@ __global__ __launch_bounds__(WAVES * 64) void grouped_gemm_kernel(GemmArgs a) {
         const int rl = q / OUT_CHUNKS, c = q - rl * OUT_CHUNKS;
         const int r = r_lo + rl;
         long to = r;
-        if (a.scatter) to = cell_of_row(r);
+        if (a.scatter) to = s_cell[r];
         // streaming stores: the output is not read again by this kernel, and written through the
         // L2 like ordinary stores it pushes the operand lines out that the column tiles share
         if (to >= 0 && n0 + c * 8 < a.N)
