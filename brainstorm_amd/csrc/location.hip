@@ -62,7 +62,7 @@ int env_int(const char* name, int fallback) {
   return v ? atoi(v) : fallback;
 }
 
-ScanGeometry scan_geometry(int T, int E) {
+ScanGeometry scan_geometry(int T, int E, bool tag_mode) {
   ScanGeometry g;
   int shift = 0;
   while ((1 << shift) < std::min(E, kWave)) ++shift;
@@ -70,11 +70,21 @@ ScanGeometry scan_geometry(int T, int E) {
   g.waves_pb = kWavesPB;
   const int rps = kWave >> shift;  // rows per load instruction
   static const int forced_bands = env_int("BRT_SCAN_BANDS", 0);  // tuning knob, read once
-  // Small masks (decode-sized batches): when every wavefront of one 8-wavefront workgroup can
-  // hold its rows in one batch of loads, that workgroup does both passes in one launch (the
-  // column sums meet in LDS): 5.5 us instead of 8.6 us for two launches.  Larger masks are
-  // faster spread over many CUs, launch cost and all.
-  if (forced_bands <= 0 && E <= kWave &&
+  // Small masks (decode-sized batches) take one launch of one workgroup, the column sums of its
+  // wavefronts meeting in LDS.  Up to four loads per lane of a 4-wavefront workgroup that is
+  // the ordinary kernel with a single band (16 x 8: 4.1 us, 128 x 8: 4.7 us); up to one batch of
+  // loads per lane of an 8-wavefront workgroup it is the 512-thread form (128 x 64: 4.7 us,
+  // 512 x 16: 6.8 us, against 6.9-7.3 us for two launches).  Tag indices scatter their stores
+  // over the whole matrix, which one CU does slowly: beyond 128 rows they take the two launches
+  // (512 x 16: 8.9 us against 10.6 us).  Larger masks are faster spread over many CUs, launch
+  // cost and all.
+  if (forced_bands <= 0 && E <= kWave && static_cast<long>(T) <= 4l * kWavesPB * rps) {
+    long rows_pw = (static_cast<long>(T) + kWavesPB - 1) / kWavesPB;
+    g.rows_pw = static_cast<int>(std::max<long>((rows_pw + rps - 1) / rps * rps, rps));
+    g.bands = 1;
+    return g;
+  }
+  if (forced_bands <= 0 && E <= kWave && (!tag_mode || T <= 128) &&
       static_cast<long>(T) <= static_cast<long>(kWavesSingle) * kBatch * rps) {
     long rows_pw = (static_cast<long>(T) + kWavesSingle - 1) / kWavesSingle;
     rows_pw = std::max<long>((rows_pw + rps - 1) / rps * rps, rps);
@@ -378,7 +388,7 @@ __global__ __launch_bounds__(256) void tag_to_seat_kernel(const int* __restrict_
 }
 
 int launch_scan(int mode, ScanArgs& a, void* workspace, size_t workspace_bytes, void* stream) {
-  const ScanGeometry g = scan_geometry(a.T, a.E);
+  const ScanGeometry g = scan_geometry(a.T, a.E, mode == kTag);
   const size_t need = brt_hip_scan_workspace_bytes(a.T, a.E);
   if (workspace == nullptr || workspace_bytes < need)
     return fail(BRT_E_WORKSPACE, "scan workspace too small: %zu < %zu bytes", workspace_bytes,
@@ -420,8 +430,9 @@ using namespace brt;
 
 extern "C" size_t brt_hip_scan_workspace_bytes(int T, int E) {
   if (T <= 0 || E <= 0) return 0;
-  const ScanGeometry g = scan_geometry(T, E);
-  return (static_cast<size_t>(g.bands) + 1) * E * sizeof(int);
+  // enough for either index format (tag indices leave the one-workgroup form earlier)
+  const int bands = std::max(scan_geometry(T, E, false).bands, scan_geometry(T, E, true).bands);
+  return (static_cast<size_t>(bands) + 1) * E * sizeof(int);
 }
 
 extern "C" int brt_hip_generate_indices_and_loads(const int32_t* mask, int32_t* indices,
