@@ -316,8 +316,15 @@ __global__ __launch_bounds__(kBlock) void dispatch_by_rows_kernel(RowsArgs a) {
           if (a.weights != nullptr && filled) {
             float x[NE];
             unpack<DT, 16>(val[u], x);
+            // The product is an fp32 product, then rounded to the data type.  The empty asm keeps
+            // it one: multiply and conversion to fp16 would otherwise be merged into a
+            // mixed-precision instruction that rounds the exact product once, which differs from
+            // the fp32 product in the last bit now and then (and has no bf16 counterpart).
 #pragma unroll
-            for (int q = 0; q < NE; ++q) x[q] = x[q] * g;
+            for (int q = 0; q < NE; ++q) {
+              x[q] = x[q] * g;
+              asm volatile("" : "+v"(x[q]));
+            }
             pack_store<DT, NE, kStream>(dst + to + off, x);
           } else {
             store_unit<kStream>(dst + to + off, val[u]);

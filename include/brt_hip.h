@@ -297,7 +297,8 @@ int brt_hip_combine_by_index(const void* in_data, void* out_data, const void* in
  *   not shared between calls that run at the same time).
  *
  * brt_hip_dispatch_by_rows: dst[r] = src[(row_entries[r]-1) / k] (times weights[row_entries[r]-1]
- *   when weights != NULL, rounded once to the data type), zero rows where row_entries[r] == 0.
+ *   when weights != NULL: an fp32 product, then rounded to the data type), zero rows where
+ *   row_entries[r] == 0.
  *   dst [P,cell] is written whole.  Rows must be whole 16-byte units.
  *
  * brt_hip_combine_by_rows: dst[t] = sum over the entries j of cell t with seat_rows[t,j] != 0,

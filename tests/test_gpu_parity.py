@@ -681,3 +681,36 @@ def test_compact_route_empty_and_tiny_inputs(hip):
     out = hip.combine_by_rows(np.zeros((0, 8), dtype=np.float32), np.zeros((3, 1), dtype=np.int32),
                               np.zeros((3, 1), dtype=np.int32), out_bits=x)
     assert np.array_equal(out, x)                              # nothing routed: the residual stays
+
+
+def test_compact_route_random_shapes(hip):
+    """Seeded random shapes: odd path counts, up to 8 entries per cell, holes, every capacity mode,
+    rows of odd numbers of 16-byte units; route, dispatch and combine against the oracle."""
+    rng = np.random.default_rng(2024)
+    for case in range(40):
+        T = int(rng.integers(1, 3000))
+        E = int(rng.integers(1, 200))
+        k = int(rng.integers(1, min(E, 8) + 1))
+        dtype = ("f32", "f16", "bf16")[case % 3]
+        cell = int(rng.integers(1, 40)) * (4 if dtype == "f32" else 8)
+        ids = _compact_route(T, E, k, seed=case, hole=float(rng.choice([0.0, 0.1, 0.5])))
+        mode = case % 4
+        cap = max(1, (T * k) // max(1, 2 * E))
+        caps = [None, [cap], [cap, 3 * cap, T * k], [cap, 3 * cap, T * k]][mode]
+        pad = mode >= 2
+        loads0 = oracle.route_by_path(ids, E, caps, pad)[0]
+        mpl = int(loads0.max()) if mode == 3 else 0
+        P = max(1, E * mpl if mpl else int(loads0.sum()) + int(rng.integers(0, 4)))
+        want = oracle.route_by_path(ids, E, caps, pad, False, mpl, P)
+        got = hip.route_by_path(ids, E, caps, pad, False, mpl, P)
+        for g, w, name in zip(got, want, ("loads", "counts", "seat_rows", "row_entries")):
+            assert np.array_equal(g, w), (case, T, E, k, mode, name)
+        _, _, seat_rows, row_entries = want
+        weights = rng.random((T, k)).astype(np.float32) if case % 2 else None
+        x = as_dtype_bits(rng.standard_normal((T, cell)).astype(np.float32), dtype)
+        assert np.array_equal(hip.dispatch_by_rows(x, row_entries, k, weights, dtype),
+                              oracle.dispatch_by_rows(x, row_entries, k, weights, dtype)), (case, "dispatch")
+        y = as_dtype_bits(rng.standard_normal((P, cell)).astype(np.float32), dtype)
+        res = as_dtype_bits(rng.standard_normal((T, cell)).astype(np.float32), dtype) if case % 3 == 0 else None
+        assert np.array_equal(hip.combine_by_rows(y, ids, seat_rows, weights, res, dtype),
+                              oracle.combine_by_rows(y, ids, seat_rows, weights, res, dtype)), (case, "combine")
