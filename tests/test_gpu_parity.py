@@ -714,3 +714,46 @@ def test_compact_route_random_shapes(hip):
         res = as_dtype_bits(rng.standard_normal((T, cell)).astype(np.float32), dtype) if case % 3 == 0 else None
         assert np.array_equal(hip.combine_by_rows(y, ids, seat_rows, weights, res, dtype),
                               oracle.combine_by_rows(y, ids, seat_rows, weights, res, dtype)), (case, "combine")
+
+
+def test_dense_route_random_shapes(hip):
+    """Seeded random shapes for the dense ops: odd path counts, any row length, every capacity
+    mode and dtype pairing (gates in another type than the data in combine); index generation,
+    dispatch and combine against the oracle."""
+    rng = np.random.default_rng(77)
+    for case in range(40):
+        T = int(rng.integers(1, 2500))
+        E = int(rng.integers(1, 150))
+        k = int(rng.integers(1, min(E, 4) + 1))
+        dtype = ("f32", "f16", "bf16")[case % 3]
+        cell = int(rng.integers(1, 300))
+        mask, logits = topk_mask(T, E, k, seed=1000 + case)
+        mode = case % 4
+        cap = max(1, (T * k) // max(1, 2 * E))
+        caps = [None, [cap], [cap, 3 * cap, T * k], [cap, 3 * cap, T * k]][mode]
+        pad = mode >= 2
+        tag = case % 5 == 0
+        want_idx, loads = oracle.generate_indices_and_loads(mask, caps, pad, is_tag_index=tag)
+        got_idx, got_loads = hip.generate_indices_and_loads(mask, caps, pad, is_tag_index=tag)
+        assert np.array_equal(got_idx, want_idx) and np.array_equal(got_loads, loads), (case, "indices")
+        if tag:
+            continue
+        idx = want_idx
+        mpl = int(loads.max()) if mode == 3 else 0
+        x = as_dtype_bits(rng.standard_normal((T, cell)), dtype)
+        gates = as_dtype_bits(softmax(logits), dtype) if case % 2 else None
+        want, want_tags = oracle.dispatch(x, idx, loads, gates=gates, tag_generating=True,
+                                          max_path_padding=mpl != 0, max_path_load=mpl, dtype=dtype)
+        got, got_tags = hip.dispatch(x, idx, loads, gates, None, True, max_path_load=mpl, dtype=dtype)
+        assert same_bits(got, want) and np.array_equal(got_tags, want_tags), (case, "dispatch")
+        P = want.shape[0]
+        out_dtype = "f32" if case % 4 == 1 else dtype
+        gate_dtype = ("f32", dtype)[case % 2]
+        y = as_dtype_bits(rng.standard_normal((P, cell)), dtype)
+        cg = as_dtype_bits(softmax(logits), gate_dtype) if case % 3 else None
+        res = as_dtype_bits(rng.standard_normal((T, cell)), out_dtype) if case % 2 == 0 else None
+        want = oracle.combine(y, idx, loads, gates=cg, out_data=res, max_path_padding=mpl != 0,
+                              in_dtype=dtype, out_dtype=out_dtype, gate_dtype=gate_dtype)
+        got = hip.combine(y, idx, loads, cg, res, max_path_load=mpl, in_dtype=dtype, out_dtype=out_dtype,
+                          gate_dtype=gate_dtype)
+        assert same_bits(got, want), (case, "combine", dtype, out_dtype, gate_dtype)
