@@ -328,3 +328,18 @@ def test_workgroups_walking_several_column_tiles(K, N):
     loads = [160] * 64
     loads[5], loads[17], loads[40] = 0, 3, 97
     run(loads, K, N, act="none", bias=False, seed=K, slack=100)
+
+
+def test_grouped_gemm_random_shapes():
+    """Seeded random expert counts, ragged loads (many empty), K and N that are any multiple of
+    8, bias and activation at random, slack rows behind the loads."""
+    rng = np.random.default_rng(31)
+    for case in range(16):
+        E = int(rng.integers(1, 90))
+        loads = [int(v) for v in rng.integers(0, 400, E) * (rng.random(E) < 0.6)]
+        if sum(loads) == 0:
+            loads[0] = 5
+        K = int(rng.integers(1, 100)) * 8
+        N = int(rng.integers(1, 120)) * 8
+        run(loads, K, N, act=("none", "gelu", "relu")[case % 3], bias=bool(case % 2), seed=case,
+            slack=int(rng.integers(0, 9)))
