@@ -757,3 +757,28 @@ def test_dense_route_random_shapes(hip):
         got = hip.combine(y, idx, loads, cg, res, max_path_load=mpl, in_dtype=dtype, out_dtype=out_dtype,
                           gate_dtype=gate_dtype)
         assert same_bits(got, want), (case, "combine", dtype, out_dtype, gate_dtype)
+
+
+def test_tag_gather_random_shapes(hip):
+    """Seeded random tag sets (dense and sparse in their range, negative values, both widths) and
+    random row sums (skewed indices: rows with long contributor lists, rows with none)."""
+    rng = np.random.default_rng(5)
+    for case in range(30):
+        n = int(rng.integers(1, 40000))
+        lo = int(rng.integers(-1000, 1000))
+        span = int(rng.integers(1, 8 * n + 10))
+        kind = (np.int32, np.int64)[case % 2]
+        tags = rng.integers(lo, lo + span, size=n).astype(kind)
+        unique, inverse = hip.unique_tags(tags)
+        want_u, want_i = oracle.unique_tags(tags)
+        assert np.array_equal(unique, want_u) and np.array_equal(inverse, want_i), (case, "unique")
+        P = int(rng.integers(1, 5000))
+        n_out = int(rng.integers(1, 3000))
+        dtype = ("f32", "f16", "bf16")[case % 3]
+        cell = int(rng.integers(1, 100))
+        out_dtype = "f32" if case % 4 == 3 else dtype
+        bits = as_dtype_bits(rng.standard_normal((P, cell)).astype(np.float32), dtype)
+        index = np.minimum(rng.geometric(min(1.0, 8.0 / n_out), size=P) - 1, n_out + 1).astype(kind)
+        got = hip.combine_by_index(bits, index, n_out, dtype, out_dtype)
+        want = oracle.combine_by_index(bits, index, n_out, dtype, out_dtype)
+        assert same_bits(got, want), (case, "sum", P, n_out, cell, dtype, out_dtype)
