@@ -107,7 +107,7 @@ struct Staged {
   u32x4 v[N];
 };
 
-template <int MT, int NT, int WAVES, int ACT, bool WALKS>
+template <int MT, int NT, int WAVES, int ACT, bool WALKS, bool WSTREAM>
 __global__ __launch_bounds__(WAVES * 64) void grouped_gemm_kernel(GemmArgs a) {
   constexpr int THREADS = WAVES * 64;
   constexpr int BM = MT * 32, WN = NT * 32, BN = WAVES * WN;
@@ -261,7 +261,7 @@ __global__ __launch_bounds__(WAVES * 64) void grouped_gemm_kernel(GemmArgs a) {
           s.v[i] = __builtin_amdgcn_raw_buffer_load_b128(res_a, off_a[i < A_LOADS ? i : 0], k0 * 2, 0);
       } else {
         s.v[i] = __builtin_amdgcn_raw_buffer_load_b128(res_b, off_b[i >= A_LOADS ? i - A_LOADS : 0],
-                                                       k0 * 2, kStreamingLoad);
+                                                       k0 * 2, WSTREAM ? kStreamingLoad : 0);
       }
     }
   };
@@ -527,22 +527,37 @@ int launch_act(GemmArgs& a, hipStream_t st) {
   }
   if (forced_walk > 0) a.walk = std::min(forced_walk, a.tiles_n);
   a.groups_n = (a.tiles_n + a.walk - 1) / a.walk;
-  const long grid = static_cast<long>(a.tiles_m_max) * a.groups_n;
+  // Weight loads are streamed (non-temporal) when a weight tile is read about once per launch:
+  // experts of at most one row block on average.  Experts with many row blocks read their
+  // weights once per row block, and those re-reads are served by the caches only if the first
+  // read left the lines there.
+  const bool stream_weights = static_cast<long>(a.P) <= static_cast<long>(a.E) * BM;
+  // only the 4-wavefront tiles have the registers to walk column tiles
+  constexpr bool kCanWalk = WAVES == 4;
+  if (!kCanWalk) a.walk = 1, a.groups_n = a.tiles_n;
+  const long grid_wgs = static_cast<long>(a.tiles_m_max) * a.groups_n;
+  const dim3 blocks(static_cast<unsigned>(grid_wgs)), threads(WAVES * 64);
   // more than 64 KB of dynamic LDS has to be allowed once per device and kernel
-  static bool configured[64] = {};
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 63;
-  if (!configured[dev] || dev == 63) {
-    for (const void* fn : {reinterpret_cast<const void*>(&grouped_gemm_kernel<MT, NT, WAVES, ACT, false>),
-                           reinterpret_cast<const void*>(&grouped_gemm_kernel<MT, NT, WAVES, ACT, true>)})
-      if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)) != hipSuccess)
+  auto run = [&](auto walks, auto wstream) -> int {
+    auto* fn = &grouped_gemm_kernel<MT, NT, WAVES, ACT, decltype(walks)::value, decltype(wstream)::value>;
+    static bool configured[64] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 63;
+    if (!configured[dev] || dev == 63) {
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize,
+                              static_cast<int>(lds)) != hipSuccess)
         return fail(BRT_E_LAUNCH, "cannot reserve %zu bytes of LDS", lds);
-    configured[dev] = true;
+      configured[dev] = true;
+    }
+    hipLaunchKernelGGL(fn, blocks, threads, lds, st, a);
+    return check_launch("grouped_gemm_kernel");
+  };
+  using Yes = std::integral_constant<bool, true>;
+  using No = std::integral_constant<bool, false>;
+  if constexpr (kCanWalk) {
+    if (a.walk > 1) return stream_weights ? run(Yes{}, Yes{}) : run(Yes{}, No{});
   }
-  const dim3 blocks(static_cast<unsigned>(grid)), threads(WAVES * 64);
-  if (a.walk > 1) hipLaunchKernelGGL((grouped_gemm_kernel<MT, NT, WAVES, ACT, true>), blocks, threads, lds, st, a);
-  else hipLaunchKernelGGL((grouped_gemm_kernel<MT, NT, WAVES, ACT, false>), blocks, threads, lds, st, a);
-  return check_launch("grouped_gemm_kernel");
+  return stream_weights ? run(No{}, Yes{}) : run(No{}, No{});
 }
 
 template <int MT, int NT, int WAVES>
