@@ -1051,11 +1051,11 @@ StepMap make_step_map(int E) {
 // Rows of the index matrix per wavefront: enough units that each lane has a
 // handful of 16-byte accesses in flight, few enough index words that one batch
 // of kSteps loads covers them.
-int rows_per_wave(int forced_rows, int cpr, int E, long T) {
+int rows_per_wave(int forced_rows, int cpr, int E, long T, long min_waves = 4096) {
   int rows = forced_rows;
   if (rows <= 0) {
     rows = std::max(1, 384 / std::max(cpr, 1));
-    while (rows > 1 && (T + rows - 1) / rows < 4096) rows >>= 1;  // keep every SIMD busy
+    while (rows > 1 && (T + rows - 1) / rows < min_waves) rows >>= 1;  // keep every SIMD busy
   }
   const StepMap m = make_step_map(E);
   if (E <= kWave) {  // register path: whole steps of 64 >> ep_shift rows
@@ -1225,7 +1225,9 @@ extern "C" int brt_hip_combine(const void* src, void* dst, const void* gates,
   a.cpr = static_cast<int>(row_bytes / bytes);
   a.is_residual = is_residual; a.gate_dtype = gate_dtype;
   a.map = make_step_map(E);
-  a.rows_pw = rows_per_wave(knobs().combine_rows, a.cpr, E, T);
+  // a gather makes two dependent memory round trips per cell: twice the wavefronts of dispatch
+  // to hide them (5.8 -> 5.6 us at 8192 x 768 bf16, 8.5 -> 8.3 us at 100352 x 96 fp16)
+  a.rows_pw = rows_per_wave(knobs().combine_rows, a.cpr, E, T, 8192);
   a.lds_pw = 2 * E + a.rows_pw + 2 * a.rows_pw * E;
   LaunchShape sh;
   if (!launch_shape(T, a.rows_pw, a.lds_pw, &sh))
