@@ -115,6 +115,8 @@ __global__ void inverse_kernel(const K* __restrict__ keys, long n, long lo, long
 constexpr int kSmallRange = 32768;
 constexpr long kSmallCount = 1l << 15;
 
+constexpr int kKeysInFlight = 8;
+
 template <typename K>
 __global__ __launch_bounds__(kScanThreads) void unique_small_kernel(const K* __restrict__ keys, int n,
                                                                     long lo, int range,
@@ -124,11 +126,31 @@ __global__ __launch_bounds__(kScanThreads) void unique_small_kernel(const K* __r
   extern __shared__ int s_table[];
   __shared__ int s_wave[kScanThreads / kWave];
   const int tid = threadIdx.x, wave = tid >> 6;
+  // The keys are fetched in batches of kKeysInFlight loads per thread (unconditional: an index
+  // past the end reads the last key again and is dropped), all in flight together; one at a
+  // time, every key would be a memory round trip of its own for this one workgroup.  The first
+  // batch stays in registers for the inverse at the end.
+  auto key_batch = [&](int base, K (&v)[kKeysInFlight]) {
+#pragma unroll
+    for (int j = 0; j < kKeysInFlight; ++j) v[j] = keys[min(base + j * kScanThreads + tid, n - 1)];  // n >= 1
+  };
+  K held[kKeysInFlight];
+  key_batch(0, held);
   for (int i = tid; i < range; i += kScanThreads) s_table[i] = 0;
   __syncthreads();
-  for (int i = tid; i < n; i += kScanThreads) {
-    const long k = static_cast<long>(keys[i]) - lo;
-    if (k >= 0 && k < range) s_table[k] = 1;
+  for (int base = 0; base < n; base += kKeysInFlight * kScanThreads) {
+    K v[kKeysInFlight];
+    if (base == 0) {
+#pragma unroll
+      for (int j = 0; j < kKeysInFlight; ++j) v[j] = held[j];
+    } else {
+      key_batch(base, v);
+    }
+#pragma unroll
+    for (int j = 0; j < kKeysInFlight; ++j) {
+      const long k = static_cast<long>(v[j]) - lo;
+      if (base + j * kScanThreads + tid < n && k >= 0 && k < range) s_table[k] = 1;
+    }
   }
   __syncthreads();
   // every thread scans a run of consecutive entries; an odd run length keeps the lanes of a
@@ -150,9 +172,20 @@ __global__ __launch_bounds__(kScanThreads) void unique_small_kernel(const K* __r
   }
   if (tid == kScanThreads - 1) *n_unique = rank;
   __syncthreads();
-  for (int i = tid; i < n; i += kScanThreads) {
-    const long k = static_cast<long>(keys[i]) - lo;
-    inverse[i] = (k >= 0 && k < range) ? s_table[k] : -1;
+  for (int base = 0; base < n; base += kKeysInFlight * kScanThreads) {
+    K v[kKeysInFlight];
+    if (base == 0) {
+#pragma unroll
+      for (int j = 0; j < kKeysInFlight; ++j) v[j] = held[j];
+    } else {
+      key_batch(base, v);
+    }
+#pragma unroll
+    for (int j = 0; j < kKeysInFlight; ++j) {
+      const int i = base + j * kScanThreads + tid;
+      const long k = static_cast<long>(v[j]) - lo;
+      if (i < n) inverse[i] = (k >= 0 && k < range) ? s_table[k] : -1;
+    }
   }
 }
 
@@ -314,7 +347,7 @@ extern "C" int brt_hip_unique_tags(const void* tags, int tag_bits, long n, long 
   const size_t need = brt_hip_unique_tags_workspace_bytes(lo, hi);
   if (workspace_bytes < need || !aligned(workspace, 4))
     return fail(BRT_E_INVALID, "workspace of %zu bytes, need %zu", workspace_bytes, need);
-  if (range <= kSmallRange && n <= kSmallCount) {
+  if (range <= kSmallRange && n >= 1 && n <= kSmallCount) {  // (no keys: the general path below)
     const size_t lds = static_cast<size_t>(range) * sizeof(int);
     // more than 64 KB of dynamic LDS has to be allowed once per device and kernel
     static bool configured[2][64] = {};
