@@ -37,13 +37,13 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 
 # Bytes per launch seen by the memory side for this workload: rocprofv3 --pmc
 # FETCH_SIZE and WRITE_SIZE (KiB), each scaled by what the same counter reads for
-# a 12 MiB device-to-device copy (fetch x1.995, write x1.000).
+# a 12 MiB device-to-device copy (fetch x1.996, write x1.000).
 MEASURED_TRAFFIC_BYTES = {
-    "dispatch": int((7207.5 * 1.995 + 12466.3) * 1024),
-    "combine": int((6221.5 * 1.995 + 12288.1) * 1024),
-    "combine_gather": int((7197.0 * 1.995 + 12288.0) * 1024),
-    "ffn_gemm1_gelu": int((154299.4 * 1.995 + 49152.6) * 1024),
-    "ffn_gemm2": int((172251.8 * 1.995 + 12288.0) * 1024),
+    "dispatch": int((7197.5 * 1.996 + 12459.4) * 1024),
+    "combine": int((6221.5 * 1.996 + 12288.0) * 1024),
+    "combine_gather": int((7196.0 * 1.996 + 12288.2) * 1024),
+    "ffn_gemm1_gelu": int((155947.1 * 1.996 + 49152.0) * 1024),
+    "ffn_gemm2": int((172184.1 * 1.996 + 12288.0) * 1024),
 }
 
 T, D, E, DFF = 8192, 768, 64, 3072
