@@ -40,3 +40,39 @@ def test_argument_errors_do_not_need_a_gpu():
     assert handle.brt_hip_combine(None, None, None, None, None, 4, 4, 4, 4, 0, 0, 7, 7, 0, None) == -4
     assert handle.brt_hip_generate_indices_and_loads(
         None, None, None, None, 4, 4, None, 0, 1, 0, 0, None, 0, None) == -1
+
+
+def test_ops_refuse_host_tensors_instead_of_falling_back():
+    """Every routing op needs device tensors; on host tensors it raises, it computes nothing."""
+    import pytest
+    import torch
+    from brainstorm_amd._C import router as ops
+
+    mask = torch.ones(8, 4, dtype=torch.int32)
+    rows = torch.ones(8, 16)
+    score = torch.rand(8, 4)
+    ids = torch.zeros(8, 1, dtype=torch.int32)
+    calls = [
+        lambda: ops.generate_indices_and_loads(mask),
+        lambda: ops.throttle_hotmask(mask, torch.zeros(4, dtype=torch.int32),
+                                     torch.full((4,), 2, dtype=torch.int32)),
+        lambda: ops.convert_index_format(mask, torch.full((4,), 8, dtype=torch.int32), False),
+        lambda: ops.dispatch_with_indices_and_loads(rows, mask, torch.full((4,), 8, dtype=torch.int32)),
+        lambda: ops.combine_with_indices_and_loads(rows, mask, torch.full((4,), 2, dtype=torch.int32)),
+        lambda: ops.gate_topk(score, 1),
+        lambda: ops.route_by_path(ids, 4),
+        lambda: ops.dispatch_by_rows(rows, torch.arange(1, 9, dtype=torch.int32), 1),
+        lambda: ops.combine_by_rows(rows, ids, torch.ones(8, 1, dtype=torch.int32)),
+    ]
+    for call in calls:
+        with pytest.raises(RuntimeError, match="must be a CUDA tensor"):
+            call()
+
+
+def test_missing_library_is_an_error(monkeypatch, tmp_path):
+    import pytest
+
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libbrt_hip.so"))
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        _lib.lib()
