@@ -441,3 +441,44 @@ def test_compact_route_ops_equal_the_routers(brt_mod, top_k, dtype):
         c_router.route_by_path(ids.long(), E)
     with pytest.raises(RuntimeError):
         c_router.dispatch_by_rows(x, row_entries, top_k, weights=weights.half())
+
+
+def test_row_buffers_beyond_two_gib(brt_mod):
+    """Row offsets are 64-bit: 1.2 M rows of 2 KiB (2.3 GiB in, 2.3 GiB out) go through both route
+    formats; no oracle at this size, so the checks are the gather that defines dispatch (done by
+    torch indexing on the tags) and the round trip back to the input."""
+    _, ops, _, _ = brt_mod
+    dev = torch.device("cuda:0")
+    T, d, E = 1_200_000, 1024, 8
+    g = torch.Generator(device=dev).manual_seed(11)
+    # bit patterns of normal bf16 numbers of either sign (the combine multiplies by a unit gate and
+    # adds to zero in fp32, which keeps every such pattern but not NaN payloads or -0)
+    x = torch.randint(128, 30000, (T, d), dtype=torch.int16, device=dev, generator=g)
+    x = (x - 32768 * torch.randint(0, 2, (T, 1), dtype=torch.int16, device=dev, generator=g))
+    x = x.to(torch.int16).view(torch.bfloat16)
+    path = torch.randint(0, E, (T,), device=dev, generator=g)
+    mask = torch.zeros(T, E, dtype=torch.int32, device=dev)
+    mask[torch.arange(T, device=dev), path] = 1
+
+    idx, loads = ops.generate_indices_and_loads(mask)
+    assert int(loads.sum()) == T
+    y, tags = ops.dispatch_with_indices_and_loads(x, idx, loads, tag_generating=True)
+    assert y.shape == (T, d)
+    tags64 = tags.long()
+    assert torch.equal(torch.sort(tags64).values, torch.arange(1, T + 1, device=dev))
+    # seat order: path by path, tokens ascending inside a path
+    assert torch.equal(path[tags64 - 1], torch.sort(path).values)
+    assert torch.equal(y.view(torch.int16), x[tags64 - 1].view(torch.int16))
+    back = ops.combine_with_indices_and_loads(y, idx, loads)[0]
+    assert torch.equal(back.view(torch.int16), x.view(torch.int16))
+    del back
+
+    ids = path.to(torch.int32).view(T, 1)
+    r_loads, r_counts, seat_rows, row_entries = ops.route_by_path(ids, E)[:4]
+    assert torch.equal(r_loads.cpu(), loads.cpu())
+    assert torch.equal(row_entries, tags)
+    y2 = ops.dispatch_by_rows(x, row_entries, 1)
+    assert torch.equal(y2.view(torch.int16), y.view(torch.int16))
+    del y2
+    back2 = ops.combine_by_rows(y, ids, seat_rows)
+    assert torch.equal(back2.view(torch.int16), x.view(torch.int16))
