@@ -13,7 +13,10 @@
  *     (brt_hip_last_error() gives the message of the calling thread's last
  *     failure); they never throw, never allocate device memory, never
  *     synchronise the stream, and only enqueue work on `stream`;
- *   - the caller owns every buffer, including workspaces.
+ *   - the caller owns every buffer, including workspaces;
+ *   - sizes: element counts of index-shaped arguments (T*E, T*k) must stay
+ *     below 2^31 (BRT_E_UNSUPPORTED otherwise); row buffers may be of any
+ *     size, their offsets are 64-bit.
  */
 #ifndef BRT_HIP_H_
 #define BRT_HIP_H_
