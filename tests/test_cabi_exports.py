@@ -76,3 +76,18 @@ def test_missing_library_is_an_error(monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libbrt_hip.so"))
     with pytest.raises(RuntimeError, match="no CPU fallback"):
         _lib.lib()
+
+
+def test_counts_of_two_to_the_31_and_more_are_refused():
+    """Index-shaped arguments are addressed with 32-bit element counts; larger ones are an
+    error before anything is launched (no GPU needed)."""
+    handle = _lib.lib()
+    T, E = 1 << 26, 64
+    assert handle.brt_hip_dispatch(None, None, None, None, None, None, None, None,
+                                   T, 4, E, 4, 0, 1, 0, 0, None) == -4
+    assert b"2^31" in handle.brt_hip_last_error()
+    assert handle.brt_hip_combine(None, None, None, None, None, T, 4, E, 4, 0, 0, 0, 0, 0, None) == -4
+    assert handle.brt_hip_topk_hot_mask(None, None, T, E, 1, 0, None) == -4
+    assert handle.brt_hip_route_by_path(None, 1 << 30, 2, E, None, 0, 0, 0, 0, None, None, None,
+                                        None, 0, None, 0, None) == -4
+    assert b"T*k" in handle.brt_hip_last_error()
