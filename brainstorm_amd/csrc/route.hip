@@ -1012,10 +1012,16 @@ __global__ __launch_bounds__(kBlock) void combine_rows_kernel(CombineRowsArgs a)
           if (off < cpr) {
             if constexpr (IN_DT == OUT_DT) {
               // streaming store, as in dispatch (rows of more than 128 bytes): nothing here reads the row again
-              store_unit<LS >= 4>(reinterpret_cast<U*>(dst + (to + off) * 16), val[u]);
+              // (a row that is summed into a zero accumulator comes out with +0 for every -0)
+              U v = val[u];
+#pragma unroll
+              for (int q = 0; q < 4; ++q) v[q] = plus_zero<IN_DT>(v[q]);
+              store_unit<LS >= 4>(reinterpret_cast<U*>(dst + (to + off) * 16), v);
             } else {
               float x[NE];
               unpack<IN_DT, 16>(val[u], x);
+#pragma unroll
+              for (int q = 0; q < NE; ++q) x[q] = x[q] + 0.0f;  // -0 -> +0, as the sum would
               pack_store<OUT_DT, NE>(dst + (to + off) * OUT_BYTES, x);
             }
           }

@@ -24,6 +24,21 @@ __device__ __forceinline__ uint32_t unit_word(const typename Unit<BYTES>::type& 
   else return v;
 }
 
+// A word of DT elements with every -0 turned into +0, all other bit patterns kept: what adding the
+// element to a zero accumulator does to it (0 + -0 = +0), for kernels that move a row instead of
+// summing it.  16-bit halves: flip the sign bits, find the halves that are now zero without a carry
+// crossing between them, clear the sign of exactly those.
+template <int DT>
+__device__ __forceinline__ uint32_t plus_zero(uint32_t w) {
+  if constexpr (DT == BRT_F32) {
+    return w == 0x80000000u ? 0u : w;
+  } else {
+    const uint32_t t = w ^ 0x80008000u;
+    const uint32_t nonzero = (((t & 0x7fff7fffu) + 0x7fff7fffu) | t) & 0x80008000u;
+    return w & ~(nonzero ^ 0x80008000u);
+  }
+}
+
 constexpr int elem_bytes(int dt) { return dt == BRT_F32 ? 4 : 2; }
 
 // Unpacks BYTES of DT elements to fp32.

@@ -329,7 +329,10 @@ def test_combine_by_tags_equals_gather_combine(hip, T, E, cell, in_dtype, out_dt
                                         max_path_padding=mpl != 0, max_path_load=mpl, dtype=in_dtype)
     assert same_bits(y, want_y) and same_bits(y0, want_y)
     assert np.array_equal(tags, want_tags) and np.array_equal(tags0, want_tags)
-    expert_out = as_dtype_bits(rng.standard_normal(y.shape), in_dtype)
+    vals = rng.standard_normal(y.shape)
+    vals[::3, ::5] = -0.0                 # a summed row turns -0 into +0 (0 + -0); a moved row must too
+    vals[1::4, 2::7] = 0.0
+    expert_out = as_dtype_bits(vals, in_dtype)
     res = as_dtype_bits(rng.standard_normal((T, cell)), out_dtype)
     want = oracle.combine(expert_out, idx, loads, out_data=res, max_path_padding=mpl != 0,
                           in_dtype=in_dtype, out_dtype=out_dtype)

@@ -366,6 +366,21 @@ def test_combine_inverts_top1_dispatch_exactly():
     assert np.array_equal(oracle.combine(y, idx, loads), x)
 
 
+def test_combine_turns_minus_zero_into_plus_zero():
+    """The output starts at zero and the row is added to it (atomicAdd into torch::zeros,
+    route.cu:236-244, router.cc:460): IEEE 0 + -0 is +0, so a -0 never survives a combine, while
+    a dispatch, which moves rows, keeps it."""
+    mask = np.array([[1, 0], [0, 1]], dtype=np.int32)
+    idx, loads = oracle.generate_indices_and_loads(mask)
+    x = np.array([[-0.0, 1.5], [2.5, -0.0]], dtype=np.float32)
+    y, _ = oracle.dispatch(x, idx, loads)
+    assert np.array_equal(y.view(np.uint32), x.view(np.uint32))
+    out = oracle.combine(y, idx, loads)
+    assert np.array_equal(out.view(np.uint32), np.abs(x).view(np.uint32))
+    res = oracle.combine(y, idx, loads, out_data=np.full((2, 2), 9.0, dtype=np.float32))
+    assert np.array_equal(res.view(np.uint32), np.abs(x).view(np.uint32))
+
+
 def test_combine_of_topk_dispatch_is_k_times_input():
     # sample/cpp/dispatch.ipynb cells 1-3: allclose(final, 2 * in) for top-2 without drops
     T, E, d = 2048, 4, 24
