@@ -35,6 +35,7 @@
 #include <type_traits>
 
 #include "common.hpp"
+#include "rows.hpp"
 
 namespace brt {
 namespace {
@@ -478,9 +479,14 @@ __global__ __launch_bounds__(WAVES * 64) void grouped_gemm_kernel(GemmArgs a) {
         if (a.scatter) to = s_cell[r];
         // streaming stores: the output is not read again by this kernel, and written through the
         // L2 like ordinary stores it pushes the operand lines out that the column tiles share
-        if (to >= 0 && n0 + c * 8 < a.N)
-          stream_out(*reinterpret_cast<const u32x4*>(stage_out + rl * OUT_ROW + c * 16),
-                     reinterpret_cast<u32x4*>(oc + static_cast<size_t>(to) * a.N + c * 8));
+        if (to >= 0 && n0 + c * 8 < a.N) {
+          u32x4 v = *reinterpret_cast<const u32x4*>(stage_out + rl * OUT_ROW + c * 16);
+          if (a.scatter) {  // the combine this store stands for adds the row to zero: -0 becomes +0
+#pragma unroll
+            for (int w = 0; w < 4; ++w) v[w] = plus_zero<BRT_BF16>(v[w]);
+          }
+          stream_out(v, reinterpret_cast<u32x4*>(oc + static_cast<size_t>(to) * a.N + c * 8));
+        }
       }
     }
     if (nt + 1 < nt_end) {

@@ -155,7 +155,8 @@ int brt_hip_combine(const void* src, void* dst, const void* gates, const int32_t
  * them on the tag stack of the routed tensor).  Gives exactly the rows that
  * brt_hip_combine(..., gates=NULL, is_residual=1) gives for such a route, with
  * one memory round trip less: a row and its tag are fetched together, nothing has
- * to be looked up in the [T,E] index matrix first.
+ * to be looked up in the [T,E] index matrix first.  "Exactly" includes the zero that a
+ * sum starting at zero makes of a -0 (0 + -0 = +0): a -0 element is stored as +0.
  *
  *   src       [P, cell] in in_dtype
  *   dst       [T, cell] in out_dtype (= in_dtype, or BRT_F32); rows of cells that
@@ -212,8 +213,8 @@ int brt_hip_grouped_gemm(const void* x, const void* const* weights, const void* 
  *                 slot is a row of zeros.  gather_in=0: x is [P,K] as above.
  *   scatter_out=1 out is cell-major [T,N]; row s of expert e is stored to
  *                 out[tags[s,e]-1] (what combine does for a route in which no cell is
- *                 on more than one path, without gates, with out as the residual);
- *                 rows of empty slots are dropped.  scatter_out=0: out is [P,N].
+ *                 on more than one path, without gates, with out as the residual,
+ *                 including +0 for a -0 element); rows of empty slots are dropped.  scatter_out=0: out is [P,N].
  *   Only rows s < loads[e] of column e are used, so a clipped capacity drops the
  *   overflow exactly as seat indices beyond loads[e] do.  With gather_in the cell-major
  *   input is limited to 2 GiB.

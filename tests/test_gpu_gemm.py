@@ -343,3 +343,43 @@ def test_grouped_gemm_random_shapes():
         N = int(rng.integers(1, 120)) * 8
         run(loads, K, N, act=("none", "gelu", "relu")[case % 3], bias=bool(case % 2), seed=case,
             slack=int(rng.integers(0, 9)))
+
+
+def test_scattering_gemm_stores_plus_zero_where_the_combine_would():
+    """Products that underflow leave -0 in the output of the plain GEMM; the combine adds the row
+    to zero and so stores +0, and the GEMM that stores through the route has to do the same."""
+    from brainstorm_amd._C import router as c_router
+    from brainstorm_amd.jit import grouped_linear
+
+    T, E, K, N = 256, 4, 64, 64
+    path = torch.arange(T) % E
+    mask = torch.zeros(T, E, dtype=torch.int32)
+    mask[torch.arange(T), path] = 1
+    d_mask = mask.cuda()
+    x = torch.full((T, K), 2.0 ** -70, dtype=torch.bfloat16, device="cuda")
+    ws = []
+    for e in range(E):
+        w = torch.randn(N, K, generator=torch.Generator().manual_seed(e)) * 2.0 ** 60
+        w[::2] = -(2.0 ** -70)   # 64 products of -2^-140: half a bf16 step below zero
+        w[1::4] = -(2.0 ** -100)  # products far below the smallest fp32 number
+        ws.append(w.to(torch.bfloat16).cuda())
+    table = torch.tensor([w.data_ptr() for w in ws], dtype=torch.int64, device="cuda")
+
+    idx, loads = c_router.generate_indices_and_loads(d_mask)
+    (y,) = c_router.dispatch_with_indices_and_loads(x, idx, loads)
+    y2 = torch.empty(T, N, dtype=torch.bfloat16, device="cuda")
+    grouped_linear(y, y2, table, None, loads, K, N)
+    assert (y2.view(torch.int16) == -32768).any(), "the case is meant to produce -0"
+    residual = torch.ones(T, N, dtype=torch.bfloat16, device="cuda")
+    (want,) = c_router.combine_with_indices_and_loads(y2, idx, loads, None, residual.clone())
+    assert not (want.view(torch.int16) == -32768).any()
+
+    tags, _ = c_router.generate_indices_and_loads(d_mask, None, False, False, True)
+    out = residual.clone()
+    grouped_linear(y, out, table, None, loads, K, N, tags=tags, scatter=True, rows=T)
+    assert torch.equal(out.view(torch.int16), want.view(torch.int16))
+    ids = path.to(torch.int32).view(T, 1).cuda()
+    row_entries = c_router.route_by_path(ids, E, rows=T)[3]
+    out_r = residual.clone()
+    grouped_linear(y, out_r, table, None, loads, K, N, row_entries=row_entries, scatter=True, rows=T)
+    assert torch.equal(out_r.view(torch.int16), want.view(torch.int16))
