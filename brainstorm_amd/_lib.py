@@ -36,6 +36,12 @@ SIGNATURES = {
         [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_int,
          _c_ptr, _c_size, _c_ptr],
     ),
+    "brt_hip_static_scratch_bytes": (_c_size, []),
+    "brt_hip_generate_indices_and_loads_static": (
+        _c_int,
+        [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_int,
+         _c_ptr],
+    ),
     "brt_hip_throttle_hotmask": (
         _c_int, [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr, _c_size, _c_ptr]),
     "brt_hip_convert_index_format": (

@@ -34,8 +34,16 @@
 // wavefronts' column sums meet in LDS (one launch).
 #include <algorithm>
 #include <cstdlib>
+#include <mutex>
 
 #include "common.hpp"
+
+// Scratch of brt_hip_generate_indices_and_loads_static: the per-band column sums that the first
+// kernel of index generation hands to the second, for callers that cannot bring a workspace of
+// their own.  Every GPU holds its own copy at its own address for the life of the process; in
+// host code the name is only a handle for hipGetSymbolAddress, never an address to pass on.
+constexpr size_t kStaticScratchInts = size_t{1} << 18;  // 1 MiB
+static __device__ __align__(256) int scratch[kStaticScratchInts];
 
 namespace brt {
 namespace {
@@ -423,6 +431,30 @@ int launch_scan(int mode, ScanArgs& a, void* workspace, size_t workspace_bytes, 
   return check_launch("band_apply_kernel");
 }
 
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+// Device address of `scratch` on the current device, resolved once per device.
+int static_scratch(void** out) {
+  int device = -1;
+  hipError_t err = hipGetDevice(&device);
+  if (err != hipSuccess) return fail(BRT_E_LAUNCH, "hipGetDevice: %s", hipGetErrorString(err));
+  if (device < 0 || device >= kMaxDevices)
+    return fail(BRT_E_UNSUPPORTED, "device ordinal %d outside [0, %d)", device, kMaxDevices);
+  std::lock_guard<std::mutex> hold(g_scratch_mutex);
+  if (g_scratch_ptr[device] == nullptr) {
+    void* ptr = nullptr;
+    err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (err != hipSuccess || ptr == nullptr)
+      return fail(BRT_E_LAUNCH, "hipGetSymbolAddress(scratch) on device %d: %s", device,
+                  hipGetErrorString(err));
+    g_scratch_ptr[device] = ptr;
+  }
+  *out = g_scratch_ptr[device];
+  return BRT_OK;
+}
+
 }  // namespace
 }  // namespace brt
 
@@ -471,6 +503,31 @@ extern "C" int brt_hip_generate_indices_and_loads(const int32_t* mask, int32_t* 
   a.capacity_padding = capacity_padding;
   a.path_wise_padding = path_wise_padding;
   return launch_scan(is_tag_index ? kTag : kSeat, a, workspace, workspace_bytes, stream);
+}
+
+extern "C" size_t brt_hip_static_scratch_bytes(void) { return kStaticScratchInts * sizeof(int); }
+
+extern "C" int brt_hip_generate_indices_and_loads_static(const int32_t* mask, int32_t* indices,
+                                                         int32_t* loads, int32_t* counts, int T,
+                                                         int E, const int32_t* caps, int C,
+                                                         int capacity_padding,
+                                                         int path_wise_padding, int is_tag_index,
+                                                         void* stream) {
+  if (T < 0 || E <= 0) return fail(BRT_E_INVALID, "bad shape T=%d E=%d", T, E);
+  if (static_cast<long>(T) * E >= (1l << 31)) return fail(BRT_E_UNSUPPORTED, "T*E >= 2^31");
+  const size_t need = brt_hip_scan_workspace_bytes(T, E);
+  if (need > kStaticScratchInts * sizeof(int))
+    return fail(BRT_E_WORKSPACE,
+                "a [%d,%d] mask needs %zu bytes of scratch, the built-in buffer holds %zu: use "
+                "brt_hip_generate_indices_and_loads with a workspace",
+                T, E, need, kStaticScratchInts * sizeof(int));
+  void* ptr = nullptr;
+  if (const int rc = static_scratch(&ptr)) return rc;
+  // nothing in the scratch has to start at zero: every word the second kernel reads was written
+  // by the first kernel of the same call
+  return brt_hip_generate_indices_and_loads(mask, indices, loads, counts, T, E, caps, C,
+                                            capacity_padding, path_wise_padding, is_tag_index, ptr,
+                                            kStaticScratchInts * sizeof(int), stream);
 }
 
 extern "C" int brt_hip_throttle_hotmask(const int32_t* mask, int32_t* out, int32_t* prefix,

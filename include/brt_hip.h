@@ -80,6 +80,26 @@ int brt_hip_generate_indices_and_loads(const int32_t* mask, int32_t* indices, in
                                        void* stream);
 
 /*
+ * brt_hip_generate_indices_and_loads for callers that cannot allocate (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
+ * reference.  Same arguments and results without the workspace: the per-band column sums go
+ * through a buffer built into the library (brt_hip_static_scratch_bytes() bytes, 1 MiB, held on
+ * every GPU the library runs on until the process ends).  The entry point calls no allocating
+ * routine.  A mask whose brt_hip_scan_workspace_bytes(T, E) exceeds the buffer is refused with
+ * BRT_E_WORKSPACE (nothing is launched); [8192,64], [100352,8] and [1<<20,64] fit.  The buffer
+ * carries nothing from call to call and needs no clearing, but every call on one GPU uses the
+ * same buffer: calls that can overlap on one GPU (two streams, two threads) race.  The first
+ * call on a device looks the buffer's address up (hipGetSymbolAddress); make that call outside
+ * graph capture.
+ */
+size_t brt_hip_static_scratch_bytes(void);
+int brt_hip_generate_indices_and_loads_static(const int32_t* mask, int32_t* indices,
+                                              int32_t* loads, int32_t* counts, int T, int E,
+                                              const int32_t* caps, int C, int capacity_padding,
+                                              int path_wise_padding, int is_tag_index,
+                                              void* stream);
+
+/*
  * Replaces router::ThrottleHotmask (location.h:13-19, location.cu:59-130,304-315).
  *   out[t,e] = 1 iff mask[t,e]==1 and prefix[e] + cumsum(mask)[t,e] <= threshold[e]
  *   prefix[e] <- min(prefix[e] + sum(mask[:,e]), threshold[e])   (in place)
