@@ -210,7 +210,11 @@ __global__ __launch_bounds__(WAVES * 64) void grouped_gemm_kernel(GemmArgs a) {
         cell = a.tag_div > 1 ? (entry - 1) / a.tag_div : entry - 1;
         cell = (entry >= 1 && cell < a.T) ? cell : -1;
       } else {
-        const int tag = a.tags[static_cast<size_t>(seat0 + r) * a.E + e];
+        // the tag matrix has T rows; a load padded beyond T (capacity above the batch size) names
+        // slots that do not exist: they are empty, as in dispatch (route.cu:84-92 bounds the slot
+        // by the cell count)
+        const int slot = seat0 + r;
+        const int tag = slot < a.T ? a.tags[static_cast<size_t>(slot) * a.E + e] : 0;
         cell = (tag >= 1 && tag <= a.T) ? tag - 1 : -1;
       }
       s_cell[r] = cell;

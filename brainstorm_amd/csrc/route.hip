@@ -74,7 +74,10 @@ __device__ __forceinline__ void wave_path_tables(const int* __restrict__ loads, 
   int carry = 0;
   for (int base = 0; base < E; base += kWave) {
     const int e = base + lane;
-    const int v = e < E ? loads[e] : 0;
+    int v = e < E ? loads[e] : 0;
+    // fixed stride: a path's block ends at the stride, seats beyond it are dropped (the reference
+    // would write them into the next path's block, racing with that path's own rows)
+    if (stride != 0) v = min(v, stride);
     const int incl = wave_inclusive_scan(v);
     if (e < E) {
       s_loads[e] = v;
@@ -452,6 +455,7 @@ __device__ __forceinline__ SmallTables small_tables(const int* __restrict__ load
                                                     int ep_shift, int lane) {
   SmallTables t;
   t.my_load = lane < E ? loads[lane] : 0;
+  if (mpl != 0) t.my_load = min(t.my_load, mpl);  // fixed stride: a path's block ends at the stride
   const int incl = wave_inclusive_scan(t.my_load);
   t.my_start = mpl != 0 ? lane * mpl : incl - t.my_load;
   if (ep_shift == 6) {

@@ -142,7 +142,9 @@ int brt_hip_convert_index_format(const int32_t* src, int32_t* dst, const int32_t
  *   cell      elements per row, in units of `dtype`
  *   P         rows of dst (rows >= P are never written)
  *   max_path_load  0 = paths packed back to back (start[e] = sum(loads[:e]));
- *             otherwise start[e] = e*max_path_load
+ *             otherwise start[e] = e*max_path_load and seats beyond max_path_load are
+ *             dropped (a path's block ends at the stride; brt_hip_combine applies the
+ *             same bound)
  *   Weighted rows are src*gate rounded once to `dtype`; unweighted rows are
  *   byte copies.
  */
@@ -235,8 +237,9 @@ int brt_hip_grouped_gemm(const void* x, const void* const* weights, const void* 
  *                 out[tags[s,e]-1] (what combine does for a route in which no cell is
  *                 on more than one path, without gates, with out as the residual,
  *                 including +0 for a -0 element); rows of empty slots are dropped.  scatter_out=0: out is [P,N].
- *   Only rows s < loads[e] of column e are used, so a clipped capacity drops the
- *   overflow exactly as seat indices beyond loads[e] do.  With gather_in the cell-major
+ *   Only rows s < min(loads[e], T) of column e are used, so a clipped capacity drops the
+ *   overflow exactly as seat indices beyond loads[e] do, and a load padded beyond the T rows
+ *   the tag matrix has (a capacity above the batch size) names empty slots.  With gather_in the cell-major
  *   input is limited to 2 GiB.
  */
 int brt_hip_grouped_gemm_routed(const void* x, const void* const* weights,

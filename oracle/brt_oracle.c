@@ -285,7 +285,10 @@ static void copy_row(const void* src, size_t src_row, void* dst, size_t dst_row,
  *   new_tags (zero-filled by the caller) receive old_tags[source row]
  *         (route.cu:51-53); old_tags NULL means "no tag generation".
  *   Rows >= P are never written (guard added here; the reference would write
- *   out of bounds).
+ *   out of bounds).  With a fixed stride (max_path_load != 0) seats beyond the
+ *   stride are dropped: the reference would write them into the next path's
+ *   block, racing with that path's own rows (route.cu:37-50 has no such guard),
+ *   so there is no defined result to reproduce.
  */
 void oracle_dispatch(const void* src, void* dst, const void* gates, const int32_t* idx,
                      const int32_t* loads, const int32_t* old_tags, int32_t* new_tags, int T,
@@ -296,6 +299,7 @@ void oracle_dispatch(const void* src, void* dst, const void* gates, const int32_
   for (int e = 0; e < E; ++e) {
     long load_start = max_path_load != 0 ? (long)e * max_path_load : start;
     int path_load = loads[e];
+    if (max_path_load != 0 && path_load > max_path_load) path_load = max_path_load;
     if (!is_tag_index) {
       for (int t = 0; t < T; ++t) {
         int seat = idx[(size_t)t * E + e];
@@ -357,6 +361,8 @@ void oracle_combine(const void* src, void* dst, const void* gates, const int32_t
         int load = loads[e];
         long load_start = max_path_load != 0 ? (long)e * max_path_load : start;
         start += load;
+        /* fixed stride: a path's block ends at the stride (see oracle_dispatch) */
+        if (max_path_load != 0 && load > max_path_load) load = max_path_load;
         if (seat == 0 || seat > load || seat < 0) continue;
         long row = load_start + seat - 1;
         if (row >= P) continue;

@@ -121,6 +121,8 @@ def _expert_tables(E, K, N, seed):
     (2048, 16, 256, 512, 160, True),      # every expert padded to 160 rows (empty slots = zero rows)
     (1000, 8, 136, 264, 400, False),      # several row blocks per expert, K and N tails
     (300, 64, 64, 128, 16, False),        # most experts nearly empty
+    (16, 4, 64, 128, 32, True),           # capacity above the batch size: loads name slots past the tag matrix
+    (100, 3, 72, 136, 256, True),         # the same with a row block that ends past the matrix
 ])
 def test_ffn_with_gather_and_scatter_equals_dispatch_ffn_combine(T, E, d, dff, cap, pad):
     """index generation in tag mode -> GEMM reading cells through the tags -> GEMM storing

@@ -274,6 +274,32 @@ def test_combine_max_path_padding_and_odd_rows(hip):
             assert same_bits(got, want)
 
 
+@pytest.mark.parametrize("T,E,k,cell", [(400, 4, 1, 8), (2048, 64, 1, 768), (900, 100, 2, 24)])
+def test_loads_above_the_fixed_stride_are_clipped_to_it(hip, T, E, k, cell):
+    """max_path_load below some loads (a router that froze its stride on an earlier, smaller
+    batch): seats beyond the stride are dropped by dispatch and combine alike, in every kernel
+    family (lane tables, tag generation, LDS tables for more than 64 paths)."""
+    mask, logits = topk_mask(T, E, k, seed=T + E)
+    idx, loads = oracle.generate_indices_and_loads(mask)
+    counts = mask.sum(0).astype(np.int32)
+    mpl = max(1, int(loads.max()) // 2)
+    rng = np.random.default_rng(T)
+    for dtype in ("f32", "bf16"):
+        x = as_dtype_bits(rng.standard_normal((T, cell)), dtype)
+        want, want_tags = oracle.dispatch(x, idx, loads, tag_generating=True, max_path_padding=True,
+                                          max_path_load=mpl, dtype=dtype)
+        for c in (None, counts):
+            for tg in (False, True):
+                got, got_tags = hip.dispatch(x, idx, loads, None, c, tg, max_path_load=mpl, dtype=dtype)
+                assert same_bits(got, want)
+                assert not tg or np.array_equal(got_tags, want_tags)
+        gates = as_dtype_bits(softmax(logits), dtype)
+        for g in (None, gates):
+            want_c = oracle.combine(want, idx, loads, gates=g, max_path_padding=True, in_dtype=dtype)
+            got_c = hip.combine(want, idx, loads, g, max_path_load=mpl, in_dtype=dtype)
+            assert same_bits(got_c, want_c)
+
+
 # ------------------------------------------------- gate front-end: top-k hot mask
 @pytest.mark.parametrize("T,E,k,dtype", [
     (8192, 64, 1, "f32"), (16384, 32, 2, "f32"), (100352, 8, 1, "f16"), (1000, 5, 3, "bf16"),

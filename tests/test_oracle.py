@@ -449,6 +449,24 @@ def test_combine_max_path_padding():
     assert np.array_equal(oracle.combine(y, idx, loads, max_path_padding=True), x)
 
 
+def test_fixed_stride_drops_seats_beyond_the_stride():
+    """A path whose load exceeds the fixed stride keeps only the seats inside its block (the
+    reference would write the others into the next path's block): dispatch equals the numpy
+    gather with the loads clipped to the stride, and combine reads back exactly those rows."""
+    T, E, d, mpl = 400, 4, 8, 60
+    mask, _ = topk_mask(T, E, 1, seed=93)
+    idx, loads = oracle.generate_indices_and_loads(mask)
+    assert loads.max() > mpl and loads.min() < mpl + 60
+    x = np.random.default_rng(94).standard_normal((T, d)).astype(np.float32)
+    y, tags = oracle.dispatch(x, idx, loads, tag_generating=True, max_path_padding=True,
+                              max_path_load=mpl)
+    want, src = brute_dispatch(x, idx, np.minimum(loads, mpl), max_path_load=mpl)
+    assert y.shape[0] == E * mpl and np.array_equal(y, want) and np.array_equal(tags, src + 1)
+    back = oracle.combine(y, idx, loads, max_path_padding=True)
+    kept = ((idx >= 1) & (idx <= mpl)).any(1)
+    assert np.array_equal(back[kept], x[kept]) and not back[~kept].any()
+
+
 # ------------------------------------------------------------------ top-k hot mask
 def _topk_mask_by_stable_sort(score, k):
     """Independent statement: stable sort of the columns by descending score (NaN first)."""
