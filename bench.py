@@ -1,30 +1,40 @@
 #!/usr/bin/env python3
 """Benchmark of the MoE routing hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only PHASE] [--no-cpu-baseline]
 
-Workload: the Switch-MoE layer of the baseline configurations, bf16, 8192 tokens x d=768,
-64 experts, top-1 softmax gate over N(0,1) logits, capacity factor 1.25
-(capacity 160, overflow dropped), expert FFN 768->3072->768 GELU with N(0,0.02)
-weights; seeded synthetic data, everything resident in HBM before timing.
+Workload: the Switch-MoE layer of the baseline configurations (BASELINE.json configs[1]), bf16,
+8192 tokens x d=768, 64 experts, top-1 softmax gate over N(0,1) logits, capacity factor 1.25
+(capacity 160, overflow dropped), expert FFN 768->3072->768 GELU with N(0,0.02) weights; seeded
+synthetic data, everything resident in HBM before timing.
 
-A step is one pass of the hot path over the batch, called through the C ABI of
-libbrt_hip.so and replayed as one HIP graph:
+A step is one pass of the hot path over the batch, called through the C ABI of libbrt_hip.so and
+replayed as one HIP graph:
     index/load generation -> dispatch -> grouped FFN (two launches) -> combine.
-The route is top-1, so the step takes the path the routers take for single-path
-protocols: dispatch also writes the per-row tags and combine is the tag-driven
-scatter form (brt_hip_combine_by_tags); the index-driven gather form
-(brt_hip_combine) is timed beside it as `combine_gather`.
-`value` is the headline metric: algorithmic bytes of dispatch + combine divided
-by the sum of their kernel times.  Kernel times are measured in this process
-with HIP events around graphs of back-to-back launches of the one kernel, on the
-stream the kernels are launched on.  The reference's PyTorch CPU routing path
-(oracle/torch_path.py) is timed on the host cores as `cpu_baseline`.
-Prints ONE JSON line.
+The route is top-1, so the step takes the path the routers take for single-path protocols:
+dispatch also writes the per-row tags and combine is the tag-driven scatter form
+(brt_hip_combine_by_tags); the index-driven gather form (brt_hip_combine) is timed beside it.
+
+Phases (`--only` runs the set-up and one of them, so that a profiler sees one kind of launch):
+  step     the K timed steps as one HIP graph                          -> ms_per_step, layer_us
+  instep   the step launched eagerly with an event after every launch: kernel durations with the
+           inputs as the layer leaves them                             -> `value`, `roofline`
+  cold     every routing kernel launched back to back over a ring of buffer sets larger than the
+           last-level cache, so that every launch reads its inputs from HBM
+  warm     the same kernels back to back on ONE set of buffers (cache resident at this size)
+  ffn      the two grouped GEMMs of the layer                          -> `roofline_ffn`
+  configs  the other BASELINE configurations at full size (routing of 1, 3, 4; FFN of 3 and 5)
+  extras   gate / compact route / tag-index gather / folded layers, library GEMMs
+`value` is dispatch + combine bytes over the sum of their durations INSIDE THE STEP, with the bytes
+each kernel has to move (the tag-driven combine does not read the [T,E] index matrix).  Kernel
+times are measured in this process with HIP events on the stream the kernels are launched on.  The reference's PyTorch CPU routing path (oracle/torch_path.py) is timed on the host
+cores as `cpu_baseline`.  Prints ONE JSON line.
 """
 import argparse
 import json
+import math
 import os
+import re
 import sys
 import time
 
@@ -34,21 +44,14 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E
 MFMA_BF16_PEAK_TFLOPS = 2500.0
-
-# Bytes per launch seen by the memory side for this workload: rocprofv3 --pmc
-# FETCH_SIZE and WRITE_SIZE (KiB), each scaled by what the same counter reads for
-# a 12 MiB device-to-device copy (fetch x1.996, write x1.000).
-MEASURED_TRAFFIC_BYTES = {
-    "dispatch": int((7197.5 * 1.996 + 12459.4) * 1024),
-    "combine": int((6221.5 * 1.996 + 12288.0) * 1024),
-    "combine_gather": int((7196.0 * 1.996 + 12288.2) * 1024),
-    "ffn_gemm1_gelu": int((155947.1 * 1.996 + 49152.0) * 1024),
-    "ffn_gemm2": int((172184.1 * 1.996 + 12288.0) * 1024),
-}
+LAST_LEVEL_CACHE_BYTES = 256 << 20
+RING_BYTES = 768 << 20      # what one kernel touches going once round a ring of buffer sets: 3 x the last-level cache
 
 T, D, E, DFF = 8192, 768, 64, 3072
 CAPACITY = int(1.25 * (T // E))  # 160
 SEED = 2
+PHASES = ("all", "step", "instep", "cold", "warm", "ffn", "configs", "extras")
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "switch_moe_8k_pmc_traffic.md")
 
 
 def parse():
@@ -56,256 +59,556 @@ def parse():
     p.add_argument("--gpus", type=int, default=1)
     p.add_argument("--steps", type=int, default=200)
     p.add_argument("--warmup", type=int, default=20)
+    p.add_argument("--only", choices=PHASES, default="all")
     p.add_argument("--no-cpu-baseline", action="store_true")
     return p.parse_args()
 
 
-def main():
-    args = parse()
-    if args.gpus != 1:
-        sys.exit("bench.py measures one GPU: the routing hot path is built and measured on a "
-                 "single MI355X (no collectives in this build); run with --gpus 1")
-    import numpy as np
-    import torch
-
-    from brainstorm_amd import _lib
-
-    if not torch.cuda.is_available():
-        sys.exit("bench.py needs a GPU")
-    L = _lib.lib()
-    dev = torch.device("cuda:0")
-    torch.cuda.set_device(dev)
-    stream = torch.cuda.Stream()  # every kernel and every timing event goes on this stream
-
-    # ---------------------------------------------------------------- inputs
-    g = torch.Generator().manual_seed(SEED)
-    x32 = torch.randn(T, D, generator=g)
-    logits = torch.randn(T, E, generator=g)
-    probs = torch.softmax(logits, dim=1)
-    expert = probs.argmax(dim=1)
-    mask_h = torch.zeros(T, E, dtype=torch.int32)
-    mask_h[torch.arange(T), expert] = 1
-    wi_h = (torch.randn(E, DFF, D, generator=g) * 0.02).to(torch.bfloat16)
-    wo_h = (torch.randn(E, D, DFF, generator=g) * 0.02).to(torch.bfloat16)
-
-    x = x32.to(torch.bfloat16).to(dev)
-    mask = mask_h.to(dev)
-    caps = torch.tensor([CAPACITY], dtype=torch.int32, device=dev)
-    idx = torch.empty_like(mask)
-    loads_counts = torch.empty(2, E, dtype=torch.int32, device=dev)
-    loads, counts = loads_counts[0], loads_counts[1]
-    ws = torch.empty(max(16, L.brt_hip_scan_workspace_bytes(T, E)), dtype=torch.uint8, device=dev)
-
-    def sptr():
-        return stream.cuda_stream
-
-    def k_indexgen():
-        _lib.check(L.brt_hip_generate_indices_and_loads(
-            mask.data_ptr(), idx.data_ptr(), loads.data_ptr(), counts.data_ptr(), T, E,
-            caps.data_ptr(), 1, 0, 0, 0, ws.data_ptr(), ws.numel(), sptr()))
-
-    with torch.cuda.stream(stream):
-        k_indexgen()
-    stream.synchronize()
-    loads_h, counts_h = loads.cpu(), counts.cpu()
-    P = int(loads_h.sum())                               # rows of the dispatched buffer
-    R = int(torch.minimum(loads_h, counts_h).sum())      # rows actually routed
-    y = torch.empty(P, D, dtype=torch.bfloat16, device=dev)
-    row_tags = torch.empty(P, dtype=torch.int32, device=dev)
-    out = x.clone()                                      # residual: unrouted tokens keep x
-    out_gather = x.clone()
-
-    wi = wi_h.to(dev)
-    wo = wo_h.to(dev)
-    wi_tab = torch.tensor([wi[e].data_ptr() for e in range(E)], dtype=torch.int64, device=dev)
-    wo_tab = torch.tensor([wo[e].data_ptr() for e in range(E)], dtype=torch.int64, device=dev)
-    h = torch.empty(P, DFF, dtype=torch.bfloat16, device=dev)
-    y2 = torch.empty(P, D, dtype=torch.bfloat16, device=dev)
-
-    def k_dispatch():
-        _lib.check(L.brt_hip_dispatch(
-            x.data_ptr(), y.data_ptr(), None, idx.data_ptr(), loads.data_ptr(), counts.data_ptr(),
-            None, row_tags.data_ptr(), T, D, E, P, 0, 1, 0, _lib.BF16, sptr()))
-
-    def k_gemm1():
-        _lib.check(L.brt_hip_grouped_gemm(
-            y.data_ptr(), wi_tab.data_ptr(), None, h.data_ptr(), loads.data_ptr(), E, P, D, DFF,
-            _lib.ACT_GELU, sptr()))
-
-    def k_gemm2():
-        _lib.check(L.brt_hip_grouped_gemm(
-            h.data_ptr(), wo_tab.data_ptr(), None, y2.data_ptr(), loads.data_ptr(), E, P, DFF, D,
-            _lib.ACT_NONE, sptr()))
-
-    have_ffn = True
+def measured_traffic():
+    """HBM bytes per launch from the committed rocprofv3 --pmc summary (FETCH_SIZE / WRITE_SIZE,
+    scaled by a plain copy of known size): a line `traffic_bytes_per_launch: {...}` and the
+    commit the counters were taken at."""
     try:
-        with torch.cuda.stream(stream):
-            k_gemm1()
-            k_gemm2()
-        stream.synchronize()
-    except (NotImplementedError, RuntimeError) as err:
-        have_ffn = False
-        ffn_note = str(err)
+        text = open(TRAFFIC_FILE).read()
+    except OSError:
+        return {}, None
+    m = re.search(r"^traffic_bytes_per_launch:\s*(\{.*\})\s*$", text, re.M)
+    c = re.search(r"^taken_at_commit:\s*(\S+)", text, re.M)
+    return (json.loads(m.group(1)) if m else {}), (c.group(1) if c else None)
 
-    combine_src = y2 if have_ffn else y
 
-    def k_combine():
-        _lib.check(L.brt_hip_combine_by_tags(
-            combine_src.data_ptr(), out.data_ptr(), row_tags.data_ptr(), P, D, T,
-            _lib.BF16, _lib.BF16, sptr()))
+class Gpu:
+    """Stream, graph capture and event timing shared by all phases."""
 
-    def k_combine_gather():
-        _lib.check(L.brt_hip_combine(
-            combine_src.data_ptr(), out_gather.data_ptr(), None, idx.data_ptr(), loads.data_ptr(),
-            T, D, E, P, 0, 1, _lib.BF16, _lib.BF16, _lib.F32, sptr()))
+    def __init__(self, torch, lib_mod):
+        self.torch = torch
+        self._lib = lib_mod
+        self.L = lib_mod.lib()
+        self.dev = torch.device("cuda:0")
+        torch.cuda.set_device(self.dev)
+        self.stream = torch.cuda.Stream()  # every kernel and every timing event goes on this stream
 
-    # the same layer with dispatch folded into the operand load of the first GEMM and combine
-    # into the result store of the second one (tag-index matrix instead of seat indices)
+    def sptr(self):
+        return self.stream.cuda_stream
+
+    def check(self, code):
+        self._lib.check(code)
+
+    def run(self, *fns):
+        with self.torch.cuda.stream(self.stream):
+            for fn in fns:
+                fn()
+        self.stream.synchronize()
+
+    def capture(self, fns, repeat=1):
+        """One HIP graph holding `repeat` rounds of the launches in `fns`."""
+        torch = self.torch
+        fns = list(fns) if isinstance(fns, (list, tuple)) else [fns]
+        self.run(*fns)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=self.stream):
+            for _ in range(repeat):
+                for fn in fns:
+                    fn()
+        return graph
+
+    def timed(self, graph, replays=1):
+        torch = self.torch
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        with torch.cuda.stream(self.stream):
+            a.record(self.stream)
+            for _ in range(replays):
+                graph.replay()
+            b.record(self.stream)
+        self.stream.synchronize()
+        return a.elapsed_time(b)  # ms
+
+    def launch_us(self, fns, launches=400, repeats=3):
+        """Average duration of one launch: `fns` (one callable per buffer set, or a single one) are
+        launched round robin inside one graph, about `launches` launches per replay."""
+        fns = list(fns) if isinstance(fns, (list, tuple)) else [fns]
+        rounds = max(1, launches // len(fns))
+        graph = self.capture(fns, rounds)
+        self.timed(graph, 1)
+        runs = [self.timed(graph, 1) for _ in range(repeats)]
+        return sum(runs) / len(runs) * 1e3 / (rounds * len(fns))
+
+
+def ring_size(launch_bytes, most=64):
+    """Buffer sets in a ring such that one kernel, touching `launch_bytes` per launch, has gone
+    through RING_BYTES before it sees a set again."""
+    return max(2, min(most, math.ceil(RING_BYTES / max(launch_bytes, 1))))
+
+
+# ------------------------------------------------------------------ the Switch layer (configs[1])
+class SwitchLayer:
+    """Buffers and launches of the benchmark layer.  `sets` buffer sets hold the activations and
+    index matrices (set 0 is the one the step uses); the expert weights exist once: at 604 MB they
+    do not fit the last-level cache anyway."""
+
+    def __init__(self, gpu, sets, index_sets=1):
+        torch, L, dev = gpu.torch, gpu.L, gpu.dev
+        self.gpu = gpu
+        g = torch.Generator().manual_seed(SEED)
+        self.x32 = torch.randn(T, D, generator=g)
+        self.logits = torch.randn(T, E, generator=g)
+        self.probs = torch.softmax(self.logits, dim=1)
+        self.expert = self.probs.argmax(dim=1)
+        self.mask_h = torch.zeros(T, E, dtype=torch.int32)
+        self.mask_h[torch.arange(T), self.expert] = 1
+        wi_h = (torch.randn(E, DFF, D, generator=g) * 0.02).to(torch.bfloat16)
+        wo_h = (torch.randn(E, D, DFF, generator=g) * 0.02).to(torch.bfloat16)
+        self.caps = torch.tensor([CAPACITY], dtype=torch.int32, device=dev)
+        self.ws = torch.empty(max(16, L.brt_hip_scan_workspace_bytes(T, E)), dtype=torch.uint8, device=dev)
+        self.loads_counts = torch.empty(2, E, dtype=torch.int32, device=dev)
+        self.loads, self.counts = self.loads_counts[0], self.loads_counts[1]
+        x = self.x32.to(torch.bfloat16).to(dev)
+        mask = self.mask_h.to(dev)
+        self.sets = [dict(x=x, mask=mask, idx=torch.empty_like(mask))]
+        gpu.run(lambda: self.indexgen(0))
+        loads_h, counts_h = self.loads.cpu(), self.counts.cpu()
+        self.P = int(loads_h.sum())                               # rows of the dispatched buffer
+        self.R = int(torch.minimum(loads_h, counts_h).sum())      # rows actually routed
+        for s in range(sets):
+            if s > 0:
+                self.sets.append(dict(x=x.clone(), mask=mask.clone(), idx=torch.empty_like(mask)))
+            b = self.sets[s]
+            b["y"] = torch.empty(self.P, D, dtype=torch.bfloat16, device=dev)
+            b["row_tags"] = torch.empty(self.P, dtype=torch.int32, device=dev)
+            b["y2"] = torch.empty(self.P, D, dtype=torch.bfloat16, device=dev)
+            b["out"] = x.clone()                                  # residual: unrouted tokens keep x
+            b["out_gather"] = x.clone()
+        self.wi, self.wo = wi_h.to(dev), wo_h.to(dev)
+        self.wi_tab = torch.tensor([self.wi[e].data_ptr() for e in range(E)], dtype=torch.int64, device=dev)
+        self.wo_tab = torch.tensor([self.wo[e].data_ptr() for e in range(E)], dtype=torch.int64, device=dev)
+        self.h = torch.empty(self.P, DFF, dtype=torch.bfloat16, device=dev)
+        # every set needs valid indices, tags and rows before its kernels are timed on their own
+        for s in range(sets):
+            gpu.run(lambda: self.indexgen(s), lambda: self.dispatch(s), lambda: self.gemm1(s),
+                    lambda: self.gemm2(s))
+        # index generation touches 4 MB per launch: its ring is longer and holds masks and index
+        # matrices only
+        self.index_ring = [dict(mask=b["mask"], idx=b["idx"]) for b in self.sets]
+        while len(self.index_ring) < index_sets:
+            self.index_ring.append(dict(mask=mask.clone(), idx=torch.empty_like(mask)))
+
+    # ---- launches through the C ABI (s = buffer set) ---------------------------------------
+    def indexgen(self, s, ring=False):
+        b, gpu = (self.index_ring if ring else self.sets)[s], self.gpu
+        gpu.check(gpu.L.brt_hip_generate_indices_and_loads(
+            b["mask"].data_ptr(), b["idx"].data_ptr(), self.loads.data_ptr(), self.counts.data_ptr(),
+            T, E, self.caps.data_ptr(), 1, 0, 0, 0, self.ws.data_ptr(), self.ws.numel(), gpu.sptr()))
+
+    def dispatch(self, s):
+        b, gpu = self.sets[s], self.gpu
+        gpu.check(gpu.L.brt_hip_dispatch(
+            b["x"].data_ptr(), b["y"].data_ptr(), None, b["idx"].data_ptr(), self.loads.data_ptr(),
+            self.counts.data_ptr(), None, b["row_tags"].data_ptr(), T, D, E, self.P, 0, 1, 0,
+            gpu._lib.BF16, gpu.sptr()))
+
+    def gemm1(self, s):
+        b, gpu = self.sets[s], self.gpu
+        gpu.check(gpu.L.brt_hip_grouped_gemm(
+            b["y"].data_ptr(), self.wi_tab.data_ptr(), None, self.h.data_ptr(), self.loads.data_ptr(),
+            E, self.P, D, DFF, gpu._lib.ACT_GELU, gpu.sptr()))
+
+    def gemm2(self, s):
+        b, gpu = self.sets[s], self.gpu
+        gpu.check(gpu.L.brt_hip_grouped_gemm(
+            self.h.data_ptr(), self.wo_tab.data_ptr(), None, b["y2"].data_ptr(), self.loads.data_ptr(),
+            E, self.P, DFF, D, gpu._lib.ACT_NONE, gpu.sptr()))
+
+    def combine(self, s):
+        b, gpu = self.sets[s], self.gpu
+        gpu.check(gpu.L.brt_hip_combine_by_tags(
+            b["y2"].data_ptr(), b["out"].data_ptr(), b["row_tags"].data_ptr(), self.P, D, T,
+            gpu._lib.BF16, gpu._lib.BF16, gpu.sptr()))
+
+    def combine_gather(self, s):
+        b, gpu = self.sets[s], self.gpu
+        gpu.check(gpu.L.brt_hip_combine(
+            b["y2"].data_ptr(), b["out_gather"].data_ptr(), None, b["idx"].data_ptr(),
+            self.loads.data_ptr(), T, D, E, self.P, 0, 1, gpu._lib.BF16, gpu._lib.BF16,
+            gpu._lib.F32, gpu.sptr()))
+
+    def step(self, s=0):
+        self.indexgen(s)
+        self.dispatch(s)
+        self.gemm1(s)
+        self.gemm2(s)
+        self.combine(s)
+
+    # ---- bytes and flops per launch ------------------------------------------------------------
+    def bytes(self):
+        es, idx_bytes, P, R = 2, 4 * T * E, self.P, self.R
+        experts_used = int((self.loads.cpu() > 0).sum())
+        return {
+            # mask in, index matrix out
+            "indexgen": 2 * idx_bytes + 8 * E,
+            # routed rows in, every row of the buffer out, the index matrix in, the row tags out
+            "dispatch": R * D * es + P * D * es + idx_bytes + 4 * P,
+            # tag-driven: routed rows in and out, 4 bytes of tag per row; no index matrix
+            "combine": 2 * R * D * es + 4 * P,
+            # index-driven: rows in, every routed cell out, the index matrix in
+            "combine_gather": 2 * R * D * es + idx_bytes,
+            # weights of the experts that have rows, rows in, rows out
+            "ffn_gemm1_gelu": experts_used * D * DFF * es + R * D * es + R * DFF * es,
+            "ffn_gemm2": experts_used * D * DFF * es + R * DFF * es + R * D * es,
+        }
+
+    def flops(self):
+        return {"ffn_gemm1_gelu": 2.0 * self.R * D * DFF, "ffn_gemm2": 2.0 * self.R * DFF * D}
+
+
+def check_switch_layer(gpu, layer):
+    """Both combine forms must agree bit for bit on this route before anything is timed."""
+    torch = gpu.torch
+    gpu.run(lambda: layer.step(0), lambda: layer.combine_gather(0))
+    b = layer.sets[0]
+    if not torch.equal(b["out"].view(torch.int16), b["out_gather"].view(torch.int16)):
+        sys.exit("bench.py: tag-driven and index-driven combine disagree")
+    routed = (b["idx"] > 0) & (b["idx"] <= layer.loads.view(1, -1))
+    if int(routed.any(1).sum()) != layer.R:
+        sys.exit("bench.py: routed row count does not match the loads")
+
+
+def phase_step(gpu, layer, steps, warmup):
+    """The K steps are one HIP graph (as the layers of a model would be), launched once, so the
+    time per step holds no launch gaps between graphs; the warm-up replays a one-step graph."""
+    torch = gpu.torch
+    g_step = gpu.capture(lambda: layer.step(0))
+    g_steps = gpu.capture(lambda: layer.step(0), steps)
+    with torch.cuda.stream(gpu.stream):
+        for _ in range(warmup):
+            g_step.replay()
+    gpu.stream.synchronize()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ms_total = gpu.timed(g_steps, 1)
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    per_graph_launch_us = gpu.timed(g_step, steps) / steps * 1e3  # one graph launch per step
+    return {"ms_per_step": ms_total / steps, "wall_ms": wall_ms,
+            "layer_us_one_graph_launch_per_step": per_graph_launch_us}
+
+
+ROUTING_KERNELS = ("indexgen", "dispatch", "combine", "combine_gather")
+
+
+def phase_routing(gpu, layer, sets, index_sets):
+    """Average launch duration of each routing kernel over a ring of `sets` buffer sets."""
+    us = {}
+    for name in ROUTING_KERNELS:
+        fn = getattr(layer, name)
+        if name == "indexgen":
+            us[name] = gpu.launch_us([(lambda s=s: fn(s, True)) for s in range(index_sets)])
+        else:
+            us[name] = gpu.launch_us([(lambda s=s: fn(s)) for s in range(sets)])
+    return us
+
+
+def phase_ffn(gpu, layer):
+    us = {}
+    for name, fn in (("ffn_gemm1_gelu", layer.gemm1), ("ffn_gemm2", layer.gemm2)):
+        us[name] = gpu.launch_us(lambda: fn(0), launches=100)
+    return us
+
+
+# ------------------------------------------------------------------ the other configurations
+def _bits(torch, a, dtype):
+    """numpy float array -> device tensor of the named 16/32-bit type."""
+    t = torch.from_numpy(a.astype("float32"))
+    return t.to({"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[dtype]).cuda()
+
+
+def routing_config(gpu, name, c):
+    """Index generation (with the throttle where the configuration has one), dispatch and combine
+    of one configuration at full size, through the C ABI, over a ring of buffer sets."""
+    import numpy as np
+    import workloads
+
+    torch, L, lib, dev = gpu.torch, gpu.L, gpu._lib, gpu.dev
+    Tn, En, d, k, cap, dtype = c["T"], c["E"], c["d"], c["k"], c["cap"], c["dtype"]
+    es = 4 if dtype == "f32" else 2
+    dt = {"f32": lib.F32, "f16": lib.F16, "bf16": lib.BF16}[dtype]
+    top2 = name.startswith("cfg3")
+    swin = name.startswith("cfg4")
+    bias = workloads.zipf_bias(En, 1.2, seed=c["seed"]) if top2 else None
+    mask_np, logits = workloads.topk_mask(Tn, En, k, seed=c["seed"], bias=bias)
+    x_np = np.random.default_rng(c["seed"]).standard_normal((Tn, d))
+    gates = None
+    if top2:
+        p = workloads.softmax(logits) * mask_np
+        gates = torch.from_numpy((p / p.sum(1, keepdims=True)).astype(np.float32)).cuda()
+    out_dt = lib.F32 if top2 else dt                      # configuration 3 combines into fp32
+    out_es = 4 if top2 else es
+    mpl = cap if swin else 0                              # the Swin glue pads every path to the capacity
+    caps = torch.tensor([cap], dtype=torch.int32, device=dev)
+    thr = torch.full((En,), cap, dtype=torch.int32, device=dev)
+    prefix = torch.zeros(En, dtype=torch.int32, device=dev)
+    ws = torch.empty(max(16, L.brt_hip_scan_workspace_bytes(Tn, En)), dtype=torch.uint8, device=dev)
+    loads_counts = torch.empty(2, En, dtype=torch.int32, device=dev)
+    loads, counts = loads_counts[0], loads_counts[1]
+    mask = torch.from_numpy(mask_np).cuda()
+    x = _bits(torch, x_np, dtype)
+    throttles = top2 or swin
+    routed_mask = torch.empty_like(mask) if throttles else mask
+    idx = torch.empty_like(mask)
+
+    def k_throttle(b, out=None):
+        gpu.check(L.brt_hip_throttle_hotmask(
+            b["mask"].data_ptr(), (b["routed"] if out is None else out).data_ptr(), prefix.data_ptr(),
+            thr.data_ptr(), Tn, En, ws.data_ptr(), ws.numel(), gpu.sptr()))
+
+    def k_indexgen(b):
+        gpu.check(L.brt_hip_generate_indices_and_loads(
+            b["routed"].data_ptr(), b["idx"].data_ptr(), loads.data_ptr(), counts.data_ptr(), Tn, En,
+            None if top2 else caps.data_ptr(), 0 if top2 else 1, int(swin), 0, 0, ws.data_ptr(),
+            ws.numel(), gpu.sptr()))
+
+    first = dict(mask=mask, routed=routed_mask, idx=idx, x=x)
+    if throttles:
+        gpu.run(lambda: k_throttle(first))
+    gpu.run(lambda: k_indexgen(first))
+    loads_h, counts_h = loads.cpu(), counts.cpu()
+    P = En * mpl if mpl else int(loads_h.sum())
+    R = int(torch.minimum(loads_h, counts_h).sum())
+    idx_bytes = 4 * Tn * En
+    n = ring_size(min(Tn, P) * d * es * 2)
+    ring = []
+    for s in range(n):
+        b = first if s == 0 else dict(mask=mask.clone(), routed=routed_mask.clone(), idx=idx.clone(),
+                                      x=x.clone())
+        b["y"] = torch.empty(P, d, dtype=x.dtype, device=dev)
+        b["out"] = torch.empty(Tn, d, dtype=torch.float32 if top2 else x.dtype, device=dev)
+        ring.append(b)
+
+    def k_dispatch(b):
+        gpu.check(L.brt_hip_dispatch(
+            b["x"].data_ptr(), b["y"].data_ptr(), None, b["idx"].data_ptr(), loads.data_ptr(),
+            counts.data_ptr(), None, None, Tn, d, En, P, mpl, 1, 0, dt, gpu.sptr()))
+
+    def k_combine(b):
+        gpu.check(L.brt_hip_combine(
+            b["y"].data_ptr(), b["out"].data_ptr(), None if gates is None else gates.data_ptr(),
+            b["idx"].data_ptr(), loads.data_ptr(), Tn, d, En, P, mpl, 0, dt, out_dt, lib.F32,
+            gpu.sptr()))
+
+    for b in ring:
+        gpu.run(lambda: k_dispatch(b), lambda: k_combine(b))
+    # round trip on the first set: an unweighted combine returns the kept cells (times k)
+    if gates is None:
+        kept = (ring[0]["idx"] > 0) & (ring[0]["idx"] <= loads.view(1, -1))
+        if mpl:
+            kept &= ring[0]["idx"] <= mpl
+        kept = kept.any(1)
+        if not torch.equal(ring[0]["out"][kept], x[kept]) or bool(ring[0]["out"][~kept].any()):
+            sys.exit(f"bench.py: {name}: combine(dispatch(x)) does not return the kept cells")
+    res = {"ring_of_buffer_sets": n, "dispatched_rows": P, "routed_rows": R}
+    gate_bytes = 4 * Tn * En if gates is not None else 0
+    entries = {
+        "indexgen": (lambda b: k_indexgen(b), 2 * idx_bytes + 8 * En),
+        "dispatch": (k_dispatch, R * d * es + P * d * es + idx_bytes),
+        "combine": (k_combine, R * d * es + Tn * d * out_es + idx_bytes + gate_bytes),
+    }
+    if throttles:
+        # timed into a scratch output with the prefix left to run up (the kernel's work does not
+        # depend on it); the throttled masks the other kernels read stay as they are
+        scratch = torch.empty_like(mask)
+        entries["throttle"] = (lambda b: k_throttle(b, scratch), 2 * idx_bytes + 12 * En)
+    for kname, (fn, nbytes) in entries.items():
+        t_us = gpu.launch_us([(lambda b=b: fn(b)) for b in ring], launches=240)
+        res[kname] = {"us": round(t_us, 2), "bytes": nbytes, "GBps": round(nbytes / t_us / 1e3, 1),
+                      "hbm_frac": round(nbytes / t_us / 1e3 / HBM_PEAK_GBPS, 4)}
+    dc_bytes = entries["dispatch"][1] + entries["combine"][1]
+    dc_us = res["dispatch"]["us"] + res["combine"]["us"]
+    res["dispatch_combine_GBps"] = round(dc_bytes / dc_us / 1e3, 1)
+    return res
+
+
+def ffn_config(gpu, loads_np, d, dff, seed, spot_checks=3):
+    """Both grouped GEMMs of an expert FFN over the given ragged loads: d -> dff with GELU, then
+    dff -> d.  Weights ~ N(0, 0.02) drawn on the device.  A few experts are checked against
+    F.linear in fp32 before the launches are timed."""
+    torch, L, lib, dev = gpu.torch, gpu.L, gpu._lib, gpu.dev
+    En, rows = len(loads_np), int(loads_np.sum())
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    x = torch.randn(rows, d, generator=g, device=dev).to(torch.bfloat16)
+    w1 = torch.empty(En, dff, d, dtype=torch.bfloat16, device=dev)
+    w2 = torch.empty(En, d, dff, dtype=torch.bfloat16, device=dev)
+    for e in range(En):
+        w1[e] = (torch.randn(dff, d, generator=g, device=dev) * 0.02).to(torch.bfloat16)
+        w2[e] = (torch.randn(d, dff, generator=g, device=dev) * 0.02).to(torch.bfloat16)
+    t1 = torch.tensor([w1[e].data_ptr() for e in range(En)], dtype=torch.int64, device=dev)
+    t2 = torch.tensor([w2[e].data_ptr() for e in range(En)], dtype=torch.int64, device=dev)
+    loads = torch.from_numpy(loads_np.astype("int32")).cuda()
+    h = torch.empty(rows, dff, dtype=torch.bfloat16, device=dev)
+    y = torch.empty(rows, d, dtype=torch.bfloat16, device=dev)
+
+    def k1():
+        gpu.check(L.brt_hip_grouped_gemm(x.data_ptr(), t1.data_ptr(), None, h.data_ptr(),
+                                         loads.data_ptr(), En, rows, d, dff, lib.ACT_GELU, gpu.sptr()))
+
+    def k2():
+        gpu.check(L.brt_hip_grouped_gemm(h.data_ptr(), t2.data_ptr(), None, y.data_ptr(),
+                                         loads.data_ptr(), En, rows, dff, d, lib.ACT_NONE, gpu.sptr()))
+
+    gpu.run(k1, k2)
+    starts = [0]
+    for m in loads_np.tolist():
+        starts.append(starts[-1] + m)
+    order = sorted(range(En), key=lambda e: -int(loads_np[e]))
+    picks = [order[0], order[len(order) // 2]] + [e for e in order[::-1] if loads_np[e] > 0][:1]
+    for e in picks[:spot_checks]:
+        m = int(loads_np[e])
+        if m == 0:
+            continue
+        rs = slice(starts[e], starts[e] + m)
+        ref1 = torch.nn.functional.gelu(torch.nn.functional.linear(x[rs].float(), w1[e].float()))
+        ref2 = torch.nn.functional.linear(h[rs].float(), w2[e].float())
+        for got, ref in ((h[rs], ref1), (y[rs], ref2)):
+            if float((got.float() - ref).abs().max()) > 1e-2 * float(ref.abs().max()):
+                sys.exit(f"bench.py: grouped GEMM off by more than 1e-2 on expert {e} ({m} rows)")
+    used = int((loads_np > 0).sum())
+    flop = 2.0 * rows * d * dff
+    nbytes = used * d * dff * 2 + rows * d * 2 + rows * dff * 2
+    res = {"rows": rows, "experts": En, "experts_with_rows": used, "largest_load": int(loads_np.max()),
+           "flop_per_gemm": flop, "algorithmic_bytes_per_gemm": nbytes}
+    for name, fn in (("gemm1_gelu", k1), ("gemm2", k2)):
+        launches = 60 if flop < 2e11 else 12
+        t_us = gpu.launch_us(fn, launches=launches)
+        res[name] = {
+            "us": round(t_us, 1), "TFLOPs": round(flop / t_us / 1e6, 1),
+            "mfma_frac": round(flop / t_us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4),
+            "GBps": round(nbytes / t_us / 1e3, 1),
+            "hbm_frac": round(nbytes / t_us / 1e3 / HBM_PEAK_GBPS, 4),
+        }
+    # which roofline bounds this shape: time at the MFMA peak against time at the HBM peak
+    t_mfma, t_hbm = flop / MFMA_BF16_PEAK_TFLOPS / 1e6, nbytes / HBM_PEAK_GBPS / 1e3
+    res["bound"] = "mfma" if t_mfma > t_hbm else "hbm"
+    res["us_at_mfma_peak"], res["us_at_hbm_peak"] = round(t_mfma, 1), round(t_hbm, 1)
+    del w1, w2, x, h, y
+    torch.cuda.empty_cache()
+    return res
+
+
+def phase_configs(gpu):
+    import numpy as np
+    import workloads
+
+    out = {"note": "the other BASELINE configurations at full size, same process, same timing "
+                   "method (graphs of launches over a ring of buffer sets larger than the "
+                   "last-level cache); bytes by the per-kernel formulas of the routing kernels"}
+    for name, c in workloads.ROUTING_CONFIGS.items():
+        out[name] = routing_config(gpu, name, c)
+    loads3 = workloads.top2_skewed_route()[3]
+    out["cfg3_ffn_32e_1024_4096"] = ffn_config(gpu, loads3.astype(np.int64), 1024, 4096, seed=3)
+    loads5 = workloads.dirichlet_loads(32768, 128, 0.3, seed=5)
+    out["cfg5_task_moe_ffn_128e_2048_8192"] = ffn_config(gpu, loads5.astype(np.int64), 2048, 8192, seed=5)
+    # what the same kernel does when the shape lets the matrix units be the bound: the same rows
+    # and feature sizes over 8 experts of 4096 rows (weights 268 MB per GEMM)
+    out["compute_bound_probe_8e_x_4096_rows_2048_8192"] = ffn_config(
+        gpu, np.full(8, 4096, dtype=np.int64), 2048, 8192, seed=6, spot_checks=1)
+    return out
+
+
+def phase_instep(gpu, layer, steps):
+    """Kernel durations inside the step: the same step launched eagerly with an event after every
+    launch.  The two GEMMs keep the GPU busy long enough for the host to stay ahead, so the
+    intervals are kernel time, not launch time; what an event record itself costs is measured in
+    the same run (events recorded back to back) and taken off.  Inputs are what the layer sees:
+    the rows dispatch reads were last touched one step (700 MB of FFN traffic) earlier, the rows
+    combine reads were just written by the second GEMM."""
+    torch = gpu.torch
+    order = [("indexgen", layer.indexgen), ("dispatch", layer.dispatch), ("ffn_gemm1_gelu", layer.gemm1),
+             ("ffn_gemm2", layer.gemm2), ("combine", layer.combine)]
+    n_eager = max(50, min(steps, 200))
+    marks = [[torch.cuda.Event(enable_timing=True) for _ in range(len(order) + 1)] for _ in range(n_eager)]
+    with torch.cuda.stream(gpu.stream):
+        for _ in range(3):
+            layer.step(0)
+        for ev in marks:
+            ev[0].record(gpu.stream)
+            for j, (_, fn) in enumerate(order):
+                fn(0)
+                ev[j + 1].record(gpu.stream)
+        blank = [torch.cuda.Event(enable_timing=True) for _ in range(64)]
+        layer.gemm2(0)                                   # something to queue behind
+        for ev in blank:
+            ev.record(gpu.stream)
+    gpu.stream.synchronize()
+    gaps = sorted(blank[i].elapsed_time(blank[i + 1]) * 1e3 for i in range(8, 63))
+    event_us = gaps[len(gaps) // 2]                      # what an event record itself costs
+    in_step_us = {}
+    for j, (name, _) in enumerate(order):
+        spans = sorted(ev[j].elapsed_time(ev[j + 1]) * 1e3 for ev in marks)
+        in_step_us[name] = max(spans[len(spans) // 2] - event_us, 0.0)
+    return in_step_us, event_us
+
+
+# ------------------------------------------------------------------ extras (reported, not `value`)
+def phase_extras(gpu, layer, steps):
+    torch, L, lib, dev = gpu.torch, gpu.L, gpu._lib, gpu.dev
+    P, R = layer.P, layer.R
+    b0 = layer.sets[0]
+    x, mask = b0["x"], b0["mask"]
+    extras = {}
+    # ---- the layer with dispatch folded into the operand load of the first GEMM and combine into
+    # the result store of the second one (tag-index matrix instead of seat indices)
     tag_idx = torch.zeros_like(mask)
     loads_counts_t = torch.empty(2, E, dtype=torch.int32, device=dev)
     out_fused = x.clone()
     h_fused = torch.empty(P, DFF, dtype=torch.bfloat16, device=dev)
 
     def k_indexgen_tags():
-        _lib.check(L.brt_hip_generate_indices_and_loads(
+        gpu.check(L.brt_hip_generate_indices_and_loads(
             mask.data_ptr(), tag_idx.data_ptr(), loads_counts_t[0].data_ptr(),
-            loads_counts_t[1].data_ptr(), T, E, caps.data_ptr(), 1, 0, 0, 1, ws.data_ptr(),
-            ws.numel(), sptr()))
+            loads_counts_t[1].data_ptr(), T, E, layer.caps.data_ptr(), 1, 0, 0, 1, layer.ws.data_ptr(),
+            layer.ws.numel(), gpu.sptr()))
 
     def k_gemm1_gather():
-        _lib.check(L.brt_hip_grouped_gemm_routed(
-            x.data_ptr(), wi_tab.data_ptr(), None, h_fused.data_ptr(), loads_counts_t[0].data_ptr(),
-            tag_idx.data_ptr(), E, P, T, D, DFF, _lib.ACT_GELU, 1, 0, sptr()))
+        gpu.check(L.brt_hip_grouped_gemm_routed(
+            x.data_ptr(), layer.wi_tab.data_ptr(), None, h_fused.data_ptr(),
+            loads_counts_t[0].data_ptr(), tag_idx.data_ptr(), E, P, T, D, DFF, lib.ACT_GELU, 1, 0,
+            gpu.sptr()))
 
     def k_gemm2_scatter():
-        _lib.check(L.brt_hip_grouped_gemm_routed(
-            h_fused.data_ptr(), wo_tab.data_ptr(), None, out_fused.data_ptr(),
-            loads_counts_t[0].data_ptr(), tag_idx.data_ptr(), E, P, T, DFF, D, _lib.ACT_NONE, 0, 1,
-            sptr()))
+        gpu.check(L.brt_hip_grouped_gemm_routed(
+            h_fused.data_ptr(), layer.wo_tab.data_ptr(), None, out_fused.data_ptr(),
+            loads_counts_t[0].data_ptr(), tag_idx.data_ptr(), E, P, T, DFF, D, lib.ACT_NONE, 0, 1,
+            gpu.sptr()))
 
     def step_fused():
         k_indexgen_tags()
         k_gemm1_gather()
         k_gemm2_scatter()
 
-    def step():
-        k_indexgen()
-        k_dispatch()
-        if have_ffn:
-            k_gemm1()
-            k_gemm2()
-        k_combine()
+    gpu.run(lambda: layer.step(0), step_fused)
+    if not torch.equal(b0["out"].view(torch.int16), out_fused.view(torch.int16)):
+        sys.exit("bench.py: the layer with routing folded into the GEMMs disagrees")
+    g_fused = gpu.capture(step_fused, steps)
+    gpu.timed(g_fused, 1)
+    extras["layer_fused_us"] = round(gpu.timed(g_fused, 1) / steps * 1e3, 2)
+    extras["layer_fused_step"] = ("indexgen(tag indices)+GEMM1 gathering cells+GEMM2 scattering to "
+                                  "cells; K steps in one HIP graph")
 
-    def capture(fn, repeat=1):
-        with torch.cuda.stream(stream):
-            for _ in range(2):
-                fn()
-        stream.synchronize()
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph, stream=stream):
-            for _ in range(repeat):
-                fn()
-        return graph
-
-    def timed(graph, replays):
-        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        with torch.cuda.stream(stream):
-            a.record(stream)
-            for _ in range(replays):
-                graph.replay()
-            b.record(stream)
-        stream.synchronize()
-        return a.elapsed_time(b)  # ms
-
-    # both combine forms must agree bit for bit on this route before anything is timed
-    with torch.cuda.stream(stream):
-        step()
-        k_combine_gather()
-    stream.synchronize()
-    if not torch.equal(out.view(torch.int16), out_gather.view(torch.int16)):
-        sys.exit("bench.py: tag-driven and index-driven combine disagree")
-    if have_ffn:
-        with torch.cuda.stream(stream):
-            step_fused()
-        stream.synchronize()
-        if not torch.equal(out.view(torch.int16), out_fused.view(torch.int16)):
-            sys.exit("bench.py: the layer with routing folded into the GEMMs disagrees")
-
-    # ------------------------------------------------------- timed region: K steps
-    # The K steps are one HIP graph (as the layers of a model would be), launched once, so the
-    # time per step holds no launch gaps between graphs; the warm-up replays a one-step graph.
-    g_step = capture(step)
-    g_steps = capture(step, args.steps)
-    with torch.cuda.stream(stream):
-        for _ in range(args.warmup):
-            g_step.replay()
-    stream.synchronize()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    ms_total = timed(g_steps, 1)
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3
-    ms_per_step = ms_total / args.steps
-    per_graph_launch_us = timed(g_step, args.steps) / args.steps * 1e3  # one graph launch per step
-    fused_layer_us = None
-    if have_ffn:
-        g_fused = capture(step_fused, args.steps)
-        timed(g_fused, 1)
-        fused_layer_us = timed(g_fused, 1) / args.steps * 1e3
-
-    # ------------- kernel durations inside the step (cold inputs, real neighbours): the same step
-    # launched eagerly with an event after every launch.  The two GEMMs keep the GPU busy long
-    # enough for the host to stay ahead, so the intervals are kernel time, not launch time.
-    order = [("indexgen", k_indexgen), ("dispatch", k_dispatch)]
-    if have_ffn:
-        order += [("ffn_gemm1_gelu", k_gemm1), ("ffn_gemm2", k_gemm2)]
-    order.append(("combine", k_combine))
-    n_eager = max(20, min(args.steps, 100))
-    marks = [[torch.cuda.Event(enable_timing=True) for _ in range(len(order) + 1)]
-             for _ in range(n_eager)]
-    with torch.cuda.stream(stream):
-        for _ in range(3):
-            step()
-        for ev in marks:
-            ev[0].record(stream)
-            for j, (_, fn) in enumerate(order):
-                fn()
-                ev[j + 1].record(stream)
-        blank = [torch.cuda.Event(enable_timing=True) for _ in range(64)]
-        k_gemm2() if have_ffn else k_dispatch()       # something to queue behind
-        for ev in blank:
-            ev.record(stream)
-    stream.synchronize()
-    gaps = sorted(blank[i].elapsed_time(blank[i + 1]) * 1e3 for i in range(8, 63))
-    event_us = gaps[len(gaps) // 2]                   # what an event record itself costs
-    in_step_us = {}
-    for j, (name, _) in enumerate(order):
-        spans = sorted(ev[j].elapsed_time(ev[j + 1]) * 1e3 for ev in marks)
-        in_step_us[name] = max(spans[len(spans) // 2] - event_us, 0.0)  # median
-
-    # gate front-end (reported separately, not part of the step): scores -> hot mask
+    # ---- gate front-end: scores -> hot mask
     gate_mask = torch.empty_like(mask)
-    probs_d = probs.to(dev)
+    probs_d = layer.probs.to(dev)
 
     def k_gate():
-        _lib.check(L.brt_hip_topk_hot_mask(probs_d.data_ptr(), gate_mask.data_ptr(), T, E, 1,
-                                           _lib.F32, sptr()))
+        gpu.check(L.brt_hip_topk_hot_mask(probs_d.data_ptr(), gate_mask.data_ptr(), T, E, 1, lib.F32,
+                                          gpu.sptr()))
 
     def k_gate_torch():  # what the reference's TopKProtocol launches
-        torch.zeros_like(probs_d, dtype=torch.int32).scatter_(
-            1, torch.topk(probs_d, 1, dim=1).indices, 1)
+        torch.zeros_like(probs_d, dtype=torch.int32).scatter_(1, torch.topk(probs_d, 1, dim=1).indices, 1)
 
-    with torch.cuda.stream(stream):
-        k_gate()
-    stream.synchronize()
+    gpu.run(k_gate)
     if not torch.equal(gate_mask, mask):
         sys.exit("bench.py: the gate kernel does not reproduce the argmax mask")
 
-    # the same route in the compact format (k path ids per cell instead of the [T,E] mask):
-    # fused softmax + top-1 gate, route from the ids, dispatch by row entries, the same FFN, combine
-    # by the row entries (for one path per cell they are the row tags); reported beside the dense
-    # path and checked against it bit for bit, not part of `value`
-    logits_d = logits.to(dev)
+    # ---- the same route in the compact format (k path ids per cell instead of the [T,E] mask)
+    logits_d = layer.logits.to(dev)
     c_ids = torch.empty(T, 1, dtype=torch.int32, device=dev)
     c_w = torch.empty(T, 1, dtype=torch.float32, device=dev)
     c_loads_counts = torch.empty(2, E, dtype=torch.int32, device=dev)
@@ -314,13 +617,12 @@ def main():
     c_y = torch.empty(P, D, dtype=torch.bfloat16, device=dev)
     c_h = torch.empty(P, DFF, dtype=torch.bfloat16, device=dev)
     c_y2 = torch.empty(P, D, dtype=torch.bfloat16, device=dev)
-    c_out = x.clone()
-    c_out_gather = x.clone()
+    c_out, c_out_gather, c_out_fused = x.clone(), x.clone(), x.clone()
     c_ws = torch.empty(max(4, L.brt_hip_route_by_path_workspace_bytes(T, 1, E)), dtype=torch.uint8, device=dev)
 
     def k_gate_compact():
-        _lib.check(L.brt_hip_gate_topk(logits_d.data_ptr(), T, E, 1, _lib.F32, 1, c_ids.data_ptr(),
-                                       c_w.data_ptr(), None, sptr()))
+        gpu.check(L.brt_hip_gate_topk(logits_d.data_ptr(), T, E, 1, lib.F32, 1, c_ids.data_ptr(),
+                                      c_w.data_ptr(), None, gpu.sptr()))
 
     def k_gate_switch_torch():  # switch_transformer.py:240-253
         p = torch.softmax(logits_d, dim=-1)
@@ -328,92 +630,73 @@ def main():
         torch.max(p, dim=-1)
 
     def k_route_compact():
-        _lib.check(L.brt_hip_route_by_path(
-            c_ids.data_ptr(), T, 1, E, caps.data_ptr(), 1, 0, 0, 0, c_loads_counts[0].data_ptr(),
+        gpu.check(L.brt_hip_route_by_path(
+            c_ids.data_ptr(), T, 1, E, layer.caps.data_ptr(), 1, 0, 0, 0, c_loads_counts[0].data_ptr(),
             c_loads_counts[1].data_ptr(), c_seat_rows.data_ptr(), c_entries.data_ptr(), P,
-            c_ws.data_ptr(), c_ws.numel(), sptr()))
+            c_ws.data_ptr(), c_ws.numel(), gpu.sptr()))
 
     def k_dispatch_rows():
-        _lib.check(L.brt_hip_dispatch_by_rows(x.data_ptr(), c_y.data_ptr(), None, c_entries.data_ptr(),
-                                              P, T, 1, D, _lib.BF16, sptr()))
+        gpu.check(L.brt_hip_dispatch_by_rows(x.data_ptr(), c_y.data_ptr(), None, c_entries.data_ptr(),
+                                             P, T, 1, D, lib.BF16, gpu.sptr()))
 
     def k_combine_rows():
-        _lib.check(L.brt_hip_combine_by_rows(
-            (c_y2 if have_ffn else c_y).data_ptr(), c_out_gather.data_ptr(), None, c_ids.data_ptr(),
-            c_seat_rows.data_ptr(), T, 1, D, P, 1, _lib.BF16, _lib.BF16, sptr()))
+        gpu.check(L.brt_hip_combine_by_rows(
+            c_y2.data_ptr(), c_out_gather.data_ptr(), None, c_ids.data_ptr(), c_seat_rows.data_ptr(),
+            T, 1, D, P, 1, lib.BF16, lib.BF16, gpu.sptr()))
 
     def step_compact():
         k_route_compact()
         k_dispatch_rows()
-        if have_ffn:
-            _lib.check(L.brt_hip_grouped_gemm(
-                c_y.data_ptr(), wi_tab.data_ptr(), None, c_h.data_ptr(), c_loads_counts[0].data_ptr(),
-                E, P, D, DFF, _lib.ACT_GELU, sptr()))
-            _lib.check(L.brt_hip_grouped_gemm(
-                c_h.data_ptr(), wo_tab.data_ptr(), None, c_y2.data_ptr(), c_loads_counts[0].data_ptr(),
-                E, P, DFF, D, _lib.ACT_NONE, sptr()))
-        _lib.check(L.brt_hip_combine_by_tags(
-            (c_y2 if have_ffn else c_y).data_ptr(), c_out.data_ptr(), c_entries.data_ptr(), P, D, T,
-            _lib.BF16, _lib.BF16, sptr()))
-
-    # ... and with dispatch and combine folded into the GEMMs as well (rows named by the entries)
-    c_out_fused = x.clone()
+        gpu.check(L.brt_hip_grouped_gemm(
+            c_y.data_ptr(), layer.wi_tab.data_ptr(), None, c_h.data_ptr(), c_loads_counts[0].data_ptr(),
+            E, P, D, DFF, lib.ACT_GELU, gpu.sptr()))
+        gpu.check(L.brt_hip_grouped_gemm(
+            c_h.data_ptr(), layer.wo_tab.data_ptr(), None, c_y2.data_ptr(), c_loads_counts[0].data_ptr(),
+            E, P, DFF, D, lib.ACT_NONE, gpu.sptr()))
+        gpu.check(L.brt_hip_combine_by_tags(
+            c_y2.data_ptr(), c_out.data_ptr(), c_entries.data_ptr(), P, D, T, lib.BF16, lib.BF16,
+            gpu.sptr()))
 
     def step_compact_fused():
         k_route_compact()
-        _lib.check(L.brt_hip_grouped_gemm_by_rows(
-            x.data_ptr(), wi_tab.data_ptr(), None, c_h.data_ptr(), c_loads_counts[0].data_ptr(),
-            c_entries.data_ptr(), 1, E, P, T, D, DFF, _lib.ACT_GELU, 1, 0, sptr()))
-        _lib.check(L.brt_hip_grouped_gemm_by_rows(
-            c_h.data_ptr(), wo_tab.data_ptr(), None, c_out_fused.data_ptr(),
-            c_loads_counts[0].data_ptr(), c_entries.data_ptr(), 1, E, P, T, DFF, D, _lib.ACT_NONE,
-            0, 1, sptr()))
+        gpu.check(L.brt_hip_grouped_gemm_by_rows(
+            x.data_ptr(), layer.wi_tab.data_ptr(), None, c_h.data_ptr(), c_loads_counts[0].data_ptr(),
+            c_entries.data_ptr(), 1, E, P, T, D, DFF, lib.ACT_GELU, 1, 0, gpu.sptr()))
+        gpu.check(L.brt_hip_grouped_gemm_by_rows(
+            c_h.data_ptr(), layer.wo_tab.data_ptr(), None, c_out_fused.data_ptr(),
+            c_loads_counts[0].data_ptr(), c_entries.data_ptr(), 1, E, P, T, DFF, D, lib.ACT_NONE, 0, 1,
+            gpu.sptr()))
 
-    with torch.cuda.stream(stream):
-        k_gate_compact()
-        step_compact()
-        k_combine_rows()
-        if have_ffn:
-            step_compact_fused()
-    stream.synchronize()
-    if have_ffn and not torch.equal(c_out_fused.view(torch.int16), out.view(torch.int16)):
+    gpu.run(k_gate_compact, step_compact, k_combine_rows, step_compact_fused)
+    out_bits = b0["out"].view(torch.int16)
+    if not torch.equal(c_out_fused.view(torch.int16), out_bits):
         sys.exit("bench.py: the compact layer with routing folded into the GEMMs disagrees")
-    if not torch.equal(c_ids.view(-1).long(), expert.to(dev)):
+    if not torch.equal(c_ids.view(-1).long(), layer.expert.to(dev)):
         sys.exit("bench.py: the compact gate does not reproduce the argmax")
-    if not torch.allclose(c_w.view(-1).cpu(), probs.max(dim=1).values, rtol=2e-6, atol=0):
+    if not torch.allclose(c_w.view(-1).cpu(), layer.probs.max(dim=1).values, rtol=2e-6, atol=0):
         sys.exit("bench.py: the compact gate's softmax weight is off")
-    if not (torch.equal(c_out.view(torch.int16), out.view(torch.int16))
-            and torch.equal(c_out_gather.view(torch.int16), out.view(torch.int16))
-            and torch.equal(c_loads_counts, loads_counts)):
+    if not (torch.equal(c_out.view(torch.int16), out_bits)
+            and torch.equal(c_out_gather.view(torch.int16), out_bits)
+            and torch.equal(c_loads_counts, layer.loads_counts)):
         sys.exit("bench.py: the layer on the compact route disagrees with the dense one")
-    g_compact = capture(step_compact, args.steps)
-    timed(g_compact, 1)
-    compact_layer_us = timed(g_compact, 1) / args.steps * 1e3
-    compact_fused_layer_us = None
-    if have_ffn:
-        g_compact_fused = capture(step_compact_fused, args.steps)
-        timed(g_compact_fused, 1)
-        compact_fused_layer_us = timed(g_compact_fused, 1) / args.steps * 1e3
+    for key, fn, what in (
+            ("layer_compact", step_compact,
+             "route from path ids+dispatch by rows+ffn+combine by row tags"),
+            ("layer_compact_fused", step_compact_fused,
+             "route from path ids+GEMM1 gathering cells+GEMM2 scattering to cells, rows named by the row entries")):
+        gk = gpu.capture(fn, steps)
+        gpu.timed(gk, 1)
+        extras[key + "_us"] = round(gpu.timed(gk, 1) / steps * 1e3, 2)
+        extras[key + "_step"] = what + "; K steps in one HIP graph"
 
-    # the library's batched GEMM on the same FFN, every expert padded to the full capacity (the
-    # only shape a batched routine takes), GELU as its own elementwise launch: reported beside
-    # the grouped kernel, not part of the step
+    # ---- the library's batched GEMM on the same FFN, every expert padded to the full capacity
+    # (the only shape a batched routine takes), GELU as its own elementwise launch
     xb = torch.randn(E, CAPACITY, D, device=dev).to(torch.bfloat16)
     hb = torch.empty(E, CAPACITY, DFF, dtype=torch.bfloat16, device=dev)
     yb = torch.empty(E, CAPACITY, D, dtype=torch.bfloat16, device=dev)
 
-    def k_bmm1():
-        torch.bmm(xb, wi.transpose(1, 2), out=hb)
-
-    def k_bmm_gelu():
-        torch.nn.functional.gelu(hb)
-
-    def k_bmm2():
-        torch.bmm(hb, wo.transpose(1, 2), out=yb)
-
-    # generic tag-index gather (the default gather path of the reference: unique over the row
-    # tags, then a sum of the rows that carry the same tag) on this step's rows and tags,
-    # beside the library calls the reference makes for it; reported only, not part of the step
+    # ---- generic tag-index gather (the default gather path of the reference) on this step's rows
+    row_tags, combine_src = b0["row_tags"], b0["y2"]
     n_unique_d = torch.empty(1, dtype=torch.int32, device=dev)
     uniq = torch.empty(P, dtype=torch.int32, device=dev)
     inverse = torch.empty(P, dtype=torch.int64, device=dev)
@@ -422,208 +705,225 @@ def main():
     gathered = torch.empty(P, D, dtype=torch.bfloat16, device=dev)
 
     def k_tag_unique():
-        _lib.check(L.brt_hip_unique_tags(row_tags.data_ptr(), 32, P, 0, T, ws_u.data_ptr(),
-                                         ws_u.numel(), uniq.data_ptr(), inverse.data_ptr(),
-                                         n_unique_d.data_ptr(), sptr()))
+        gpu.check(L.brt_hip_unique_tags(row_tags.data_ptr(), 32, P, 0, T, ws_u.data_ptr(), ws_u.numel(),
+                                        uniq.data_ptr(), inverse.data_ptr(), n_unique_d.data_ptr(),
+                                        gpu.sptr()))
 
     def k_tag_sum():
-        _lib.check(L.brt_hip_combine_by_index(
+        gpu.check(L.brt_hip_combine_by_index(
             combine_src.data_ptr(), gathered.data_ptr(), inverse.data_ptr(), 64, P, D, P,
-            ws_s.data_ptr(), ws_s.numel(), _lib.BF16, _lib.BF16, sptr()))
+            ws_s.data_ptr(), ws_s.numel(), lib.BF16, lib.BF16, gpu.sptr()))
 
     def k_tag_sum_torch():   # router.cc:451,459-460
         torch.zeros(P, D, dtype=torch.bfloat16, device=dev).scatter_reduce(
             0, inverse.view(-1, 1).repeat(1, D), combine_src, "sum")
 
-    with torch.cuda.stream(stream):
+    with torch.cuda.stream(gpu.stream):
         k_tag_unique()
         k_tag_sum()
         t_u, t_i = torch.unique(row_tags, sorted=True, return_inverse=True)
-    stream.synchronize()
+    gpu.stream.synchronize()
     n_u = int(n_unique_d.item())
     if n_u != t_u.numel() or not torch.equal(uniq[:n_u], t_u) or not torch.equal(inverse, t_i):
         sys.exit("bench.py: the tag unique kernels disagree with torch.unique")
-    # every tag is carried by one row here, so the sum is the rows in tag order
     if not torch.equal(gathered[inverse].view(torch.int16), combine_src.view(torch.int16)):
         sys.exit("bench.py: the tag-index sum does not reproduce the rows")
-    with torch.cuda.stream(stream):      # torch.unique synchronises: timed eagerly
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        for _ in range(3):
-            torch.unique(row_tags, sorted=True, return_inverse=True)
-        e0.record(stream)
-        for _ in range(20):
-            torch.unique(row_tags, sorted=True, return_inverse=True)
-        e1.record(stream)
-    stream.synchronize()
-    unique_torch_us = e0.elapsed_time(e1) * 1e3 / 20
 
-    # a plain device-to-device copy of as many rows as dispatch moves: what the same traffic
-    # costs without any routing, at this size
-    def k_copy_rows():
-        y.copy_(x[:P])
-
-    # ---------------------------------------- per-kernel durations (same process)
-    INNER = 20
-    kernels = {"indexgen": k_indexgen, "dispatch": k_dispatch, "combine": k_combine,
-               "combine_gather": k_combine_gather, "gate_topk_mask": k_gate,
-               "gate_topk_mask_torch_ops": k_gate_torch,
-               "tag_gather_unique": k_tag_unique, "tag_gather_sum": k_tag_sum,
-               "tag_gather_sum_torch_ops": k_tag_sum_torch, "plain_copy_of_the_rows": k_copy_rows,
-               "compact_gate_softmax_top1": k_gate_compact,
-               "compact_gate_switch_torch_ops": k_gate_switch_torch,
-               "compact_route_by_path": k_route_compact, "compact_dispatch_by_rows": k_dispatch_rows,
-               "compact_combine_by_rows": k_combine_rows}
-    if have_ffn:
-        kernels.update({"ffn_gemm1_gelu": k_gemm1, "ffn_gemm2": k_gemm2,
-                        "indexgen_tags": k_indexgen_tags, "ffn_gemm1_gelu_gather": k_gemm1_gather,
-                        "ffn_gemm2_scatter": k_gemm2_scatter,
-                        "ffn_gemm1_library_bmm": k_bmm1, "ffn_gelu_library": k_bmm_gelu,
-                        "ffn_gemm2_library_bmm": k_bmm2})
-    replays = max(10, args.steps // 4)
-    us = {}
+    kernels = {
+        "gate_topk_mask": k_gate, "gate_topk_mask_torch_ops": k_gate_torch,
+        "compact_gate_softmax_top1": k_gate_compact, "compact_gate_switch_torch_ops": k_gate_switch_torch,
+        "compact_route_by_path": k_route_compact, "compact_dispatch_by_rows": k_dispatch_rows,
+        "compact_combine_by_rows": k_combine_rows, "indexgen_tags": k_indexgen_tags,
+        "ffn_gemm1_gelu_gather": k_gemm1_gather, "ffn_gemm2_scatter": k_gemm2_scatter,
+        "tag_gather_unique": k_tag_unique, "tag_gather_sum": k_tag_sum,
+        "tag_gather_sum_torch_ops": k_tag_sum_torch,
+        "plain_copy_of_the_rows": lambda: b0["y"].copy_(x[:P]),
+        "ffn_gemm1_library_bmm": lambda: torch.bmm(xb, layer.wi.transpose(1, 2), out=hb),
+        "ffn_gelu_library": lambda: torch.nn.functional.gelu(hb),
+        "ffn_gemm2_library_bmm": lambda: torch.bmm(hb, layer.wo.transpose(1, 2), out=yb),
+    }
+    es, idx_bytes = 2, 4 * T * E
+    kbytes = {
+        "gate_topk_mask": 2 * idx_bytes, "indexgen_tags": 2 * idx_bytes + 8 * E,
+        "plain_copy_of_the_rows": 2 * min(P, T) * D * es,
+        "compact_gate_softmax_top1": idx_bytes + 8 * T,
+        "compact_route_by_path": 2 * 4 * T + 4 * T + 4 * P + 8 * E,
+        "compact_dispatch_by_rows": R * D * es + P * D * es + 4 * P,
+        "compact_combine_by_rows": R * D * es + T * D * es + 8 * T,
+        "tag_gather_sum": 2 * P * D * es + 8 * P + 4 * (2 * P),
+    }
+    per = {}
     for name, fn in kernels.items():
-        gk = capture(fn, INNER)
-        timed(gk, 3)
-        runs = [timed(gk, replays) for _ in range(3)]
-        us[name] = sum(runs) / len(runs) * 1e3 / (replays * INNER)  # average launch duration
+        launches = 60 if "ffn" in name else 200
+        t_us = gpu.launch_us(fn, launches=launches)
+        per[name] = {"us": round(t_us, 3)}
+        if name in kbytes:
+            per[name]["GBps"] = round(kbytes[name] / t_us / 1e3, 1)
+    extras["kernels_back_to_back_one_buffer_set"] = per
+    return extras
 
-    us["tag_gather_unique_torch_op_eager"] = unique_torch_us
-    es = 2  # bf16
-    idx_bytes = 4 * T * E
-    bytes_ = {
-        "indexgen": 2 * idx_bytes + 4 * E,
-        "dispatch": R * D * es + P * D * es + idx_bytes,
-        "combine": R * D * es + T * D * es + idx_bytes,
-        "combine_gather": R * D * es + T * D * es + idx_bytes,
-    }
-    # what the kernels have to touch: the tag-driven combine reads 4 bytes of tag per row
-    # instead of the [T,E] index matrix, dispatch writes those tags
-    moved = {
-        "dispatch": bytes_["dispatch"] + 4 * P,
-        "combine": 2 * R * D * es + 4 * P,
-    }
-    flops = {"ffn_gemm1_gelu": 2.0 * R * D * DFF, "ffn_gemm2": 2.0 * R * DFF * D}
-    flops["ffn_gemm1_gelu_gather"] = flops["ffn_gemm1_gelu"]
-    flops["ffn_gemm2_scatter"] = flops["ffn_gemm2"]
-    bytes_["indexgen_tags"] = bytes_["indexgen"]
-    bytes_["gate_topk_mask"] = 2 * idx_bytes  # fp32 scores in, int32 mask out
-    bytes_["plain_copy_of_the_rows"] = 2 * min(P, T) * D * es
-    bytes_["compact_gate_softmax_top1"] = idx_bytes + 8 * T          # fp32 scores in, id + weight out
-    bytes_["compact_route_by_path"] = 2 * 4 * T + 4 * T + 4 * P + 8 * E  # ids twice, seat rows, entries
-    bytes_["compact_dispatch_by_rows"] = R * D * es + P * D * es + 4 * P
-    bytes_["compact_combine_by_rows"] = R * D * es + T * D * es + 8 * T
-    bytes_["tag_gather_sum"] = 2 * P * D * es + 8 * P + 4 * (2 * P)  # rows in/out, index, lists
-    dc_bytes = bytes_["dispatch"] + bytes_["combine"]
-    dc_us = us["dispatch"] + us["combine"]
-    value = dc_bytes / dc_us / 1e3  # GB/s
 
-    dominant = "combine" if us["combine"] >= us["dispatch"] else "dispatch"
-    roofline = {
-        "kernel": dominant,
-        "bound": "hbm",
-        "achieved": round(bytes_[dominant] / us[dominant] / 1e3, 1),
-        "peak": HBM_PEAK_GBPS,
+def cpu_baseline(layer):
+    import numpy as np
+    import torch
+    from oracle import torch_path
+
+    cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    torch.set_num_threads(cores)
+    x32, mask_h = layer.x32, layer.mask_h
+    m_idx, m_loads = torch_path.generate_indices_and_loads(mask_h, [CAPACITY], False)
+    for _ in range(3):
+        yy = torch_path.dispatch(x32, m_idx, m_loads)
+        torch_path.combine(yy, m_idx, m_loads, None, x32)
+    reps, spent, t_dc = 0, 0.0, []
+    while (spent < 10.0 and reps < 2000) or reps < 5:
+        t1 = time.perf_counter()
+        yy = torch_path.dispatch(x32, m_idx, m_loads)
+        torch_path.combine(yy, m_idx, m_loads, None, x32)
+        dt = time.perf_counter() - t1
+        t_dc.append(dt)
+        spent += dt
+        reps += 1
+    med = float(np.median(t_dc))
+    P, R = layer.P, layer.R
+    cpu_bytes = 2 * R * D * 4 + P * D * 4 + T * D * 4 + 2 * 4 * T * E  # same ops in fp32
+    return {
+        "value": round(cpu_bytes / med / 1e9, 2),
         "unit": "GB/s",
-        "frac": round(bytes_[dominant] / us[dominant] / 1e3 / HBM_PEAK_GBPS, 4),
-        "traffic": MEASURED_TRAFFIC_BYTES.get(dominant),
-        "avg_us": round(us[dominant], 3),
-        "algorithmic_bytes": bytes_[dominant],
-        "bytes_the_kernel_must_move": moved[dominant],
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": (f"{reps} passes of torch CPU dispatch+combine (index_select / index_add_, fp32) on "
+                   f"the same {T}x{D} x {E}-expert inputs, median {med * 1e3:.2f} ms"),
     }
-    per_kernel = {}
-    for name in us:
-        entry = {"us": round(us[name], 3)}
-        if name in bytes_:
-            entry["GBps"] = round(bytes_[name] / us[name] / 1e3, 1)
-            entry["hbm_frac"] = round(bytes_[name] / us[name] / 1e3 / HBM_PEAK_GBPS, 4)
-        if name in flops:
-            entry["TFLOPs"] = round(flops[name] / us[name] / 1e6, 1)
-            entry["mfma_frac"] = round(flops[name] / us[name] / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4)
-            # the expert FFN at 128 rows per expert streams its weights: HBM is the bound
-            hbm = MEASURED_TRAFFIC_BYTES.get(name.replace("_gather", "").replace("_scatter", ""))
-            entry["hbm_GBps"] = round(hbm / us[name] / 1e3, 1)
-            entry["hbm_frac"] = round(hbm / us[name] / 1e3 / HBM_PEAK_GBPS, 4)
-        per_kernel[name] = entry
 
-    # ------------------------------------------------------------ CPU baseline
-    cpu_baseline = None
-    if not args.no_cpu_baseline:
-        from oracle import torch_path
 
-        cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
-        torch.set_num_threads(cores)
-        m_idx, m_loads = torch_path.generate_indices_and_loads(mask_h, [CAPACITY], False)
-        for _ in range(3):
-            yy = torch_path.dispatch(x32, m_idx, m_loads)
-            torch_path.combine(yy, m_idx, m_loads, None, x32)
-        reps, spent = 0, 0.0
-        t_dc = []
-        while (spent < 10.0 and reps < 2000) or reps < 5:
-            t1 = time.perf_counter()
-            yy = torch_path.dispatch(x32, m_idx, m_loads)
-            torch_path.combine(yy, m_idx, m_loads, None, x32)
-            dt = time.perf_counter() - t1
-            t_dc.append(dt)
-            spent += dt
-            reps += 1
-        med = float(np.median(t_dc))
-        cpu_bytes = 2 * R * D * 4 + P * D * 4 + T * D * 4 + 2 * idx_bytes  # same ops in fp32
-        cpu_baseline = {
-            "value": round(cpu_bytes / med / 1e9, 2),
-            "unit": "GB/s",
-            "cores": torch.get_num_threads(),
-            "kind": "port",
-            "sample": (f"{reps} passes of torch CPU dispatch+combine (index_select / index_add_, "
-                       f"fp32) on the same {T}x{D} x {E}-expert inputs, median {med * 1e3:.2f} ms"),
-        }
+def main():
+    args = parse()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: the routing hot path is built and measured on a "
+                 "single MI355X (no collectives in this build); run with --gpus 1")
+    import torch
+
+    from brainstorm_amd import _lib
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    gpu = Gpu(torch, _lib)
+    only = args.only
+    want = lambda phase: only in ("all", phase)  # noqa: E731
+
+    launch_bytes = 2 * T * D * 2                     # what the leanest row kernel touches per launch
+    sets = ring_size(launch_bytes) if want("cold") else 1
+    index_sets = ring_size(2 * 4 * T * E, most=192) if want("cold") else 1
+    layer = SwitchLayer(gpu, sets, index_sets)
+    check_switch_layer(gpu, layer)
+    nbytes, flops = layer.bytes(), layer.flops()
+    traffic, traffic_commit = measured_traffic()
 
     result = {
-        "metric": "dispatch+combine GB/s",
-        "value": round(value, 1),
-        "unit": "GB/s",
-        "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 5),
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": "bf16",
-        "data": "synthetic",
+        "metric": "dispatch+combine GB/s", "value": None, "unit": "GB/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": None, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {
             "workload": "Switch-MoE layer routing hot path (BASELINE.json configs[1])",
             "tokens": T, "d_model": D, "experts": E, "d_ff": DFF, "top_k": 1,
             "capacity": CAPACITY, "capacity_mode": "clip (overflow dropped, no padding)",
-            "routed_rows": R, "dispatched_rows": P, "seed": SEED,
-            "step": "indexgen+dispatch+" + ("ffn(2 grouped GEMMs)+" if have_ffn else "") + "combine; the K steps are one HIP graph",
+            "routed_rows": layer.R, "dispatched_rows": layer.P, "seed": SEED,
+            "step": "indexgen+dispatch+ffn(2 grouped GEMMs)+combine; the K steps are one HIP graph",
         },
-        "hbm_peak_frac": round(value / HBM_PEAK_GBPS, 4),
-        "in_step": {
-            "note": "medians of event-to-event intervals of the same step launched eagerly, minus "
-                    "the interval of two adjacent event records: inputs come from HBM after the "
-                    "FFN has swept the caches, unlike the back-to-back launches on one set of "
-                    "buffers that `kernels` and `value` are measured on",
-            "event_record_us": round(event_us, 2),
-            "us": {k: round(v, 2) for k, v in in_step_us.items()},
-            "dispatch_combine_GBps": round(dc_bytes / (in_step_us["dispatch"] + in_step_us["combine"]) / 1e3, 1),
-        },
-        "layer_us": round(ms_per_step * 1e3, 2),
-        "layer_us_one_graph_launch_per_step": round(per_graph_launch_us, 2),
-        "layer_compact_us": round(compact_layer_us, 2),
-        "layer_compact_step": "route from path ids+dispatch by rows+ffn+combine by row tags; K steps in one HIP graph",
-        "layer_compact_fused_us": None if compact_fused_layer_us is None else round(compact_fused_layer_us, 2),
-        "layer_compact_fused_step": "route from path ids+GEMM1 gathering cells+GEMM2 scattering to cells, rows named by the row entries; K steps in one HIP graph",
-        "layer_fused_us": None if fused_layer_us is None else round(fused_layer_us, 2),
-        "layer_fused_step": "indexgen(tag indices)+GEMM1 gathering cells+GEMM2 scattering to cells; K steps in one HIP graph",
-        "wall_ms_timed_region": round(wall_ms, 3),
-        "algorithmic_bytes_dispatch_combine": dc_bytes,
-        "kernels": per_kernel,
-        "roofline": roofline,
-        "cpu_baseline": cpu_baseline,
+        "phases_run": only,
     }
-    if not have_ffn:
-        result["ffn"] = None
-        result["ffn_note"] = ffn_note
+
+    if want("step"):
+        st = phase_step(gpu, layer, args.steps, args.warmup)
+        result["ms_per_step"] = round(st["ms_per_step"], 5)
+        result["layer_us"] = round(st["ms_per_step"] * 1e3, 2)
+        result["layer_us_one_graph_launch_per_step"] = round(st["layer_us_one_graph_launch_per_step"], 2)
+        result["wall_ms_timed_region"] = round(st["wall_ms"], 3)
+
+    def per_kernel(us):
+        out = {}
+        for name, t_us in us.items():
+            entry = {"us": round(t_us, 3), "bytes": nbytes[name],
+                     "GBps": round(nbytes[name] / t_us / 1e3, 1),
+                     "hbm_frac": round(nbytes[name] / t_us / 1e3 / HBM_PEAK_GBPS, 4)}
+            if name in flops:
+                entry["TFLOPs"] = round(flops[name] / t_us / 1e6, 1)
+                entry["mfma_frac"] = round(flops[name] / t_us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4)
+            out[name] = entry
+        return out
+
+    if want("instep"):
+        us, event_us = phase_instep(gpu, layer, args.steps)
+        dc_bytes = nbytes["dispatch"] + nbytes["combine"]
+        value = dc_bytes / (us["dispatch"] + us["combine"]) / 1e3
+        result["value"] = round(value, 1)
+        result["hbm_peak_frac"] = round(value / HBM_PEAK_GBPS, 4)
+        result["value_is"] = (
+            f"(bytes dispatch and the tag-driven combine have to move = {dc_bytes}) / (sum of their "
+            "durations inside the step: medians of event-to-event intervals of the eagerly launched "
+            "step minus the cost of an event record).  Inputs are as the layer leaves them: not the "
+            "cache-resident buffers of back-to-back launches (dispatch_combine_warm_GBps), not the "
+            "never-touched ones of the ring (dispatch_combine_cold_ring_GBps)")
+        result["in_step"] = {"event_record_us": round(event_us, 2), "kernels": per_kernel(us)}
+        dominant = "combine" if us["combine"] >= us["dispatch"] else "dispatch"
+        result["roofline"] = {
+            "kernel": dominant, "bound": "hbm",
+            "achieved": round(nbytes[dominant] / us[dominant] / 1e3, 1), "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s", "frac": round(nbytes[dominant] / us[dominant] / 1e3 / HBM_PEAK_GBPS, 4),
+            "traffic": traffic.get(dominant), "traffic_taken_at_commit": traffic_commit,
+            "avg_us": round(us[dominant], 3), "algorithmic_bytes": nbytes[dominant],
+            "launches": "inside the step (bench.py --only instep runs nothing else)",
+        }
+
+    if want("cold"):
+        us = phase_routing(gpu, layer, sets, index_sets)
+        b0 = layer.sets
+        us_copy = gpu.launch_us([(lambda s=s: b0[s]["y"].copy_(b0[s]["x"][:layer.P])) for s in range(sets)])
+        result["kernels_cold_ring"] = per_kernel(us)
+        result["kernels_cold_ring"]["plain_copy_of_the_rows"] = {
+            "us": round(us_copy, 3), "bytes": 2 * layer.P * D * 2,
+            "GBps": round(2 * layer.P * D * 2 / us_copy / 1e3, 1)}
+        result["cold_ring"] = (f"ring of {sets} buffer sets ({index_sets} for index generation): a kernel has "
+                               f"touched {RING_BYTES >> 20} MiB before it sees a set again, so every launch reads "
+                               "from HBM; the runtime's device-to-device copy of the same rows is timed the same way")
+        result["dispatch_combine_cold_ring_GBps"] = round(
+            (nbytes["dispatch"] + nbytes["combine"]) / (us["dispatch"] + us["combine"]) / 1e3, 1)
+        result["dispatch_combine_index_driven_cold_ring_GBps"] = round(
+            (nbytes["dispatch"] + nbytes["combine_gather"]) / (us["dispatch"] + us["combine_gather"]) / 1e3, 1)
+
+    if want("warm"):
+        us = phase_routing(gpu, layer, 1, 1)
+        result["kernels_warm_one_buffer_set"] = per_kernel(us)
+        result["dispatch_combine_warm_GBps"] = round(
+            (nbytes["dispatch"] + nbytes["combine"]) / (us["dispatch"] + us["combine"]) / 1e3, 1)
+
+    if want("ffn"):
+        us = phase_ffn(gpu, layer)
+        result["kernels_ffn"] = per_kernel(us)
+        name = "ffn_gemm1_gelu" if us["ffn_gemm1_gelu"] >= us["ffn_gemm2"] else "ffn_gemm2"
+        t_mfma = flops[name] / MFMA_BF16_PEAK_TFLOPS / 1e6
+        t_hbm = nbytes[name] / HBM_PEAK_GBPS / 1e3
+        result["roofline_ffn"] = {
+            "kernel": name + " (grouped_gemm_kernel, the longest kernel of the step)",
+            "bound": "hbm" if t_hbm >= t_mfma else "mfma",
+            "achieved": round(nbytes[name] / us[name] / 1e3, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+            "frac": round(nbytes[name] / us[name] / 1e3 / HBM_PEAK_GBPS, 4),
+            "mfma_frac": round(flops[name] / us[name] / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4),
+            "us_at_hbm_peak": round(t_hbm, 1), "us_at_mfma_peak": round(t_mfma, 1),
+            "traffic": traffic.get(name), "traffic_taken_at_commit": traffic_commit,
+            "avg_us": round(us[name], 3), "algorithmic_bytes": nbytes[name], "flop": flops[name],
+        }
+
+    if want("configs"):
+        result["configs"] = phase_configs(gpu)
+
+    if want("extras"):
+        result.update(phase_extras(gpu, layer, args.steps))
+
+    result["cpu_baseline"] = None
+    if only == "all" and not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(layer)
     print(json.dumps(result))
 
 

@@ -35,6 +35,7 @@
 #include <type_traits>
 
 #include "common.hpp"
+#include "grouped_gemm.hpp"
 #include "rows.hpp"
 
 namespace brt {
@@ -55,48 +56,6 @@ constexpr int kBK = 64;               // k elements per stage
 constexpr int kChunks = kBK / 8;      // 16-byte chunks per tile row
 constexpr int kRowBytes = kBK * 2;    // LDS row (swizzled, unpadded)
 constexpr int kXcds = 8;
-
-struct GemmArgs {
-  const __bf16* x;
-  const __bf16* const* w;
-  const __bf16* const* bias;
-  __bf16* out;
-  const int* loads;
-  const int* tags;  // [T,E] tag matrix (column e: 1-based cells of path e in seat order), or the
-                    // row-entry vector [P] of the compact route (1-based entry t*k+j+1 per row), or null
-  int tag_vector;   // tags is the row-entry vector
-  int tag_div;      // entries per cell (k) of the row-entry vector
-  int E, P, K, N, T;
-  int gather, scatter;  // rows of x / of out are addressed through the tags
-  int tiles_n, tiles_m_max;
-  int walk, groups_n;  // column tiles one workgroup walks, ceil(tiles_n / walk)
-};
-
-// GELU(v) = v * Phi(v) = max(v, 0) - |v| * Phi(-|v|), branch free.  The tail probability is
-// exp2(Q(|v|)) with Q a degree-7 fit of log2 Phi(-x) on [0, 8] (|Q - log2 Phi| < 5e-5 there, so the
-// tail is good to 3.5e-5 relative; beyond 8 the product is below 5e-15 and Q keeps falling to -inf).
-// Against the erf form in double the result is within 4.3e-6 absolute everywhere, two orders below
-// half a bf16 step at the values where that bound is reached.  The clamp keeps +-inf inputs from
-// turning inf * 0 into NaN.  Cost per element: seven multiply-adds, one exp2, min, max, one more fma.
-__device__ __forceinline__ float gelu_erf(float v) {
-  const float av = fminf(fabsf(v), 1e30f);
-  float q = -1.262479145e-06f;
-  q = __builtin_fmaf(q, av, 4.820351751e-05f);
-  q = __builtin_fmaf(q, av, -8.072460769e-04f);
-  q = __builtin_fmaf(q, av, 7.944535464e-03f);
-  q = __builtin_fmaf(q, av, -5.263513327e-02f);
-  q = __builtin_fmaf(q, av, -4.599574506e-01f);
-  q = __builtin_fmaf(q, av, -1.150609374e+00f);
-  q = __builtin_fmaf(q, av, -1.000043273e+00f);
-  return __builtin_fmaf(-av, __builtin_amdgcn_exp2f(q), fmaxf(v, 0.0f));
-}
-
-template <int ACT>
-__device__ __forceinline__ float apply_act(float v) {
-  if (ACT == BRT_ACT_GELU) return gelu_erf(v);
-  if (ACT == BRT_ACT_RELU) return fmaxf(v, 0.0f);
-  return v;
-}
 
 // Cache policy of the weight loads (auxiliary operand of the buffer load: bit 1 = non-temporal on
 // gfx94x/gfx950).  Every weight byte is read exactly once per launch; loaded as a stream it does
@@ -621,6 +580,7 @@ int grouped_gemm_impl(const void* x, const void* const* weights, const void* con
   a.tag_div = entries_per_cell;
   a.E = E; a.P = P; a.K = K; a.N = N; a.T = T;
   a.gather = gather_in != 0; a.scatter = scatter_out != 0;
+  if (wide_gemm_applies(a)) return launch_wide_gemm(a, act, as_stream(stream));
   // Tile choice.  A wavefront owns 160 x 64 outputs (7 LDS fragment reads feed 10 MFMAs); a
   // workgroup is 2, 3 or 4 of them side by side.  The kernel is bound by how fast a CU can fill
   // its L1 (about 29 KB/us, L2 hits included), so the shape is the one that gives the busiest CU

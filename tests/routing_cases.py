@@ -7,35 +7,12 @@ oracle finishes in seconds.
 import numpy as np
 
 
-def topk_mask(T, E, k, seed, bias=None):
-    """int32 [T,E] hot mask with exactly k ones per row (top-k of N(0,1) logits)."""
-    rng = np.random.default_rng(seed)
-    logits = rng.standard_normal((T, E)).astype(np.float32)
-    if bias is not None:
-        logits = logits + bias.astype(np.float32)[None, :]
-    top = np.argsort(-logits, axis=1, kind="stable")[:, :k]
-    mask = np.zeros((T, E), dtype=np.int32)
-    np.put_along_axis(mask, top, 1, axis=1)
-    return mask, logits
+from workloads import softmax, topk_mask, zipf_bias  # noqa: F401  (re-exported)
 
 
 def bernoulli_mask(T, E, p, seed):
     rng = np.random.default_rng(seed)
     return (rng.random((T, E)) < p).astype(np.int32)
-
-
-def zipf_bias(E, s, seed):
-    """log of a Zipf(s) pmf over a seeded permutation of the experts."""
-    rng = np.random.default_rng(seed)
-    pmf = 1.0 / np.arange(1, E + 1) ** s
-    pmf /= pmf.sum()
-    return np.log(pmf)[rng.permutation(E)]
-
-
-def softmax(x):
-    x = x - x.max(axis=1, keepdims=True)
-    e = np.exp(x)
-    return e / e.sum(axis=1, keepdims=True)
 
 
 def to_bf16_bits(x):

@@ -109,6 +109,68 @@ def test_ragged_dirichlet_loads_task_moe_shape():
     run(loads, 2048, 512, slack=3)
 
 
+def _ffn_at_full_size(loads, d, dff, seed):
+    """Both GEMMs of an expert FFN (d -> dff with GELU, dff -> d) in one launch each over the
+    given loads, against per-expert ``F.linear`` in fp32 on the bf16 operands (1e-2 of the largest
+    magnitude, test/python/jit_test.py:183-203 with the tolerance of bf16 outputs).  Weights are
+    drawn on the device, N(0, 0.02)."""
+    from brainstorm_amd.jit import grouped_linear
+
+    E, rows = len(loads), int(sum(loads))
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    x = torch.randn(rows, d, generator=g, device="cuda").to(torch.bfloat16)
+    w1 = torch.empty(E, dff, d, dtype=torch.bfloat16, device="cuda")
+    w2 = torch.empty(E, d, dff, dtype=torch.bfloat16, device="cuda")
+    for e in range(E):
+        w1[e] = (torch.randn(dff, d, generator=g, device="cuda") * 0.02).to(torch.bfloat16)
+        w2[e] = (torch.randn(d, dff, generator=g, device="cuda") * 0.02).to(torch.bfloat16)
+    t1 = torch.tensor([w1[e].data_ptr() for e in range(E)], dtype=torch.int64, device="cuda")
+    t2 = torch.tensor([w2[e].data_ptr() for e in range(E)], dtype=torch.int64, device="cuda")
+    d_loads = torch.tensor(loads, dtype=torch.int32, device="cuda")
+    h = torch.full((rows, dff), float("nan"), dtype=torch.bfloat16, device="cuda")
+    y = torch.full((rows, d), float("nan"), dtype=torch.bfloat16, device="cuda")
+    grouped_linear(x, h, t1, None, d_loads, d, dff, "gelu")
+    grouped_linear(h, y, t2, None, d_loads, dff, d)
+    torch.cuda.synchronize()
+    assert torch.isfinite(h.float()).all() and torch.isfinite(y.float()).all()
+    worst1 = worst2 = 0.0
+    scale1 = scale2 = 0.0
+    start = 0
+    for e, m in enumerate(loads):
+        if m:
+            rows_e = slice(start, start + m)
+            ref1 = torch.nn.functional.gelu(torch.nn.functional.linear(x[rows_e].float(), w1[e].float()))
+            ref2 = torch.nn.functional.linear(h[rows_e].float(), w2[e].float())
+            worst1 = max(worst1, float((h[rows_e].float() - ref1).abs().max()))
+            worst2 = max(worst2, float((y[rows_e].float() - ref2).abs().max()))
+            scale1 = max(scale1, float(ref1.abs().max()))
+            scale2 = max(scale2, float(ref2.abs().max()))
+        start += m
+    assert worst1 < 1e-2 * scale1, (worst1, scale1)
+    assert worst2 < 1e-2 * scale2, (worst2, scale2)
+
+
+def test_task_moe_ragged_ffn_at_full_size():
+    """BASELINE configuration 5 (benchmark/task_moe/moe_layer.py:151-175): 32768 rows x 2048 bf16,
+    128 experts, loads = 32768 * Dirichlet(0.3) by largest remainder (seed 5: 20 experts empty,
+    one with 5771 rows), FFN 2048 -> 8192 -> 2048, one launch per GEMM over the ragged batches."""
+    from workloads import dirichlet_loads
+
+    loads = dirichlet_loads(32768, 128, 0.3, seed=5).tolist()
+    assert min(loads) == 0 and max(loads) > 4096
+    _ffn_at_full_size(loads, 2048, 8192, seed=5)
+
+
+def test_top2_moe_ffn_at_full_size():
+    """BASELINE configuration 3's expert FFN: 32 experts, 1024 -> 4096 -> 1024, loads of the
+    Zipf-skewed top-2 route throttled to 2048 cells per path (four paths full, some nearly empty)."""
+    from workloads import top2_skewed_route
+
+    loads = top2_skewed_route()[3].tolist()
+    assert max(loads) == 2048 and min(loads) < 16
+    _ffn_at_full_size(loads, 1024, 4096, seed=3)
+
+
 # --------------------------------------------------- routing folded into the GEMM
 def _expert_tables(E, K, N, seed):
     g = torch.Generator().manual_seed(seed)
