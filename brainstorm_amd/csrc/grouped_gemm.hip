@@ -490,7 +490,7 @@ int launch_act(GemmArgs& a, hipStream_t st) {
   // Column tiles one workgroup walks: the largest number that neither leaves CUs without a
   // workgroup nor adds a round of tiles to the busiest CU (estimated like the tile shape,
   // from the row blocks a capacity-filled route has; the loads themselves live on the device).
-  static const int forced_walk = std::getenv("BRT_GEMM_WALK") ? std::atoi(std::getenv("BRT_GEMM_WALK")) : 0;
+  constexpr int forced_walk = 0;  // a fixed walk length, for experiments
   a.walk = 1;
   if (WAVES == 4) {  // the narrower tiles stage more per thread and have no registers left for it
     const long slots = static_cast<long>(device_cus()) * (WAVES == 2 ? 2 : 1);
@@ -580,13 +580,12 @@ int grouped_gemm_impl(const void* x, const void* const* weights, const void* con
   a.tag_div = entries_per_cell;
   a.E = E; a.P = P; a.K = K; a.N = N; a.T = T;
   a.gather = gather_in != 0; a.scatter = scatter_out != 0;
-  if (wide_gemm_applies(a)) return launch_wide_gemm(a, act, as_stream(stream));
   // Tile choice.  A wavefront owns 160 x 64 outputs (7 LDS fragment reads feed 10 MFMAs); a
   // workgroup is 2, 3 or 4 of them side by side.  The kernel is bound by how fast a CU can fill
   // its L1 (about 29 KB/us, L2 hits included), so the shape is the one that gives the busiest CU
   // the fewest operand bytes: wide tiles re-read the activation rows less often, narrow ones
   // keep all CUs busy when there are few tiles (only the 2-wavefront tile fits twice on a CU).
-  static const int forced = std::getenv("BRT_GEMM_SHAPE") ? std::atoi(std::getenv("BRT_GEMM_SHAPE")) : 0;
+  constexpr int forced = 0;  // a fixed tile shape (21..24), for experiments
   int shape = forced;
   if (shape == 0) {
     const int cus = device_cus();

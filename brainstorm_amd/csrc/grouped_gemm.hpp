@@ -47,9 +47,4 @@ __device__ __forceinline__ float apply_act(float v) {
   return v;
 }
 
-// Second kernel of the grouped GEMM: 256 x 256 tiles for experts with many rows (grouped_gemm_wide.hip).
-// Returns BRT_OK after queueing the launch; the caller has checked the arguments.
-bool wide_gemm_applies(const GemmArgs& a);
-int launch_wide_gemm(GemmArgs& a, int act, hipStream_t st);
-
 }  // namespace brt

@@ -65,11 +65,6 @@ struct ScanGeometry {
 
 constexpr int kWavesSingle = 8;  // 512 threads: the kernel keeps its 256 registers per lane
 
-int env_int(const char* name, int fallback) {
-  const char* v = getenv(name);
-  return v ? atoi(v) : fallback;
-}
-
 ScanGeometry scan_geometry(int T, int E, bool tag_mode) {
   ScanGeometry g;
   int shift = 0;
@@ -77,7 +72,7 @@ ScanGeometry scan_geometry(int T, int E, bool tag_mode) {
   g.ep_shift = shift;
   g.waves_pb = kWavesPB;
   const int rps = kWave >> shift;  // rows per load instruction
-  static const int forced_bands = env_int("BRT_SCAN_BANDS", 0);  // tuning knob, read once
+  constexpr int forced_bands = 0;  // a fixed number of workgroups, for experiments
   // Small masks (decode-sized batches) take one launch of one workgroup, the column sums of its
   // wavefronts meeting in LDS.  Up to four loads per lane of a 4-wavefront workgroup that is
   // the ordinary kernel with a single band (16 x 8: 4.1 us, 128 x 8: 4.7 us); up to one batch of

@@ -1045,16 +1045,12 @@ int pick_unit_bytes(size_t row_bytes, int elem, const void* p0, const void* p1, 
   return 0;
 }
 
-// Tuning knobs from the environment, read once per process.
-int env_int(const char* name, int fallback) {
-  const char* v = getenv(name);
-  return v ? atoi(v) : fallback;
-}
+// Launch shape constants (0 = chosen per launch from the shape).
 struct Knobs {
-  int dispatch_rows = env_int("BRT_DISPATCH_ROWS", 0);
-  int combine_rows = env_int("BRT_COMBINE_ROWS", 0);
-  int waves_pb = env_int("BRT_WAVES_PB", kBlock / kWave);
-  bool no_lean = env_int("BRT_NO_LEAN", 0) != 0;
+  int dispatch_rows = 0;
+  int combine_rows = 0;
+  int waves_pb = kBlock / kWave;
+  bool no_lean = false;
 };
 const Knobs& knobs() {
   static const Knobs k;
