@@ -570,13 +570,13 @@ def phase_extras(gpu, layer, steps):
         gpu.check(L.brt_hip_grouped_gemm_routed(
             x.data_ptr(), layer.wi_tab.data_ptr(), None, h_fused.data_ptr(),
             loads_counts_t[0].data_ptr(), tag_idx.data_ptr(), E, P, T, D, DFF, lib.ACT_GELU, 1, 0,
-            gpu.sptr()))
+            None, gpu.sptr()))
 
     def k_gemm2_scatter():
         gpu.check(L.brt_hip_grouped_gemm_routed(
             h_fused.data_ptr(), layer.wo_tab.data_ptr(), None, out_fused.data_ptr(),
             loads_counts_t[0].data_ptr(), tag_idx.data_ptr(), E, P, T, DFF, D, lib.ACT_NONE, 0, 1,
-            gpu.sptr()))
+            None, gpu.sptr()))
 
     def step_fused():
         k_indexgen_tags()

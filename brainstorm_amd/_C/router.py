@@ -9,7 +9,6 @@ router.cc:78; identical when no stream context is active).
 """
 from __future__ import annotations
 
-import weakref
 from typing import List, Optional, Tuple
 
 import torch
@@ -21,9 +20,13 @@ _DT = {torch.float32: _lib.F32, torch.float16: _lib.F16, torch.bfloat16: _lib.BF
 __all__ = [
     "topk_hot_mask",
     "throttle_hotmask",
+    "Route",
+    "generate_route",
     "generate_indices_and_loads",
     "convert_index_format",
     "dispatch_with_indices_and_loads",
+    "dispatch_rows_of_route",
+    "combine_by_row_tags",
     "split_fused_cells_to_paths",
     "fuse_split_cells_from_paths",
     "combine_with_indices_and_loads",
@@ -90,43 +93,50 @@ def _scan_workspace(device: torch.device, T: int, E: int) -> torch.Tensor:
     return ws
 
 
-class _Pairing:
-    """Remembers which (indices, loads) pair one index-generation call produced,
-    together with the true per-path counts, so that dispatch can zero-fill the
-    padding rows itself instead of clearing the whole output first.  For routes
-    that send a cell to at most one path (``single_path``) it also keeps the
-    per-row tags the last dispatch wrote, which let combine run in scatter form."""
+class Route:
+    """What one index-generation call knows about a route, beyond the ``(indices, loads)`` pair
+    the reference returns: the true per-path counts (``loads`` may be padded), whether a cell can
+    be on more than one path, and -- once a dispatch or a gathering GEMM has run -- the cell
+    behind every row of the path-major layout.  Fabrics carry it next to the stacks of the routed
+    GridTensor and hand it to dispatch / combine with the ``route=`` keyword; without it those ops
+    take their general forms (pre-zeroed output, index-driven combine)."""
 
-    __slots__ = ("indices_ref", "indices_ptr", "indices_version", "loads_version", "counts",
-                 "single_path", "row_tags", "row_tags_stride")
+    __slots__ = ("indices", "loads", "counts", "is_tag_index", "single_path", "cells", "paths",
+                 "row_tags", "row_tags_stride", "_versions")
 
-    def __init__(self, indices, loads, counts, single_path=False):
-        self.indices_ref = weakref.ref(indices)
-        self.indices_ptr = indices.data_ptr()
-        self.indices_version = indices._version
-        self.loads_version = loads._version
-        self.counts = counts
-        self.single_path = single_path
-        self.row_tags = None        # [P] int32: 1-based cell of each dispatched row, 0 = padding
+    def __init__(self, indices, loads, counts, is_tag_index, single_path):
+        self.indices, self.loads, self.counts = indices, loads, counts
+        self.is_tag_index = bool(is_tag_index)
+        self.single_path = bool(single_path)
+        self.cells, self.paths = indices.shape
+        self.row_tags = None        # [P] int32: 1-based cell of each row of the layout, 0 = no cell
         self.row_tags_stride = 0    # max_path_load the rows were laid out with (0 = packed)
+        self._versions = (indices._version, loads._version)
+
+    def owns(self, route_indices: torch.Tensor, loads: torch.Tensor) -> bool:
+        """True when the pair is the one this route was generated with, unmodified since."""
+        return (route_indices is self.indices and loads is self.loads
+                and self._versions == (route_indices._version, loads._version))
 
 
-def _pairing_of(route_indices: torch.Tensor, loads: torch.Tensor) -> Optional[_Pairing]:
-    pairing = getattr(loads, "_brt_pairing", None)
-    if (
-        pairing is None
-        or pairing.indices_ref() is not route_indices
-        or pairing.indices_ptr != route_indices.data_ptr()
-        or pairing.indices_version != route_indices._version
-        or pairing.loads_version != loads._version
-    ):
+_fallback_logged = set()
+
+
+def _log_general_form(op: str, why: str) -> None:
+    if op not in _fallback_logged:
+        _fallback_logged.add(op)
+        from brainstorm_amd.runtime.log import get_logger
+        get_logger(__file__).info("%s runs in its general form: %s", op, why)
+
+
+def _route_for(route: Optional["Route"], route_indices, loads, op: str) -> Optional["Route"]:
+    if route is None:
+        _log_general_form(op, "no route object was passed (route=None)")
         return None
-    return pairing
-
-
-def _paired_counts(route_indices: torch.Tensor, loads: torch.Tensor) -> Optional[torch.Tensor]:
-    pairing = _pairing_of(route_indices, loads)
-    return None if pairing is None else pairing.counts
+    if not route.owns(route_indices, loads):
+        _log_general_form(op, "the route object does not describe these indices / loads any more")
+        return None
+    return route
 
 
 # ------------------------------------------------------------------------- ops
@@ -174,26 +184,26 @@ def throttle_hotmask(
     return throttled, prefix
 
 
-def generate_indices_and_loads(
+def generate_route(
     hot_mask: torch.Tensor,
     supported_capacities: Optional[torch.Tensor] = None,
     capacity_padding: bool = False,
     path_wise_padding: bool = False,
     is_tag_index: bool = False,
-    *,
     single_path: bool = False,
-) -> Tuple[torch.Tensor, torch.Tensor]:
-    """router.cc:48-80.  ``single_path`` (keyword only, not in the reference) is the
-    caller's promise that no row of ``hot_mask`` has more than one nonzero; dispatch
-    and combine calls that receive the returned pair may then use the tag-driven
-    combine (same results, one memory round trip less)."""
+) -> Route:
+    """Index generation (router.cc:48-80) returning the :class:`Route`.  ``single_path`` is the
+    caller's promise that no row of ``hot_mask`` has more than one nonzero; dispatch and combine
+    calls that receive the route may then use the tag-driven combine (same results, one memory
+    round trip less)."""
     _check_on_device(hot_mask, "hot_mask")
     _check_int32(hot_mask, "hot_mask")
     T, E = hot_mask.size(0), hot_mask.size(1)
     with _device_guard(hot_mask.device):
         if hot_mask.numel() == 0:  # router.cc:59-62
-            return (torch.zeros((0, E), dtype=hot_mask.dtype, device=hot_mask.device),
-                    torch.zeros((E,), dtype=hot_mask.dtype, device=hot_mask.device))
+            indices = torch.zeros((0, E), dtype=hot_mask.dtype, device=hot_mask.device)
+            loads = torch.zeros((E,), dtype=hot_mask.dtype, device=hot_mask.device)
+            return Route(indices, loads, loads.clone(), is_tag_index, single_path)
         caps = None
         n_caps = 0
         if supported_capacities is not None:
@@ -212,9 +222,20 @@ def generate_indices_and_loads(
             _ptr(hot_mask), _ptr(indices), _ptr(loads), _ptr(counts), T, E, _ptr(caps), n_caps,
             int(capacity_padding), int(path_wise_padding), int(is_tag_index),
             _ptr(ws), ws.numel(), _stream()))
-        if not is_tag_index:
-            loads._brt_pairing = _Pairing(indices, loads, counts, bool(single_path))
-    return indices, loads
+    return Route(indices, loads, counts, is_tag_index, single_path)
+
+
+def generate_indices_and_loads(
+    hot_mask: torch.Tensor,
+    supported_capacities: Optional[torch.Tensor] = None,
+    capacity_padding: bool = False,
+    path_wise_padding: bool = False,
+    is_tag_index: bool = False,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """router.cc:48-80."""
+    route = generate_route(hot_mask, supported_capacities, capacity_padding, path_wise_padding,
+                           is_tag_index)
+    return route.indices, route.loads
 
 
 def convert_index_format(
@@ -267,8 +288,13 @@ def dispatch_with_indices_and_loads(
     max_path_load: int = 0,
     is_1d_routing: bool = True,
     is_tag_index: bool = False,
+    *,
+    route: Optional[Route] = None,
 ) -> List[torch.Tensor]:
-    """router.cc:131-273.  Returns ``[out]`` or ``[out, new_tags]``."""
+    """router.cc:131-273.  Returns ``[out]`` or ``[out, new_tags]``.  ``route`` (keyword only,
+    not in the reference): the :class:`Route` the indices came from; the kernel then zero-fills
+    only the padding rows of an un-zeroed output and, for single-path routes, leaves the per-row
+    tags on the route for the combine."""
     _check_on_device(in_data, "in_data")
     _check_on_device(route_indices, "route_indices")
     _check_int32(route_indices, "route_indices")
@@ -296,7 +322,11 @@ def dispatch_with_indices_and_loads(
         if not is_1d_routing:
             cell //= E
 
-        pairing = None if is_tag_index else _pairing_of(route_indices, loads)
+        pairing = None
+        if not is_tag_index:
+            pairing = _route_for(route, route_indices, loads, "dispatch_with_indices_and_loads")
+            if pairing is not None and pairing.is_tag_index:
+                pairing = None
         counts = None if pairing is None else pairing.counts
         _check_int32(loads, "loads")
         dev_loads = loads if loads.is_cuda else loads.to(device, non_blocking=True)
@@ -355,6 +385,58 @@ def dispatch_with_indices_and_loads(
     if tag_generating:
         return [out, new_tags]
     return [out]
+
+
+def dispatch_rows_of_route(cells: torch.Tensor, route: Route, out: torch.Tensor) -> None:
+    """The dispatch a deferred fused dispatch stands for (not in the reference): rows of ``cells``
+    into the pre-allocated path-major ``out`` by the tag indices of ``route``; rows no path owns are
+    zero; the row tags are left on the route."""
+    if not route.is_tag_index:
+        raise RuntimeError("a deferred dispatch holds tag indices")
+    T = cells.size(0)
+    rows = out.size(0)
+    with _device_guard(cells.device):
+        out.zero_()
+        row_tags = torch.zeros((rows,), dtype=torch.int32, device=cells.device)
+        if T > 0 and rows > 0:
+            _lib.check(_lib.lib().brt_hip_dispatch(
+                _ptr(cells), _ptr(out), None, _ptr(route.indices), _ptr(route.loads), None, None,
+                _ptr(row_tags), T, cells.numel() // T, route.paths, rows, 0, 1, 1,
+                _DT[cells.dtype], _stream()))
+        route.row_tags, route.row_tags_stride = row_tags, 0
+
+
+def combine_by_row_tags(in_data: torch.Tensor, row_tags: torch.Tensor, cells: int,
+                        out_data: Optional[torch.Tensor] = None,
+                        out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """Combine of a route in which no cell is on more than one path, from the per-row tags
+    (not in the reference as an op; what its seat-index combine computes for such a route,
+    route.cu:208-282): ``out[row_tags[p] - 1] = in_data[p]`` for every tagged row.  ``out_data``
+    is updated in place (cells without a row keep their values); without it the result starts
+    from zeros."""
+    _check_on_device(in_data, "in_data")
+    if in_data.dtype not in _DT:
+        raise NotImplementedError("data type is not supported")
+    P = in_data.size(0)
+    in_data = in_data.contiguous()
+    cell = in_data.numel() // P if P > 0 else 0
+    with _device_guard(in_data.device):
+        if out_data is not None:
+            if not out_data.is_contiguous():
+                raise RuntimeError("out_data must be contiguous (it is updated in place)")
+            result = out_data
+        else:
+            shape = list(in_data.shape)
+            shape[0] = cells
+            result = torch.zeros(shape, dtype=out_dtype or in_data.dtype, device=in_data.device)
+        if result.dtype not in _DT or result.numel() != cells * cell:
+            raise RuntimeError("out_data does not match [cell_num, *cell_shape]")
+        if row_tags.numel() < P:
+            raise RuntimeError("one tag per row is needed")
+        _lib.check(_lib.lib().brt_hip_combine_by_tags(
+            _ptr(in_data), _ptr(result), _ptr(row_tags), P, cell, cells, _DT[in_data.dtype],
+            _DT[result.dtype], _stream()))
+    return result
 
 
 def split_fused_cells_to_paths(
@@ -453,6 +535,7 @@ def combine_with_indices_and_loads(
     tags: Optional[torch.Tensor] = None,
     *,
     out_dtype: Optional[torch.dtype] = None,
+    route: Optional[Route] = None,
 ) -> List[torch.Tensor]:
     """router.cc:372-473.
 
@@ -514,7 +597,7 @@ def combine_with_indices_and_loads(
             raise RuntimeError("out_data does not match [cell_num, *cell_shape]")
         # single-path routes whose rows still carry the tags of the paired dispatch:
         # scatter form (identical rows; cells without a row keep the residual)
-        pairing = _pairing_of(route_indices, loads)
+        pairing = _route_for(route, route_indices, loads, "combine_with_indices_and_loads")
         if (residual and dev_gates is None and pairing is not None and pairing.single_path
                 and pairing.row_tags is not None and pairing.row_tags.numel() == P
                 and pairing.row_tags_stride == mpl

@@ -71,8 +71,18 @@ SIGNATURES = {
     "brt_hip_grouped_gemm_routed": (
         _c_int,
         [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int,
-         _c_int, _c_int, _c_int, _c_ptr],
+         _c_int, _c_int, _c_int, _c_ptr, _c_ptr],
     ),
+    "brt_hip_grouped_gemm_f32out": (
+        _c_int,
+        [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    ),
+    "brt_hip_grouped_gemm_routed_f32out": (
+        _c_int,
+        [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int,
+         _c_int, _c_int, _c_int, _c_ptr, _c_ptr],
+    ),
+    "brt_hip_cast_f32_to_bf16": (_c_int, [_c_ptr, _c_ptr, _c_size, _c_ptr]),
     "brt_hip_grouped_gemm_by_rows": (
         _c_int,
         [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
@@ -141,8 +151,21 @@ def lib() -> ctypes.CDLL:
     return _lib
 
 
+_calls = 0
+
+
+def call_count() -> int:
+    """Calls into the library that queued device work and were checked with :func:`check` since
+    the process started (every such call is one kernel launch, except index generation, the
+    compact route and the tag-index gather, which are two).  Tests use the difference around a
+    layer to pin how many launches a route costs."""
+    return _calls
+
+
 def check(code: int) -> None:
     """Turn a negative return code into the exception the reference binding raises."""
+    global _calls
+    _calls += 1
     if code == 0:
         return
     msg = lib().brt_hip_last_error().decode()

@@ -45,6 +45,7 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 // Pointers read from the per-expert table are generic to the compiler, which would
 // make every weight load a flat load counted on the LDS counter as well; the
 // explicit global address space keeps weight loads off the LDS wait path.
@@ -77,8 +78,9 @@ struct Staged {
   u32x4 v[N];
 };
 
-template <int MT, int NT, int WAVES, int ACT, bool WALKS, bool WSTREAM>
+template <int MT, int NT, int WAVES, int ACT, bool WALKS, bool WSTREAM, bool OUTF32 = false>
 __global__ __launch_bounds__(WAVES * 64) void grouped_gemm_kernel(GemmArgs a) {
+  static_assert(!(OUTF32 && WALKS), "the fp32 epilogue is built for one column tile per workgroup");
   constexpr int THREADS = WAVES * 64;
   constexpr int BM = MT * 32, WN = NT * 32, BN = WAVES * WN;
   constexpr int TILE_ROWS = BM + BN;  // activation rows first, then weight rows
@@ -129,11 +131,24 @@ __global__ __launch_bounds__(WAVES * 64) void grouped_gemm_kernel(GemmArgs a) {
       carry_t += __shfl(incl_t, kWave - 1, kWave);
       carry_m += __shfl(incl_m, kWave - 1, kWave);
     }
-    if (!found && lane == 0) s_tile[0] = -1;
+    if (!found && lane == 0) {  // beyond the last row block: how far, and where the rows end
+      s_tile[0] = -1;
+      s_tile[1] = carry_m;
+      s_tile[2] = mt - carry_t;
+    }
   }
   __syncthreads();
   const int e = __builtin_amdgcn_readfirstlane(s_tile[0]);
-  if (e < 0) return;  // beyond the last tile
+  if (e < 0) {
+    // The row blocks past the last one clear the tags of the rows no path owns (the layout may be
+    // allocated for more rows than the loads add up to): surplus block j takes rows
+    // [total + j * BM, total + (j + 1) * BM); there are at least (P - total) / BM of them.
+    if (a.row_tags_out != nullptr && nt_first == 0) {
+      const long first = static_cast<long>(s_tile[1]) + static_cast<long>(s_tile[2]) * BM;
+      for (long r = first + tid; r < min(first + BM, static_cast<long>(a.P)); r += THREADS) a.row_tags_out[r] = 0;
+    }
+    return;
+  }
   const int row0 = __builtin_amdgcn_readfirstlane(s_tile[1]);
   const int rows = __builtin_amdgcn_readfirstlane(s_tile[2]);
   const int seat0 = __builtin_amdgcn_readfirstlane(s_tile[3]);
@@ -177,6 +192,8 @@ __global__ __launch_bounds__(WAVES * 64) void grouped_gemm_kernel(GemmArgs a) {
         cell = (tag >= 1 && tag <= a.T) ? tag - 1 : -1;
       }
       s_cell[r] = cell;
+      // side output for a combine that runs later: the cell of every row, written once per row block
+      if (a.row_tags_out != nullptr && nt_first == 0) a.row_tags_out[static_cast<size_t>(row0) + r] = cell + 1;
     }
     __syncthreads();
   }
@@ -403,6 +420,30 @@ __global__ __launch_bounds__(WAVES * 64) void grouped_gemm_kernel(GemmArgs a) {
         for (int q = 0; q < 4; ++q) bv[j][g][q] = static_cast<float>(b4[q]);
       }
     }
+    if constexpr (OUTF32) {
+      // fp32 output (the contract of the reference's expert kernel): the accumulator leaves as it
+      // is, 4 consecutive columns (16 bytes) per lane and store, no LDS.
+#pragma unroll
+      for (int i = 0; i < MT; ++i) {
+        const int r = i * 32 + frag_row_e;
+        long to = a.scatter ? (r < rows ? s_cell[r] : -1) : static_cast<long>(row0) + r;
+        if (i >= row_tiles || r >= rows || to < 0) continue;
+        float* const orow = a.out_f32 + static_cast<size_t>(to) * a.N;
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const int col = n0 + wave * WN + j * 32 + 8 * g + 4 * frag_k_e;
+            if (col >= a.N) continue;
+            f32x4 o;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) o[q] = apply_act<ACT>(acc[i][j][4 * g + q] + bv[j][g][q]) + 0.0f;  // -0 -> +0, as a combine would
+            *reinterpret_cast<f32x4*>(orow + col) = o;
+          }
+        }
+      }
+      continue;
+    }
     constexpr int OUT_CHUNKS = BN / 8;
     constexpr int kPasses = WALKS ? 2 : 1;
     constexpr int kPassTiles = (MT + kPasses - 1) / kPasses;
@@ -539,6 +580,30 @@ int launch_act(GemmArgs& a, hipStream_t st) {
   return stream_weights ? run(No{}, Yes{}) : run(No{}, No{});
 }
 
+// fp32 output: the 4-wavefront tile, one column tile per workgroup, ordinary weight loads
+template <int ACT>
+int launch_f32(GemmArgs& a, hipStream_t st) {
+  constexpr int MT = 5, NT = 2, WAVES = 4, BM = MT * 32, BN = WAVES * NT * 32;
+  constexpr int STAGE = (BM + BN) * kRowBytes;
+  a.tiles_n = (a.N + BN - 1) / BN;
+  a.tiles_m_max = ((a.P + BM - 1) / BM + a.E + kXcds - 1) / kXcds * kXcds;
+  a.walk = 1;
+  a.groups_n = a.tiles_n;
+  auto* fn = &grouped_gemm_kernel<MT, NT, WAVES, ACT, false, false, true>;
+  static bool configured[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 63;
+  if (!configured[dev] || dev == 63) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            2 * STAGE) != hipSuccess)
+      return fail(BRT_E_LAUNCH, "cannot reserve %d bytes of LDS", 2 * STAGE);
+    configured[dev] = true;
+  }
+  const long grid_wgs = static_cast<long>(a.tiles_m_max) * a.groups_n;
+  hipLaunchKernelGGL(fn, dim3(static_cast<unsigned>(grid_wgs)), dim3(WAVES * 64), 2 * STAGE, st, a);
+  return check_launch("grouped_gemm_kernel (fp32 output)");
+}
+
 template <int MT, int NT, int WAVES>
 int launch(GemmArgs& a, int act, hipStream_t st) {
   if (act == BRT_ACT_GELU) return launch_act<MT, NT, WAVES, BRT_ACT_GELU>(a, st);
@@ -555,7 +620,8 @@ namespace {
 
 int grouped_gemm_impl(const void* x, const void* const* weights, const void* const* biases, void* out,
                       const int32_t* loads, const int32_t* tags, int entries_per_cell, int E, int P,
-                      int T, int K, int N, int act, int gather_in, int scatter_out, void* stream) {
+                      int T, int K, int N, int act, int gather_in, int scatter_out, void* stream,
+                      bool out_is_f32 = false, int32_t* row_tags_out = nullptr) {
   if (E <= 0 || P < 0 || K <= 0 || N <= 0 || T < 0)
     return fail(BRT_E_INVALID, "bad shape E=%d P=%d T=%d K=%d N=%d", E, P, T, K, N);
   if (K % 8 != 0 || N % 8 != 0)
@@ -573,13 +639,20 @@ int grouped_gemm_impl(const void* x, const void* const* weights, const void* con
   a.x = static_cast<const __bf16*>(x);
   a.w = reinterpret_cast<const __bf16* const*>(weights);
   a.bias = reinterpret_cast<const __bf16* const*>(biases);
-  a.out = static_cast<__bf16*>(out);
+  a.out = out_is_f32 ? nullptr : static_cast<__bf16*>(out);
+  a.out_f32 = out_is_f32 ? static_cast<float*>(out) : nullptr;
+  a.row_tags_out = tags != nullptr ? row_tags_out : nullptr;
   a.loads = loads;
   a.tags = tags;
   a.tag_vector = entries_per_cell > 0;
   a.tag_div = entries_per_cell;
   a.E = E; a.P = P; a.K = K; a.N = N; a.T = T;
   a.gather = gather_in != 0; a.scatter = scatter_out != 0;
+  if (out_is_f32) {
+    if (act == BRT_ACT_GELU) return launch_f32<BRT_ACT_GELU>(a, as_stream(stream));
+    if (act == BRT_ACT_RELU) return launch_f32<BRT_ACT_RELU>(a, as_stream(stream));
+    return launch_f32<BRT_ACT_NONE>(a, as_stream(stream));
+  }
   // Tile choice.  A wavefront owns 160 x 64 outputs (7 LDS fragment reads feed 10 MFMAs); a
   // workgroup is 2, 3 or 4 of them side by side.  The kernel is bound by how fast a CU can fill
   // its L1 (about 29 KB/us, L2 hits included), so the shape is the one that gives the busiest CU
@@ -613,13 +686,56 @@ extern "C" int brt_hip_grouped_gemm(const void* x, const void* const* weights,
   return grouped_gemm_impl(x, weights, biases, out, loads, nullptr, 0, E, P, 0, K, N, act, 0, 0, stream);
 }
 
+extern "C" int brt_hip_grouped_gemm_f32out(const void* x, const void* const* weights,
+                                           const void* const* biases, float* out,
+                                           const int32_t* loads, int E, int P, int K, int N, int act,
+                                           void* stream) {
+  return grouped_gemm_impl(x, weights, biases, out, loads, nullptr, 0, E, P, 0, K, N, act, 0, 0, stream, true);
+}
+
 extern "C" int brt_hip_grouped_gemm_routed(const void* x, const void* const* weights,
                                            const void* const* biases, void* out,
                                            const int32_t* loads, const int32_t* tags, int E, int P,
                                            int T, int K, int N, int act, int gather_in,
-                                           int scatter_out, void* stream) {
+                                           int scatter_out, int32_t* row_tags_out, void* stream) {
   return grouped_gemm_impl(x, weights, biases, out, loads, tags, 0, E, P, T, K, N, act, gather_in,
-                           scatter_out, stream);
+                           scatter_out, stream, false, row_tags_out);
+}
+
+extern "C" int brt_hip_grouped_gemm_routed_f32out(const void* x, const void* const* weights,
+                                                  const void* const* biases, float* out,
+                                                  const int32_t* loads, const int32_t* tags, int E,
+                                                  int P, int T, int K, int N, int act, int gather_in,
+                                                  int scatter_out, int32_t* row_tags_out, void* stream) {
+  return grouped_gemm_impl(x, weights, biases, out, loads, tags, 0, E, P, T, K, N, act, gather_in,
+                           scatter_out, stream, true, row_tags_out);
+}
+
+namespace {
+// 8 values per thread: two 16-byte loads, one 16-byte store
+__global__ __launch_bounds__(256) void cast_f32_to_bf16_kernel(const float* __restrict__ src, __bf16* __restrict__ dst, size_t n) {
+  const size_t i = (static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x) * 8;
+  if (i + 8 <= n) {
+    const f32x4 lo = *reinterpret_cast<const f32x4*>(src + i), hi = *reinterpret_cast<const f32x4*>(src + i + 4);
+    bf16x8 o;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) o[q] = static_cast<__bf16>(lo[q]), o[4 + q] = static_cast<__bf16>(hi[q]);
+    *reinterpret_cast<bf16x8*>(dst + i) = o;
+  } else {
+    for (size_t j = i; j < n; ++j) dst[j] = static_cast<__bf16>(src[j]);
+  }
+}
+}  // namespace
+
+extern "C" int brt_hip_cast_f32_to_bf16(const float* src, void* dst, size_t n, void* stream) {
+  if (n == 0) return BRT_OK;
+  if (!src || !dst) return fail(BRT_E_INVALID, "null argument");
+  if (!aligned(src, 16) || !aligned(dst, 16)) return fail(BRT_E_INVALID, "src/dst must be 16-byte aligned");
+  const size_t blocks = (n + 2047) / 2048;
+  if (blocks > 0x7fffffffull) return fail(BRT_E_UNSUPPORTED, "%zu elements are too many for one launch", n);
+  hipLaunchKernelGGL(cast_f32_to_bf16_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0,
+                     as_stream(stream), src, static_cast<__bf16*>(dst), n);
+  return check_launch("cast_f32_to_bf16_kernel");
 }
 
 extern "C" int brt_hip_grouped_gemm_by_rows(const void* x, const void* const* weights,

@@ -10,6 +10,8 @@ struct GemmArgs {
   const __bf16* const* w;
   const __bf16* const* bias;
   __bf16* out;
+  float* out_f32;      // non-null: the output is fp32 (the accumulator after bias and activation), `out` is unused
+  int* row_tags_out;   // non-null (routed forms): [P], the 1-based cell behind every row of the layout, 0 = empty slot
   const int* loads;
   const int* tags;  // [T,E] tag matrix (column e: 1-based cells of path e in seat order), or the
                     // row-entry vector [P] of the compact route (1-based entry t*k+j+1 per row), or null

@@ -20,6 +20,7 @@ import torch
 import torch.nn as nn
 
 from brainstorm_amd import _lib
+from brainstorm_amd.runtime import deferred
 
 __all__ = ["make_jit_kernel", "grouped_linear", "GroupedLinearKernel"]
 
@@ -46,7 +47,8 @@ def grouped_linear(x: torch.Tensor, out: torch.Tensor, weight_table: torch.Tenso
                    out_features: int, activation: Optional[str] = None, *,
                    tags: Optional[torch.Tensor] = None, gather: bool = False,
                    scatter: bool = False, rows: Optional[int] = None,
-                   row_entries: Optional[torch.Tensor] = None, entries_per_cell: int = 1) -> torch.Tensor:
+                   row_entries: Optional[torch.Tensor] = None, entries_per_cell: int = 1,
+                   row_tags_out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``out[s_e : s_e + loads[e]] = act(x[s_e : s_e + loads[e]] @ W_e^T + b_e)`` for every
     branch e, ``s_e = sum(loads[:e])``, in one launch.  ``weight_table`` /
     ``bias_table`` are int64 device tensors holding the branch pointers.
@@ -60,9 +62,17 @@ def grouped_linear(x: torch.Tensor, out: torch.Tensor, weight_table: torch.Tenso
 
     ``row_entries`` (the vector ``route_by_path`` writes: 1-based entry ``t * k + j + 1`` of every
     row of the dispatched layout, ``k = entries_per_cell``) names the rows instead of ``tags``:
-    row r is cell ``(row_entries[r] - 1) // k``."""
-    if x.dtype != torch.bfloat16 or out.dtype != torch.bfloat16:
-        raise NotImplementedError("the grouped GEMM computes in bf16 (fp32 accumulation)")
+    row r is cell ``(row_entries[r] - 1) // k``.
+
+    ``out`` may be fp32 (tag-matrix and plain forms): it then receives the fp32 accumulator after
+    bias and activation.  ``row_tags_out`` (``[rows]`` int32, tag-matrix form) receives the
+    1-based cell behind every row of the layout, which is what a later tag-driven combine needs."""
+    if x.dtype != torch.bfloat16 or out.dtype not in (torch.bfloat16, torch.float32):
+        raise NotImplementedError("the grouped GEMM computes in bf16 (fp32 accumulation); "
+                                  "the output is bf16 or fp32")
+    f32_out = out.dtype == torch.float32
+    if f32_out and row_entries is not None:
+        raise NotImplementedError("the row-entry form writes bf16")
     if not (x.is_cuda and out.is_cuda and loads.is_cuda):
         raise RuntimeError("grouped_linear needs device tensors")
     if loads.dtype != torch.int32:
@@ -92,6 +102,8 @@ def grouped_linear(x: torch.Tensor, out: torch.Tensor, weight_table: torch.Tenso
         if (gather and x.shape[0] != cells) or (scatter and out.shape[0] != cells):
             raise RuntimeError("a gathered input / scattered output has one row per cell")
     if rows is None:
+        # both sides cell-major: at most one row per cell and path, and never more than the tag
+        # matrix has slots for
         rows = out.shape[0] if not scatter else (x.shape[0] if not gather else tags.numel())
     elif (not gather and rows > x.shape[0]) or (not scatter and rows > out.shape[0]):
         raise RuntimeError("rows exceeds the path-major buffer")
@@ -107,19 +119,58 @@ def grouped_linear(x: torch.Tensor, out: torch.Tensor, weight_table: torch.Tenso
                 row_entries.data_ptr(), int(entries_per_cell), loads.numel(), rows, cells,
                 in_features, out_features, _ACT[activation], int(gather), int(scatter), stream))
         elif routed:
-            _lib.check(lib.brt_hip_grouped_gemm_routed(
+            if row_tags_out is not None and (row_tags_out.dtype != torch.int32 or row_tags_out.numel() < rows
+                                             or not row_tags_out.is_cuda):
+                raise RuntimeError("row_tags_out must be an int32 device vector with one entry per row")
+            fn = lib.brt_hip_grouped_gemm_routed_f32out if f32_out else lib.brt_hip_grouped_gemm_routed
+            _lib.check(fn(
                 x.data_ptr(), weight_table.data_ptr(), bias_ptr, out.data_ptr(), loads.data_ptr(),
                 tags.data_ptr(), loads.numel(), rows, cells, in_features, out_features,
-                _ACT[activation], int(gather), int(scatter), stream))
+                _ACT[activation], int(gather), int(scatter),
+                None if row_tags_out is None else row_tags_out.data_ptr(), stream))
         else:
-            _lib.check(lib.brt_hip_grouped_gemm(
+            fn = lib.brt_hip_grouped_gemm_f32out if f32_out else lib.brt_hip_grouped_gemm
+            _lib.check(fn(
                 x.data_ptr(), weight_table.data_ptr(), bias_ptr, out.data_ptr(), loads.data_ptr(),
                 loads.numel(), rows, in_features, out_features, _ACT[activation], stream))
     return out
 
 
+def _to_bf16(t: torch.Tensor) -> torch.Tensor:
+    """fp32 -> bf16 (round to nearest even) with the library's cast kernel."""
+    t = t.contiguous()
+    out = torch.empty(t.shape, dtype=torch.bfloat16, device=t.device)
+    if t.numel():
+        _lib.check(_lib.lib().brt_hip_cast_f32_to_bf16(
+            t.data_ptr(), out.data_ptr(), t.numel(),
+            torch._C._cuda_getCurrentRawStream(torch._C._cuda_getDevice())))
+    return out
+
+
+class _Bf16Weights:
+    """bf16 copies of fp32 branch parameters, converted again only when a parameter changed."""
+
+    def __init__(self):
+        self.keys = None
+        self.copies = None
+
+    def get(self, tensors: Sequence[torch.Tensor]) -> List[torch.Tensor]:
+        keys = tuple((t.data_ptr(), t._version) for t in tensors)
+        if keys != self.keys:
+            self.copies = [_to_bf16(t.detach()) for t in tensors]
+            self.keys = keys
+        return self.copies
+
+
 class GroupedLinearKernel:
-    """Callable returned by ``make_jit_kernel(ModuleList[Linear], ..., "homo_fuse")``."""
+    """Callable returned by ``make_jit_kernel(ModuleList[Linear], ..., "homo_fuse")``.
+
+    The reference's kernels take and give fp32 (benchmark/switch_moe/switch_expert.py:74-92
+    allocates its outputs with ``torch.empty`` in the default dtype; test/python/jit_test.py:157-203
+    runs fp32 throughout).  This kernel multiplies bf16 operands on the matrix units with fp32
+    accumulation: fp32 shared inputs and fp32 branch parameters are converted to bf16 first (the
+    parameters once, until they change), and an fp32 output tensor receives the fp32 accumulator.
+    Against fp32 ``F.linear`` the result is within 1e-2 relative (bf16 operand rounding)."""
 
     def __init__(self, in_features: int, out_features: int, has_bias: bool,
                  activation: Optional[str] = None):
@@ -129,6 +180,8 @@ class GroupedLinearKernel:
         self.activation = activation
         self._weights = _PointerTable()
         self._biases = _PointerTable()
+        self._weights_bf16 = _Bf16Weights()
+        self._biases_bf16 = _Bf16Weights()
 
     def __call__(self, shared_inputs: List[torch.Tensor], standalone_inputs: Sequence[torch.Tensor],
                  capacities: Union[torch.Tensor, Sequence[int]] = ()):
@@ -138,17 +191,47 @@ class GroupedLinearKernel:
         weights = standalone_inputs[0::step]
         biases = standalone_inputs[1::step] if self.has_bias else None
         if not torch.is_tensor(capacities):
-            capacities = torch.tensor(list(capacities), dtype=torch.int32, device=x.device)
+            capacities = torch.tensor(list(capacities), dtype=torch.int32, device=out.device)
         if capacities.numel() > len(weights):
             raise RuntimeError("more capacities than branches")
-        for w in weights[: capacities.numel()]:
-            if w.dtype != torch.bfloat16 or not w.is_contiguous():
-                raise NotImplementedError("branch weights must be contiguous bf16 [out, in]")
+        weights = self._branch_operands(weights, capacities.numel(), self._weights_bf16, "weights")
+        if biases:
+            biases = self._branch_operands(biases, capacities.numel(), self._biases_bf16, "biases")
+        loads = capacities.to(device=out.device, dtype=torch.int32)
+        state = deferred.state_of(x)
+        if state is not None and self._can_gather(state, out):
+            # the rows of a deferred dispatch: read from the cells through the route's tag indices
+            route = state.route
+            cells = state.cells if state.cells.dtype == torch.bfloat16 else _to_bf16(state.cells)
+            row_tags = torch.empty((out.shape[0],), dtype=torch.int32, device=out.device)
+            grouped_linear(cells, out, self._weights.get(weights),
+                           self._biases.get(biases) if biases else None, loads, self.in_features,
+                           self.out_features, self.activation, tags=route.indices, gather=True,
+                           rows=out.shape[0], row_tags_out=row_tags)
+            route.row_tags, route.row_tags_stride = row_tags, 0
+            return
+        if x.dtype == torch.float32:
+            x = _to_bf16(x)  # (a deferred buffer is filled by this read)
         grouped_linear(
             x, out, self._weights.get(weights),
             self._biases.get(biases) if biases else None,
-            capacities.to(device=x.device, dtype=torch.int32), self.in_features,
-            self.out_features, self.activation)
+            loads, self.in_features, self.out_features, self.activation)
+
+    def _branch_operands(self, tensors, used: int, cache: _Bf16Weights, what: str):
+        dtypes = {t.dtype for t in tensors[:used]}
+        if dtypes == {torch.float32}:
+            return cache.get(tensors)
+        for t in tensors[:used]:
+            if t.dtype != torch.bfloat16 or not t.is_contiguous():
+                raise NotImplementedError(f"branch {what} must be contiguous bf16 or fp32 tensors of one dtype")
+        return tensors
+
+    def _can_gather(self, state, out: torch.Tensor) -> bool:
+        cells = state.cells
+        return (cells.dim() == 2 and cells.shape[1] == self.in_features and out.dim() == 2
+                and out.shape[0] == state.buffer.shape[0] and out.is_contiguous()
+                and cells.dtype in (torch.bfloat16, torch.float32)
+                and out.dtype in (torch.bfloat16, torch.float32))
 
 
 def make_jit_kernel(modules, sample_inputs=None, method: str = "forward", opt_level=None,

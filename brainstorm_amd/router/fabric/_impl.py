@@ -15,6 +15,7 @@ import torch.nn as nn
 from brainstorm_amd._C import router as c_router
 from brainstorm_amd.router.utils import make_kwargs
 from brainstorm_amd.runtime import Registry
+from brainstorm_amd.runtime.deferred import DeferredState
 from brainstorm_amd.runtime.grid_tensor import GridTensor, init_grid_tensor, to_torch_tensor
 
 _CAPTURE_MODES = ("avg", "max", "cum")
@@ -218,20 +219,26 @@ class DispatchFabric(FabricBase):
             self.path_wise_padding = False
         self.max_path_padding = kwargs.pop("max_path_padding", False)
         self.max_path_load = kwargs.pop("max_path_load", 0)
+        self._route = None  # the route of the forward call in progress
 
     def forward(self, in_flow, hot_mask: torch.Tensor, runtime_capacities: torch.Tensor = None,
                 score: torch.Tensor = None):
         caps = runtime_capacities if runtime_capacities is not None else self.supported_capacities
-        route_indices, loads = c_router.generate_indices_and_loads(
-            hot_mask, supported_capacities=caps, capacity_padding=self.capacity_padding,
-            path_wise_padding=self.path_wise_padding, is_tag_index=False,
-            single_path=getattr(hot_mask, "_brt_single_path", False))
         in_flows = [in_flow] if self.flow_num == 1 else in_flow
+        self._route = c_router.generate_route(
+            hot_mask, supported_capacities=caps, capacity_padding=self.capacity_padding,
+            path_wise_padding=self.path_wise_padding,
+            is_tag_index=self._defers(in_flows, runtime_capacities, hot_mask),
+            single_path=getattr(hot_mask, "_brt_single_path", False))
+        route_indices, loads = self._route.indices, self._route.loads
         self.capture_flow_stats(in_flows, route_indices, loads)
         all_out_flows, score = self.dispatch(in_flows, route_indices, loads, score)
         if self.flow_num == 1:
             all_out_flows = all_out_flows[0]
         return all_out_flows, score
+
+    def _defers(self, in_flows, runtime_capacities, hot_mask) -> bool:
+        return False  # only the fused fabric can leave the dispatch to the expert kernel
 
     def _dispatch_flow(self, flow_idx, flow_data, flow_tag, route_indices, loads, score):
         # positional layout of the reference call (generic.py:127-137): the 5th
@@ -239,7 +246,7 @@ class DispatchFabric(FabricBase):
         return c_router.dispatch_with_indices_and_loads(
             flow_data, route_indices, loads, score if self.transforms[flow_idx] else None,
             self.is_tag_index, flow_tag, self.max_path_padding, self.max_path_load,
-            self.route_logics[flow_idx] == "1d")
+            self.route_logics[flow_idx] == "1d", route=self._route)
 
     def dispatch(self, in_flows, route_indices, loads, score):
         all_out_flows = []
@@ -326,22 +333,74 @@ class CombineFabric(FabricBase):
 
 
 # ----------------------------------------------------------------------------- fused
+def _route_key(level: int) -> str:
+    return f"brt_route_{level}"
+
+
+def _deferred_key(level: int) -> str:
+    return f"brt_deferred_{level}"
+
+
 @register_fabric("fused_dispatch")
 class FusedDispatchFabric(DispatchFabric):
     """fabric/fused.py:18-75: one path-major buffer per flow (seat indices); the MoE
-    path.  Output GridTensor gets ``route_indices`` / ``loads`` pushed on its stacks."""
+    path.  Output GridTensor gets ``route_indices`` / ``loads`` pushed on its stacks and the
+    :class:`brt._C.router.Route` among its extra attributes.
+
+    ``defer_dispatch=True`` (an extension) leaves the dispatch to the expert kernel when the route
+    is single-path (a ``topk`` protocol with ``top_k=1``, ``swin_moe``, or ``switch_top1`` with
+    ``one_hot=True``): the buffer is allocated for an upper bound of the rows, not filled, and the
+    grouped GEMM of ``brt.jit`` gathers its rows from the cells directly; the stacks then carry
+    tag-format indices.  Any other use of the tensor runs the dispatch first."""
 
     def __init__(self, flow_num: int, route_logic="1d", transform=False, **kwargs):
         kwargs["index_format"] = "seat_index"
+        defer = bool(kwargs.pop("defer_dispatch", False))
+        caps = kwargs.get("supported_capacities")
         super().__init__(flow_num, route_logic=route_logic, transform=transform, **kwargs)
+        self.defer_dispatch = defer
+        self._host_caps = [caps] if isinstance(caps, int) else list(caps) if caps is not None else None
+
+    def _defers(self, in_flows, runtime_capacities, hot_mask) -> bool:
+        if not (self.defer_dispatch and getattr(hot_mask, "_brt_single_path", False)):
+            return False
+        if runtime_capacities is not None or self.max_path_padding or any(self.transforms):
+            return False
+        if any(logic != "1d" for logic in self.route_logics):
+            return False
+        for flow in in_flows:
+            if (flow.dim() != 2 or flow.dtype not in (torch.bfloat16, torch.float32)
+                    or flow.shape[1] % 8 != 0 or flow.shape[0] == 0):
+                return False
+        return True
+
+    def _row_bound(self, cells: int, paths: int) -> int:
+        """Rows the path-major layout can need, known without reading the loads back."""
+        if self._host_caps is None:
+            return cells
+        if self.path_wise_padding:
+            return sum(self._host_caps)
+        if self.capacity_padding:
+            return paths * max(self._host_caps)
+        return min(cells, paths * max(self._host_caps))
 
     def dispatch(self, in_flows, route_indices, loads, score):
         all_out_flows = []
+        deferred = self._route.is_tag_index
         for flow_idx, flow in enumerate(in_flows):
             data, tags, load_stack, extra = to_torch_tensor(flow, retrieve_attr=True)
             flow_tag = tags[-1]
             assert flow_tag is None  # fused dispatch starts from freshly annotated cells
-            (routed,) = self._dispatch_flow(flow_idx, data, flow_tag, route_indices, loads, score)
+            level = len(tags) - 1
+            extra = dict(extra or {})
+            extra[_route_key(level)] = self._route
+            if deferred:
+                data = data.contiguous()
+                routed = torch.empty((self._row_bound(data.shape[0], route_indices.shape[1]), data.shape[1]),
+                                     dtype=data.dtype, device=data.device)
+                extra[_deferred_key(level)] = DeferredState(data, self._route, routed, _deferred_key(level))
+            else:
+                (routed,) = self._dispatch_flow(flow_idx, data, flow_tag, route_indices, loads, score)
             all_out_flows.append(init_grid_tensor(
                 routed, tags[:-1] + [route_indices], load_stack[:-1] + [loads], extra))
         return all_out_flows, score
@@ -361,11 +420,39 @@ class FusedCombineFabric(CombineFabric):
             data, tags, load_stack, extra = to_torch_tensor(in_flow, retrieve_attr=True)
             residual = residual_flows[flow_idx] if residual_flows is not None else None
             route_indices, loads = tags.pop(), load_stack.pop()
-            (out,) = c_router.combine_with_indices_and_loads(
-                data, route_indices, loads, score if self.transform else None, residual,
-                max_path_padding=self.max_path_padding, ever_padded=self.ever_padded)
+            extra = dict(extra or {})
+            route = extra.pop(_route_key(len(tags)), None)
+            state = extra.pop(_deferred_key(len(tags)), None)
+            gates = score if self.transform else None
+            if route is not None and route.is_tag_index and route.owns(route_indices, loads):
+                out = self._combine_deferred(data, route, state, gates, residual)
+            else:
+                (out,) = c_router.combine_with_indices_and_loads(
+                    data, route_indices, loads, gates, residual,
+                    max_path_padding=self.max_path_padding, ever_padded=self.ever_padded, route=route)
             out_flows.append(init_grid_tensor(out, tags, load_stack, extra))
         return out_flows
+
+    def _combine_deferred(self, data, route, state, gates, residual):
+        """Combine of a route whose dispatch was deferred: tag-format indices; the row tags were
+        left on the route by the gathering GEMM (or by the dispatch, if something else read the
+        rows first)."""
+        if route.row_tags is None and state is not None:
+            state.materialize()
+        if route.row_tags is None:
+            raise RuntimeError("the rows of a deferred dispatch were never produced")
+        if data.size(0) != route.row_tags.numel():
+            raise RuntimeError("the expert output does not have the rows of the dispatched layout")
+        if gates is None and residual is not None:
+            return c_router.combine_by_row_tags(data, route.row_tags, route.cells, residual)
+        if gates is None:
+            return c_router.combine_by_row_tags(data, route.row_tags, route.cells)
+        # gate-weighted combine: the general kernel, which wants seat indices
+        seats = c_router.tag_to_seat_indices(route.indices, route.loads)
+        (out,) = c_router.combine_with_indices_and_loads(
+            data, seats, route.loads, gates, residual, max_path_padding=False,
+            ever_padded=self.ever_padded)
+        return out
 
 
 # -------------------------------------------------------------------------- identity

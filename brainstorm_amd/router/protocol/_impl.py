@@ -89,12 +89,21 @@ class TopKProtocol(ProtocolBase):
 
 @register_protocol("switch_top1")
 class SwitchTop1Protocol(ProtocolBase):
-    """protocol/switch.py:13-33: the score already is the (capacity-masked) one-hot."""
+    """protocol/switch.py:13-33: the score already is the (capacity-masked) hot mask.
 
-    single_path = True
+    ``one_hot=True`` (an extension) is the caller's promise that no row of the mask has more than
+    one nonzero, which lets the fabrics use the tag-driven combine and the deferred dispatch.  The
+    mask comes from the caller, so nothing is assumed by default: a row with several ones is
+    routed to all of them and summed, as in the reference."""
+
+    def __init__(self, one_hot: bool = False, **kwargs):
+        super().__init__(**kwargs)
+        self.single_path = bool(one_hot)
 
     def make_route_decision(self, score):
-        return score.reshape(-1, score.shape[-1]).to(torch.int32, non_blocking=True)
+        mask = score.reshape(-1, score.shape[-1]).to(torch.int32, non_blocking=True)
+        # never the caller's own tensor object: the single-path mark is set on what is returned
+        return mask.view_as(mask) if mask is score else mask
 
     def update(self, supported_capacities):
         self.supported_capacities = supported_capacities

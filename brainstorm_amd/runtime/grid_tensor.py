@@ -12,6 +12,8 @@ from typing import Any, Dict, List, Optional, Tuple, Union
 
 import torch
 
+from brainstorm_amd.runtime import deferred
+
 __all__ = [
     "GridTensor",
     "init_grid_tensor",
@@ -182,9 +184,22 @@ class GridTensor(torch.Tensor):
         # Only plain attribute reads happen before the super() call, so no torch
         # function is re-entered here.
         tags, loads, extra = collect_cell_attr(args)
+        if extra and not deferred.is_metadata_read(func):
+            _settle_deferred(args, extra)  # an unfilled dispatch buffer is filled before it is read
         ret = super().__torch_function__(func, types, args, kwargs or {})
         attach_cell_attr(ret, tags, loads, extra)
         return ret
+
+
+def _settle_deferred(args, extra) -> None:
+    if not any(isinstance(v, deferred.DeferredState) and v.pending for v in extra.values()):
+        return
+    for item in args:
+        if isinstance(item, GridTensor):
+            with torch._C.DisableTorchFunctionSubclass():
+                deferred.settle(item.__dict__.get(_EXTRA), item)
+        elif isinstance(item, (tuple, list)):
+            _settle_deferred(item, extra)
 
 
 def init_grid_tensor(tensor: torch.Tensor, tag_stack=None, load_stack=None,
@@ -202,11 +217,19 @@ def init_grid_tensor_from(tensor: torch.Tensor, from_gird_tensor: GridTensor) ->
     return init_grid_tensor(tensor, tags, loads, extra)
 
 
+def _as_plain(grid_t: torch.Tensor, extra) -> torch.Tensor:
+    """The tensor without the GridTensor subclass; an unfilled deferred dispatch buffer comes out
+    as a :class:`brainstorm_amd.runtime.deferred.DeferredRows`, which fills itself on first use."""
+    with torch._C.DisableTorchFunctionSubclass():
+        plain = grid_t.as_subclass(torch.Tensor)
+    return deferred.wrap_if_pending(plain, extra)
+
+
 def deinit_grid_tensor(grid_t: GridTensor, retrieve_attr=True):
     if not retrieve_attr:
-        return grid_t.as_subclass(torch.Tensor)
+        return _as_plain(grid_t, grid_t.__dict__.get(_EXTRA))
     grid_t, tags, loads, extra = grid_t.deep_unpack()
-    return grid_t.as_subclass(torch.Tensor), tags, loads, extra
+    return _as_plain(grid_t, extra), tags, loads, extra
 
 
 def to_grid_tensor(torch_t: torch.Tensor, tag_stack=None, load_stack=None,
@@ -219,6 +242,6 @@ def to_torch_tensor(grid_t: GridTensor, retrieve_attr=False) -> Union[torch.Tens
     """Strips the subclass (routers work on plain tensors so that nothing is
     propagated needlessly); optionally also returns the stacks."""
     if not retrieve_attr:
-        return grid_t.as_subclass(torch.Tensor)
+        return _as_plain(grid_t, grid_t.__dict__.get(_EXTRA) if isinstance(grid_t, GridTensor) else None)
     grid_t, tags, loads, extra = grid_t.copy_cell_attr()
-    return grid_t.as_subclass(torch.Tensor), tags, loads, extra
+    return _as_plain(grid_t, extra), tags, loads, extra

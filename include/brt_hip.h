@@ -241,11 +241,38 @@ int brt_hip_grouped_gemm(const void* x, const void* const* weights, const void* 
  *   overflow exactly as seat indices beyond loads[e] do, and a load padded beyond the T rows
  *   the tag matrix has (a capacity above the batch size) names empty slots.  With gather_in the cell-major
  *   input is limited to 2 GiB.
+ *   row_tags_out  NULL, or [P] int32: receives the 1-based cell behind every row of the path-major
+ *                 layout (0 for an empty slot and for the rows past sum(loads)), which is what
+ *                 brt_hip_dispatch writes as new_tags; brt_hip_combine_by_tags takes it, so a
+ *                 route that gathers in the first GEMM never runs dispatch at all.
  */
 int brt_hip_grouped_gemm_routed(const void* x, const void* const* weights,
                                 const void* const* biases, void* out, const int32_t* loads,
                                 const int32_t* tags, int E, int P, int T, int K, int N, int act,
-                                int gather_in, int scatter_out, void* stream);
+                                int gather_in, int scatter_out, int32_t* row_tags_out, void* stream);
+
+/*
+ * brt_hip_grouped_gemm with an fp32 result: out [P,N] float receives the fp32 accumulator after
+ * bias and activation, which is the output type of the reference's expert kernel
+ * (benchmark/switch_moe/switch_expert.py:74-92 allocates fp32 outputs, test/python/jit_test.py:157-203
+ * compares in fp32).  x and the weights stay bf16: brt_hip_cast_f32_to_bf16 converts fp32 operands.
+ */
+int brt_hip_grouped_gemm_f32out(const void* x, const void* const* weights, const void* const* biases,
+                                float* out, const int32_t* loads, int E, int P, int K, int N, int act,
+                                void* stream);
+/* brt_hip_grouped_gemm_routed with the fp32 result of brt_hip_grouped_gemm_f32out. */
+int brt_hip_grouped_gemm_routed_f32out(const void* x, const void* const* weights,
+                                       const void* const* biases, float* out, const int32_t* loads,
+                                       const int32_t* tags, int E, int P, int T, int K, int N, int act,
+                                       int gather_in, int scatter_out, int32_t* row_tags_out,
+                                       void* stream);
+
+/*
+ * dst[i] = bf16(src[i]) (round to nearest even), n elements; both 16-byte aligned.  For callers that
+ * hold the reference's fp32 activations or weights (no counterpart in the reference, whose kernels
+ * compute in fp32).
+ */
+int brt_hip_cast_f32_to_bf16(const float* src, void* dst, size_t n, void* stream);
 
 /*
  * The routed grouped GEMM on the compact route (no counterpart in the reference): as

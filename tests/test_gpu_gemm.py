@@ -86,8 +86,100 @@ def test_make_jit_kernel_homo_fuse_contract():
     assert torch.allclose(shared[1].float(), want, atol=2e-2, rtol=1e-2)
     with pytest.raises(NotImplementedError):
         make_jit_kernel(linears, None, opt_level="hetero_fuse")
-    with pytest.raises(NotImplementedError):
-        kernel([shared[0].float(), shared[1].float()], standalone, capacities)
+
+
+def test_make_jit_kernel_fp32_contract_of_the_reference():
+    """The reference's caller hands fp32 activations, fp32 nn.Linear parameters and a fp32
+    ``torch.empty`` output (benchmark/switch_moe/switch_expert.py:74-92; test/python/jit_test.py:157-203
+    compares against nn.Linear in fp32).  The operands are rounded to bf16, the result is the fp32
+    accumulator: within 1e-2 relative of fp32 F.linear (tolerance of bf16 operands), ragged loads, with
+    and without bias, and the cached bf16 parameters follow an in-place update of the fp32 ones."""
+    import torch.nn as nn
+    from brt.jit import make_jit_kernel
+
+    torch.manual_seed(3)
+    for bias in (True, False):
+        linears = nn.ModuleList(nn.Linear(256, 384, bias=bias) for _ in range(5)).cuda()
+        kernel = make_jit_kernel(linears, sample_inputs=[torch.randn(2 ** i, 256) for i in range(5)],
+                                 opt_level="homo_fuse")
+        loads = [33, 0, 170, 1, 40]
+        x = torch.randn(sum(loads), 256, device="cuda")
+        out = torch.empty(sum(loads), 384, device="cuda")  # fp32, as the reference allocates it
+        standalone = []
+        for lin in linears:
+            standalone += [lin.weight, lin.bias] if bias else [lin.weight]
+        capacities = torch.tensor(loads, dtype=torch.int32, device="cuda")
+        for update in (False, True):
+            if update:
+                with torch.no_grad():
+                    linears[2].weight.mul_(-0.5)
+            kernel(shared_inputs=[x, out], standalone_inputs=standalone, capacities=capacities)
+            want = torch.cat([linears[e](x[sum(loads[:e]):sum(loads[:e + 1])]) for e in range(5)])
+            assert out.dtype == torch.float32
+            assert torch.allclose(out, want, atol=1e-2 * want.abs().max().item(), rtol=1e-2), (bias, update)
+            # the fp32 output is the accumulator of the bf16 product, not a bf16 value widened
+            exact = torch.cat([
+                torch.nn.functional.linear(
+                    x[sum(loads[:e]):sum(loads[:e + 1])].to(torch.bfloat16).double(),
+                    linears[e].weight.to(torch.bfloat16).double(),
+                    linears[e].bias.to(torch.bfloat16).double() if bias else None)
+                for e in range(5)])
+            assert (out.double() - exact).abs().max().item() <= 2e-5 * exact.abs().max().item()
+
+
+def test_fp32_output_of_the_routed_forms_and_gelu():
+    """fp32 result through the C ABI: plain form with GELU against torch in fp64 on the bf16 operands,
+    and the gathering form (tag matrix) bit-identical to the plain form on dispatched rows."""
+    from brainstorm_amd._C import router as c_router
+    from brainstorm_amd.jit import grouped_linear
+
+    T, E, d, dff = 1500, 12, 128, 320
+    g = torch.Generator().manual_seed(8)
+    x = torch.randn(T, d, generator=g).to(torch.bfloat16).cuda()
+    mask = c_router.topk_hot_mask(torch.randn(T, E, generator=g).cuda(), 1)
+    w, table = _expert_tables(E, d, dff, 21)
+    route = c_router.generate_route(mask, single_path=True)
+    (y,) = c_router.dispatch_with_indices_and_loads(x, route.indices, route.loads, route=route)
+    P = y.shape[0]
+    plain = torch.empty(P, dff, device="cuda")
+    grouped_linear(y, plain, table, None, route.loads, d, dff, "gelu")
+    starts = np.concatenate([[0], np.cumsum(route.loads.cpu().numpy())])
+    for e in range(E):
+        rows = slice(int(starts[e]), int(starts[e + 1]))
+        want = torch.nn.functional.gelu(y[rows].double() @ w[e].double().t())
+        assert (plain[rows].double() - want).abs().max().item() <= 2e-5 * max(want.abs().max().item(), 1.0)
+    tags, loads_t = c_router.generate_indices_and_loads(mask, None, False, False, True)
+    gathered = torch.full((P, dff), float("nan"), device="cuda")
+    row_tags = torch.full((P,), -7, dtype=torch.int32, device="cuda")
+    grouped_linear(x, gathered, table, None, loads_t, d, dff, "gelu", tags=tags, gather=True, rows=P,
+                   row_tags_out=row_tags)
+    assert torch.equal(gathered, plain)
+    assert torch.equal(row_tags, route.row_tags)
+
+
+def test_row_tags_of_a_gathering_gemm_cover_a_layout_longer_than_the_loads():
+    """row_tags_out names the cell of every row and is 0 for padding rows and for the rows past
+    sum(loads) of a layout allocated for an upper bound (here 3 x the rows, and capacity padding)."""
+    from brainstorm_amd._C import router as c_router
+    from brainstorm_amd.jit import grouped_linear
+
+    T, E, d, n = 1000, 7, 64, 128
+    g = torch.Generator().manual_seed(9)
+    x = torch.randn(T, d, generator=g).to(torch.bfloat16).cuda()
+    mask = c_router.topk_hot_mask(torch.randn(T, E, generator=g).cuda(), 1)
+    _, table = _expert_tables(E, d, n, 22)
+    caps = torch.tensor([64, 200], dtype=torch.int32, device="cuda")
+    for pad in (False, True):
+        tags, loads = c_router.generate_indices_and_loads(mask, caps, pad, False, True)
+        seat, loads_s = c_router.generate_indices_and_loads(mask, caps, pad)
+        (y, want_tags) = c_router.dispatch_with_indices_and_loads(x, seat, loads_s, None, True)
+        rows = int(loads.sum())
+        P = 3 * T
+        out = torch.empty(P, n, dtype=torch.bfloat16, device="cuda")
+        row_tags = torch.full((P,), -7, dtype=torch.int32, device="cuda")
+        grouped_linear(x, out, table, None, loads, d, n, tags=tags, gather=True, rows=P, row_tags_out=row_tags)
+        assert torch.equal(row_tags[:rows], want_tags), pad
+        assert int(row_tags[rows:].abs().sum()) == 0, pad
 
 
 def test_full_size_switch_ffn():
@@ -310,14 +402,15 @@ def test_full_size_switch_layer_fused_equals_unfused():
     w1, t1 = _expert_tables(E, d, dff, 11)
     w2, t2 = _expert_tables(E, dff, d, 12)
     for pad in (False, True):
-        idx, loads = c_router.generate_indices_and_loads(mask, caps, pad, single_path=True)
-        (y,) = c_router.dispatch_with_indices_and_loads(x, idx, loads)
+        route = c_router.generate_route(mask, caps, pad, single_path=True)
+        idx, loads = route.indices, route.loads
+        (y,) = c_router.dispatch_with_indices_and_loads(x, idx, loads, route=route)
         P = y.shape[0]
         h = torch.empty(P, dff, dtype=torch.bfloat16, device="cuda")
         y2 = torch.empty(P, d, dtype=torch.bfloat16, device="cuda")
         grouped_linear(y, h, t1, None, loads, d, dff, "gelu")
         grouped_linear(h, y2, t2, None, loads, dff, d)
-        (want,) = c_router.combine_with_indices_and_loads(y2, idx, loads, None, x.clone())
+        (want,) = c_router.combine_with_indices_and_loads(y2, idx, loads, None, x.clone(), route=route)
         tags, _ = c_router.generate_indices_and_loads(mask, caps, pad, False, True)
         hf = torch.empty(P, dff, dtype=torch.bfloat16, device="cuda")
         out = x.clone()

@@ -152,6 +152,7 @@ def test_fused_moe_path_matches_oracle(brt_mod):
     x = torch.from_numpy(to_bf16_bits(np.random.default_rng(5).standard_normal((T, d))).view(np.int16)
                          ).cuda().view(torch.bfloat16)
     scatter = ScatterRouter(protocol_type="switch_top1", fabric_type="fused_dispatch",
+                            protocol_kwargs={"one_hot": True},
                             fabric_kwargs={"supported_capacities": [cap], "capacity_padding": True}).cuda()
     gather = GatherRouter(fabric_type="fused_combine").cuda()
     cells = brt.Annotator([0])(x)
@@ -164,7 +165,9 @@ def test_fused_moe_path_matches_oracle(brt_mod):
     o_y, _ = oracle.dispatch(xb, o_idx, o_loads, dtype="bf16")
     assert np.array_equal(brt.to_torch_tensor(routed).view(torch.int16).cpu().numpy().view(np.uint16), o_y)
     # a single-path protocol: dispatch left the per-row tags for the tag-driven combine
-    tags = loads._brt_pairing.row_tags
+    route = routed.extra_attr_dict["brt_route_0"]
+    assert route.owns(idx, loads) and route.single_path
+    tags = route.row_tags
     assert tags is not None and np.array_equal(
         tags.cpu().numpy(), oracle.dispatch(xb, o_idx, o_loads, tag_generating=True, dtype="bf16")[1])
     expert_out = routed * 2  # stacks travel through the expert
@@ -188,7 +191,7 @@ def test_fused_moe_path_top2_keeps_the_gather_combine(brt_mod):
     gather = GatherRouter(fabric_type="fused_combine").cuda()
     routed = scatter(brt.Annotator([0])(x), score)
     idx, loads = routed.tag, routed.load
-    assert loads._brt_pairing.row_tags is None
+    assert routed.extra_attr_dict["brt_route_0"].row_tags is None
     residual = torch.zeros_like(x)
     out = gather(routed * 1.0, residual)
     o_mask = (idx.cpu().numpy() > 0).astype(np.int32)
@@ -199,7 +202,7 @@ def test_fused_moe_path_top2_keeps_the_gather_combine(brt_mod):
     # same routers with top_k=1 take the tag-driven path and agree with the oracle too
     scatter1 = ScatterRouter(protocol_type="topk", fabric_type="fused_dispatch").cuda()
     routed1 = scatter1(brt.Annotator([0])(x), score)
-    assert routed1.load._brt_pairing.row_tags is not None
+    assert routed1.extra_attr_dict["brt_route_0"].row_tags is not None
     res1 = torch.full_like(x, 3.0)
     i1, l1 = routed1.tag.cpu().numpy(), routed1.load.cpu().numpy()
     out1 = gather(routed1 * 1.0, res1)
@@ -482,3 +485,114 @@ def test_row_buffers_beyond_two_gib(brt_mod):
     del y2
     back2 = ops.combine_by_rows(y, ids, seat_rows)
     assert torch.equal(back2.view(torch.int16), x.view(torch.int16))
+
+
+def _switch_layer(brt_mod, defer, E, d, dff, cap, pad, dtype, seed):
+    """ScatterRouter(fused_dispatch) -> two homo-fused kernels -> GatherRouter(fused_combine), written
+    as benchmark/switch_moe/switch_transformer.py:336-380 and switch_expert.py:62-99 write it."""
+    brt, _, ScatterRouter, GatherRouter = brt_mod
+    from brt.jit import make_jit_kernel
+
+    torch.manual_seed(seed)
+    wi = nn.ModuleList(nn.Linear(d, dff, bias=False) for _ in range(E)).cuda().to(dtype)
+    wo = nn.ModuleList(nn.Linear(dff, d, bias=False) for _ in range(E)).cuda().to(dtype)
+    fabric_kwargs = {"supported_capacities": [cap], "capacity_padding": pad}
+    if defer:
+        fabric_kwargs["defer_dispatch"] = True
+    scatter = ScatterRouter(protocol_type="topk", fabric_type="fused_dispatch",
+                            fabric_kwargs=fabric_kwargs).cuda()
+    gather = GatherRouter(fabric_type="fused_combine").cuda()
+    fused_wi = make_jit_kernel(wi, None, opt_level="homo_fuse", activation="gelu")
+    fused_wo = make_jit_kernel(wo, None, opt_level="homo_fuse")
+    annotator = brt.Annotator([0])
+
+    def layer(hidden, score):
+        routed = scatter(annotator(hidden), score)
+        states, tags, loads, extra = brt.to_torch_tensor(routed, retrieve_attr=True)
+        wi_out = torch.empty((states.shape[0], dff), device=states.device, dtype=states.dtype)
+        fused_wi(shared_inputs=[states, wi_out], standalone_inputs=[m.weight for m in wi], capacities=loads[-1])
+        wo_out = torch.empty((states.shape[0], d), device=states.device, dtype=states.dtype)
+        fused_wo(shared_inputs=[wi_out, wo_out], standalone_inputs=[m.weight for m in wo], capacities=loads[-1])
+        return brt.to_torch_tensor(gather(brt.to_grid_tensor(wo_out, tags, loads, extra), hidden))
+
+    return layer
+
+
+@pytest.mark.parametrize("pad", [False, True])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_deferred_fused_dispatch_is_the_same_layer_in_four_launches(brt_mod, pad, dtype):
+    """defer_dispatch=True: the expert's first kernel gathers its rows from the cells, no dispatch
+    kernel runs.  Same caller code, bit-identical result, and the layer is four calls into the
+    library (index generation, two grouped GEMMs, the tag-driven combine) against five."""
+    from brainstorm_amd import _lib
+
+    T, E, d, dff, cap = 2048, 16, 256, 512, 160
+    g = torch.Generator().manual_seed(31)
+    hidden = torch.randn(T, d, generator=g).to(dtype).cuda()
+    score = torch.randn(T, E, generator=g).cuda()
+    results, calls = [], []
+    for defer in (False, True):
+        layer = _switch_layer(brt_mod, defer, E, d, dff, cap, pad, dtype, seed=32)
+        layer(hidden.clone(), score)  # parameter copies, pointer tables, workspaces
+        residual = hidden.clone()
+        before = _lib.call_count()
+        results.append(layer(residual, score))
+        calls.append(_lib.call_count() - before)
+        assert results[-1].data_ptr() == residual.data_ptr()  # combined in place, as the reference does
+    # topk mask, index generation, [dispatch,] (casts of fp32 operands,) GEMM, GEMM, combine
+    casts = 2 if dtype == torch.float32 else 0
+    assert calls[0] == 6 + casts and calls[1] == 5 + casts, calls
+    assert torch.equal(results[0], results[1])
+    assert not torch.equal(results[0], hidden)
+
+
+def test_deferred_rows_fill_themselves_when_anything_else_reads_them(brt_mod):
+    """Any use of a deferred buffer other than the grouped GEMM runs the dispatch it stands for."""
+    brt, c_router, ScatterRouter, GatherRouter = brt_mod
+    T, E, d = 777, 5, 64
+    g = torch.Generator().manual_seed(41)
+    x = torch.randn(T, d, generator=g).to(torch.bfloat16).cuda()
+    score = torch.randn(T, E, generator=g).cuda()
+    scatter = ScatterRouter(protocol_type="topk", fabric_type="fused_dispatch",
+                            fabric_kwargs={"defer_dispatch": True}).cuda()
+    plain = ScatterRouter(protocol_type="topk", fabric_type="fused_dispatch").cuda()
+    gather = GatherRouter(fabric_type="fused_combine").cuda()
+    want = brt.to_torch_tensor(plain(brt.Annotator([0])(x), score))
+    rows = want.shape[0]
+    # through the GridTensor
+    routed = scatter(brt.Annotator([0])(x), score)
+    assert routed.shape == (T, d) and routed.extra_attr_dict["brt_deferred_0"].pending
+    doubled = routed * 2
+    assert not routed.extra_attr_dict["brt_deferred_0"].pending
+    assert torch.equal(brt.to_torch_tensor(doubled)[:rows], want * 2)
+    assert int(brt.to_torch_tensor(doubled)[rows:].abs().sum()) == 0
+    out = gather(doubled, torch.zeros_like(x))
+    assert torch.equal(brt.to_torch_tensor(out), x * 2)
+    # through the plain tensor the expert takes out of it
+    routed = scatter(brt.Annotator([0])(x), score)
+    states, tags, loads, extra = brt.to_torch_tensor(routed, retrieve_attr=True)
+    assert extra["brt_deferred_0"].pending and states.shape[0] == T and states.is_cuda
+    assert extra["brt_deferred_0"].pending  # shape, device: nothing ran
+    total = states.float().sum()
+    assert not extra["brt_deferred_0"].pending
+    assert torch.allclose(total, want.float().sum())
+
+
+def test_switch_top1_sums_a_cell_that_is_on_two_paths(brt_mod):
+    """switch_top1 takes the caller's mask as it is: without one_hot=True a row with two ones goes
+    to both paths and the combine adds the two rows (fused path, as the reference does)."""
+    brt, c_router, ScatterRouter, GatherRouter = brt_mod
+    T, E, d = 64, 4, 32
+    x = torch.randn(T, d, device="cuda")
+    mask = torch.zeros(T, E, dtype=torch.int32, device="cuda")
+    mask[torch.arange(T), torch.arange(T) % E] = 1
+    mask[5, :2] = 1
+    mask[5, 2:] = 0
+    scatter = ScatterRouter(protocol_type="switch_top1", fabric_type="fused_dispatch").cuda()
+    gather = GatherRouter(fabric_type="fused_combine").cuda()
+    routed = scatter(brt.Annotator([0])(x), mask)
+    assert not hasattr(mask, "_brt_single_path")  # the caller's tensor is left alone
+    out = brt.to_torch_tensor(gather(routed * 1.0, torch.zeros_like(x)))
+    want = x.clone()
+    want[5] = x[5] + x[5]
+    assert torch.equal(out, want)
