@@ -290,11 +290,16 @@ def dispatch_with_indices_and_loads(
     is_tag_index: bool = False,
     *,
     route: Optional[Route] = None,
+    rows: Optional[int] = None,
 ) -> List[torch.Tensor]:
     """router.cc:131-273.  Returns ``[out]`` or ``[out, new_tags]``.  ``route`` (keyword only,
     not in the reference): the :class:`Route` the indices came from; the kernel then zero-fills
     only the padding rows of an un-zeroed output and, for single-path routes, leaves the per-row
-    tags on the route for the combine."""
+    tags on the route for the combine.  ``rows`` (keyword only, not in the reference): an upper
+    bound of ``sum(loads)`` known to the caller; the output then has that many rows (those past
+    the loads are zero) and the loads are not read back to the host (router.cc:197-201 sizes
+    the output from ``loads.sum().item()``, which stalls the stream; that is what happens without
+    ``rows``)."""
     _check_on_device(in_data, "in_data")
     _check_on_device(route_indices, "route_indices")
     _check_int32(route_indices, "route_indices")
@@ -337,6 +342,8 @@ def dispatch_with_indices_and_loads(
         if max_path_padding:
             mpl = int(max_path_load) if max_path_load > 0 else int(loads.max().item())
             total = mpl * E
+        elif rows is not None:
+            total = int(rows)
         else:
             total = int(loads.sum().item())
 
@@ -350,7 +357,9 @@ def dispatch_with_indices_and_loads(
                 shape.append(1)
             shape[1] = total
             shape = shape[1:]
-        alloc = torch.empty if counts is not None else torch.zeros
+        # with the true counts the kernel writes every row up to sum(loads) itself; rows past that
+        # (an upper bound was given) have no writer
+        alloc = torch.empty if counts is not None and (rows is None or max_path_padding) else torch.zeros
         out = alloc(shape, dtype=in_data.dtype, device=device)
 
         dev_gates = None

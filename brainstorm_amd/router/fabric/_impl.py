@@ -246,7 +246,11 @@ class DispatchFabric(FabricBase):
         return c_router.dispatch_with_indices_and_loads(
             flow_data, route_indices, loads, score if self.transforms[flow_idx] else None,
             self.is_tag_index, flow_tag, self.max_path_padding, self.max_path_load,
-            self.route_logics[flow_idx] == "1d", route=self._route)
+            self.route_logics[flow_idx] == "1d", route=self._route,
+            rows=self._static_rows(flow_data, route_indices))
+
+    def _static_rows(self, flow_data, route_indices) -> Optional[int]:
+        return None  # size the output from the loads, as the reference does
 
     def dispatch(self, in_flows, route_indices, loads, score):
         all_out_flows = []
@@ -351,14 +355,18 @@ class FusedDispatchFabric(DispatchFabric):
     is single-path (a ``topk`` protocol with ``top_k=1``, ``swin_moe``, or ``switch_top1`` with
     ``one_hot=True``): the buffer is allocated for an upper bound of the rows, not filled, and the
     grouped GEMM of ``brt.jit`` gathers its rows from the cells directly; the stacks then carry
-    tag-format indices.  Any other use of the tensor runs the dispatch first."""
+    tag-format indices.  Any other use of the tensor runs the dispatch first.
+    ``static_rows=True`` (an extension) keeps the dispatch but sizes its output the same way, so
+    that nothing is read back to the host."""
 
     def __init__(self, flow_num: int, route_logic="1d", transform=False, **kwargs):
         kwargs["index_format"] = "seat_index"
         defer = bool(kwargs.pop("defer_dispatch", False))
+        static_rows = bool(kwargs.pop("static_rows", False))
         caps = kwargs.get("supported_capacities")
         super().__init__(flow_num, route_logic=route_logic, transform=transform, **kwargs)
         self.defer_dispatch = defer
+        self.static_rows = static_rows
         self._host_caps = [caps] if isinstance(caps, int) else list(caps) if caps is not None else None
 
     def _defers(self, in_flows, runtime_capacities, hot_mask) -> bool:
@@ -374,8 +382,16 @@ class FusedDispatchFabric(DispatchFabric):
                 return False
         return True
 
+    def _static_rows(self, flow_data, route_indices) -> Optional[int]:
+        """``static_rows=True`` (an extension): the output is allocated for the rows the layout can
+        need at most, and the loads are never read back to the host (no stall of the stream); the
+        reference sizes it from ``loads.sum().item()`` (router.cc:197-201), which is the default."""
+        if not self.static_rows or self.max_path_padding or self._route is None or not self._route.single_path:
+            return None
+        return self._row_bound(flow_data.shape[0], route_indices.shape[1])
+
     def _row_bound(self, cells: int, paths: int) -> int:
-        """Rows the path-major layout can need, known without reading the loads back."""
+        """Rows the path-major layout of a single-path route can need, known without reading the loads back."""
         if self._host_caps is None:
             return cells
         if self.path_wise_padding:
@@ -622,7 +638,7 @@ class DistributedFusedDispatchFabric(FusedDispatchFabric):
             (routed,) = c_router.dispatch_with_indices_and_loads(
                 data, route_indices, loads, score if self.transforms[flow_idx] else None,
                 False, None, self.max_path_padding, self.max_path_load,
-                self.route_logics[flow_idx] == "1d")
+                self.route_logics[flow_idx] == "1d", route=self._route)
             if self.task_locality:  # world of one: path i holds task i
                 host_loads = loads.cpu().tolist()
                 score = torch.repeat_interleave(

@@ -596,3 +596,142 @@ def test_switch_top1_sums_a_cell_that_is_on_two_paths(brt_mod):
     want = x.clone()
     want[5] = x[5] + x[5]
     assert torch.equal(out, want)
+
+
+def test_static_rows_dispatch_reads_nothing_back(brt_mod):
+    """rows=: the output is sized from the caller's bound, the rows past the loads are zero, the
+    routed rows are the reference's; the fused fabric does the same with static_rows=True."""
+    brt, c_router, ScatterRouter, GatherRouter = brt_mod
+    T, E, d, cap = 1500, 6, 64, 300
+    mask, logits = topk_mask(T, E, 1, seed=51)
+    x = torch.randn(T, d, device="cuda")
+    caps = torch.tensor([cap], dtype=torch.int32, device="cuda")
+    for pad in (False, True):
+        route = c_router.generate_route(torch.from_numpy(mask).cuda(), caps, pad, single_path=True)
+        (want,) = c_router.dispatch_with_indices_and_loads(x, route.indices, route.loads, route=route)
+        bound = E * cap if pad else T
+        (got,) = c_router.dispatch_with_indices_and_loads(x, route.indices, route.loads, route=route, rows=bound)
+        rows = want.shape[0]
+        assert got.shape[0] == bound and torch.equal(got[:rows], want) and int(got[rows:].abs().sum()) == 0
+        (plain,) = c_router.dispatch_with_indices_and_loads(x, route.indices, route.loads, rows=bound)
+        assert torch.equal(plain, got)
+    score = torch.from_numpy(softmax(logits).astype(np.float32)).cuda()
+    layer_out = []
+    for static in (False, True):
+        scatter = ScatterRouter(protocol_type="topk", fabric_type="fused_dispatch",
+                                fabric_kwargs={"supported_capacities": [cap], "capacity_padding": True,
+                                               "static_rows": static}).cuda()
+        gather = GatherRouter(fabric_type="fused_combine").cuda()
+        routed = scatter(brt.Annotator([0])(x), score)
+        assert routed.shape[0] == (E * cap if static else int(routed.load.sum()))
+        layer_out.append(brt.to_torch_tensor(gather(routed * 3.0, x.clone())))
+    assert torch.equal(layer_out[0], layer_out[1])
+
+
+def test_identity_fabrics_on_the_gpu(brt_mod):
+    """identity_dispatch: every path sees the whole flow (scaled by its score column with
+    transform); identity_combine: the sum of the paths and the residual
+    (fabric/identity.py:12-111).  With one flow the reference's forward returns the list of flows
+    wrapped once more and no score (identity.py:44-47), which ScatterRouter cannot unpack; the
+    fabrics are driven directly here, and through the router with two flows."""
+    brt, _, ScatterRouter, GatherRouter = brt_mod
+    from brt.router.fabric import make_fabric
+
+    T, E, d = 300, 3, 40
+    x = torch.randn(T, d, device="cuda")
+    score = torch.rand(T, E, device="cuda")
+    cells = brt.Annotator([0])(x)
+    (flows,) = make_fabric("identity_dispatch", {"path_num": E, "flow_num": 1}).cuda()(cells, None, None, score)
+    assert len(flows) == E and all(torch.equal(brt.to_torch_tensor(f), x) for f in flows)
+    (wflows,) = make_fabric("identity_dispatch", {"path_num": E, "flow_num": 1, "transform": True}).cuda()(
+        cells, None, None, score)
+    for e in range(E):
+        assert torch.equal(brt.to_torch_tensor(wflows[e]), x * score[:, e:e + 1])
+    scatter = ScatterRouter(dispatch_score=True, protocol_type="identity", fabric_type="identity_dispatch",
+                            fabric_kwargs={"path_num": E}).cuda()
+    routed, routed_score = scatter(cells, score)
+    assert all(torch.equal(brt.to_torch_tensor(f), x) for f in routed)
+    assert all(torch.equal(brt.to_torch_tensor(routed_score[e]), score[:, e].contiguous()) for e in range(E))
+    gather = GatherRouter(fabric_type="identity_combine").cuda()
+    # identity_combine adds up every cell of every path and of the residual into one cell
+    # (identity.py:104-108: cat, reshape(-1, 1, ...), sum over dim 0); for the batches of one cell
+    # it is used with, that is the element-wise sum of the paths
+    out = gather([f * (e + 1) for e, f in enumerate(flows)], x)
+    want = (torch.cat([x * (e + 1) for e in range(E)] + [x]).double().sum(0, keepdim=True)).float()
+    assert tuple(out.shape) == (1, d)
+    assert torch.allclose(brt.to_torch_tensor(out), want, rtol=1e-4, atol=1e-3)
+    one = torch.randn(1, d, device="cuda")
+    out1 = gather([one * 1.0, one * 2.0, one * 3.0], one)
+    assert torch.allclose(brt.to_torch_tensor(out1), one * 7.0, rtol=1e-6, atol=1e-6)
+
+
+def test_placeholder_combine_gives_empty_flows_of_the_recorded_shape(brt_mod):
+    _, _, _, GatherRouter = brt_mod
+    dev = torch.device("cuda", torch.cuda.current_device())
+    gather = GatherRouter(fabric_type="placeholder_combine",
+                          fabric_kwargs={"runtime_load": 0, "cell_grains": [torch.Size([1, 12, 5])],
+                                         "cell_dtypes": [torch.float16], "cell_devices": [dev]}).cuda()
+    out = gather([torch.randn(4, 12, 5, device="cuda")])
+    assert tuple(out.shape) == (0, 12, 5) and out.dtype == torch.float16 and out.device == dev
+
+
+def test_distributed_fused_fabrics_in_a_world_of_one(brt_mod):
+    """distributed_fused_dispatch / _combine on one process: the exchange is the identity, so the
+    pair equals the fused pair (fabric/distributed.py:14-158 with world size 1), against the oracle."""
+    brt, c_router, ScatterRouter, GatherRouter = brt_mod
+    T, E, d, cap = 1200, 8, 96, 180
+    mask, logits = topk_mask(T, E, 1, seed=61)
+    score = torch.from_numpy(softmax(logits).astype(np.float32)).cuda()
+    x = torch.from_numpy(np.random.default_rng(61).standard_normal((T, d)).astype(np.float32)).cuda()
+    scatter = ScatterRouter(protocol_type="topk", fabric_type="distributed_fused_dispatch",
+                            fabric_kwargs={"supported_capacities": [cap], "capacity_padding": True}).cuda()
+    gather = GatherRouter(fabric_type="distributed_fused_combine").cuda()
+    routed = scatter(brt.Annotator([0])(x), score)
+    o_idx, o_loads = oracle.generate_indices_and_loads(mask, [cap], True)
+    o_y, _ = oracle.dispatch(x.cpu().numpy(), o_idx, o_loads)
+    assert np.array_equal(brt.to_torch_tensor(routed).cpu().numpy(), o_y)
+    assert np.array_equal(routed.load.cpu().numpy(), o_loads)
+    out = gather(routed * 0.5, x.clone())
+    o_out = oracle.combine(o_y * np.float32(0.5), o_idx, o_loads, out_data=x.cpu().numpy().copy())
+    assert np.array_equal(brt.to_torch_tensor(out).cpu().numpy(), o_out)
+
+
+def test_task_hash_and_label_protocols_route_on_the_gpu(brt_mod):
+    """task: cell of task i goes to path i; hash: to two fixed paths; label: to its label
+    (protocol/hashed.py:15-91, label.py:13-33) -- masks against their closed forms, then through
+    dispatch and combine against the oracle."""
+    brt, c_router, ScatterRouter, GatherRouter = brt_mod
+    from brt.router.protocol import make_protocol
+
+    T, tasks, d = 500, 6, 32
+    rng = np.random.default_rng(71)
+    ids = torch.from_numpy(rng.integers(0, tasks, T)).cuda()
+    x = torch.from_numpy(rng.standard_normal((T, d)).astype(np.float32)).cuda()
+    task = make_protocol("task", {"num_tasks": tasks}).cuda()
+    mask = task(ids)
+    want = np.zeros((T, tasks), dtype=np.int32)
+    want[np.arange(T), ids.cpu().numpy()] = 1
+    assert mask.dtype == torch.int32 and np.array_equal(mask.cpu().numpy(), want)
+    for placement_aware in (True, False):
+        proto = make_protocol("hash", {"num_tasks": tasks, "placement_aware": placement_aware, "seed": 3}).cuda()
+        hmask = proto(ids).cpu().numpy()
+        table = proto.hash_indices.cpu().numpy()
+        hwant = np.zeros((T, tasks), dtype=np.int32)
+        for t, i in enumerate(ids.cpu().numpy()):
+            hwant[t, table[i]] = 1
+        assert np.array_equal(hmask, hwant)
+        if placement_aware:
+            assert np.array_equal(table[:, 1], (table[:, 0] + 1) % tasks)
+    label = make_protocol("label", {"path_num": tasks}).cuda()
+    assert np.array_equal(label(ids).cpu().numpy(), want)
+    # the task router end to end (TaskScatterRouter returns the flows and the task ids)
+    from brt.router import TaskScatterRouter
+    scatter = TaskScatterRouter(protocol_type="task", fabric_type="fused_dispatch",
+                                protocol_kwargs={"num_tasks": tasks}).cuda()
+    gather = GatherRouter(fabric_type="fused_combine").cuda()
+    routed, _ = scatter(brt.Annotator([0])(x), ids)
+    o_idx, o_loads = oracle.generate_indices_and_loads(want)
+    o_y, _ = oracle.dispatch(x.cpu().numpy(), o_idx, o_loads)
+    assert np.array_equal(brt.to_torch_tensor(routed).cpu().numpy(), o_y)
+    out = gather(routed * 2.0, torch.zeros_like(x))
+    assert np.array_equal(brt.to_torch_tensor(out).cpu().numpy(), x.cpu().numpy() * 2)
