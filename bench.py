@@ -50,7 +50,7 @@ RING_BYTES = 768 << 20      # what one kernel touches going once round a ring of
 T, D, E, DFF = 8192, 768, 64, 3072
 CAPACITY = int(1.25 * (T // E))  # 160
 SEED = 2
-PHASES = ("all", "step", "instep", "cold", "warm", "ffn", "configs", "extras")
+PHASES = ("all", "step", "instep", "cold", "warm", "ffn", "configs", "extras", "api")
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "switch_moe_8k_pmc_traffic.md")
 
 
@@ -763,6 +763,64 @@ def phase_extras(gpu, layer, steps):
     return extras
 
 
+def phase_api(gpu, layer, steps):
+    """The same layer driven through the drop-in Python API -- ScatterRouter(fused_dispatch), two
+    make_jit_kernel(..., "homo_fuse") kernels, GatherRouter(fused_combine), written as the
+    reference's Switch layer writes it (benchmark/switch_moe/switch_transformer.py:336-380,
+    switch_expert.py:62-99) -- captured into one HIP graph of K steps, so what is timed is the
+    device work the API issues, not the interpreter.  Two fabrics: static_rows (dispatch kernel,
+    output sized without reading the loads back, which a graph capture could not do) and
+    defer_dispatch (the first GEMM gathers its rows, no dispatch kernel)."""
+    torch = gpu.torch
+    import torch.nn as nn
+
+    import brt
+    from brt.jit import make_jit_kernel
+    from brt.router import GatherRouter, ScatterRouter
+
+    x = layer.sets[0]["x"]
+    score = layer.probs.to(gpu.dev)  # the router probabilities; the topk protocol takes the arg-max path
+    wi = nn.ModuleList(nn.Linear(D, DFF, bias=False) for _ in range(E))
+    wo = nn.ModuleList(nn.Linear(DFF, D, bias=False) for _ in range(E))
+    for e in range(E):  # the benchmark's weights
+        wi[e].weight = nn.Parameter(layer.wi[e], requires_grad=False)
+        wo[e].weight = nn.Parameter(layer.wo[e], requires_grad=False)
+    fused_wi = make_jit_kernel(wi, None, opt_level="homo_fuse", activation="gelu")
+    fused_wo = make_jit_kernel(wo, None, opt_level="homo_fuse")
+    wi_w, wo_w = [m.weight for m in wi], [m.weight for m in wo]
+    annotator = brt.Annotator([0])
+    out = {}
+    results = {}
+    for name, kwargs in (("static_rows", {"static_rows": True}), ("defer_dispatch", {"defer_dispatch": True})):
+        scatter = ScatterRouter(protocol_type="topk", fabric_type="fused_dispatch",
+                                fabric_kwargs={"supported_capacities": [CAPACITY], **kwargs}).to(gpu.dev)
+        gather = GatherRouter(fabric_type="fused_combine").to(gpu.dev)
+        residual = x.clone()
+
+        def step():
+            routed = scatter(annotator(x), score)
+            states, tags, loads, extra = brt.to_torch_tensor(routed, retrieve_attr=True)
+            h = torch.empty((states.shape[0], DFF), device=states.device, dtype=states.dtype)
+            fused_wi(shared_inputs=[states, h], standalone_inputs=wi_w, capacities=loads[-1])
+            y = torch.empty((states.shape[0], D), device=states.device, dtype=states.dtype)
+            fused_wo(shared_inputs=[h, y], standalone_inputs=wo_w, capacities=loads[-1])
+            gather(brt.to_grid_tensor(y, tags, loads, extra), residual)
+
+        before = gpu._lib.call_count()
+        gpu.run(step)
+        calls = gpu._lib.call_count() - before
+        results[name] = residual.clone()
+        graph = gpu.capture(step, steps)
+        gpu.timed(graph, 1)
+        us = min(gpu.timed(graph, 1) for _ in range(3)) * 1e3 / steps
+        out[name] = {"layer_us": round(us, 2), "library_calls_per_layer": calls}
+    if not torch.equal(results["static_rows"], results["defer_dispatch"]):
+        raise SystemExit("bench: the deferred dispatch changed the layer's result")
+    out["note"] = ("library calls per layer include the gate's top-k mask kernel; index generation is "
+                   "two kernels in one call.  Both forms give bit-identical results (checked here)")
+    return out
+
+
 def cpu_baseline(layer):
     import numpy as np
     import torch
@@ -852,6 +910,9 @@ def main():
                 entry["mfma_frac"] = round(flops[name] / t_us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4)
             out[name] = entry
         return out
+
+    if want("api"):
+        result["layer_through_router_api"] = phase_api(gpu, layer, args.steps)
 
     if want("instep"):
         us, event_us = phase_instep(gpu, layer, args.steps)

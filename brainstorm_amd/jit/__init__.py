@@ -58,7 +58,7 @@ def grouped_linear(x: torch.Tensor, out: torch.Tensor, weight_table: torch.Tenso
     GEMM: ``gather=True`` reads row s of branch e from ``x[tags[s, e] - 1]`` (``x`` is the
     cell-major tensor, no dispatch needed), ``scatter=True`` stores it to
     ``out[tags[s, e] - 1]`` (``out`` is cell-major and doubles as the residual; single-path
-    routes only).  ``rows`` bounds ``sum(loads)`` when neither side is path-major.
+    routes only).  ``rows`` bounds ``sum(loads)``; it must be given when neither side is path-major.
 
     ``row_entries`` (the vector ``route_by_path`` writes: 1-based entry ``t * k + j + 1`` of every
     row of the dispatched layout, ``k = entries_per_cell``) names the rows instead of ``tags``:
@@ -102,9 +102,11 @@ def grouped_linear(x: torch.Tensor, out: torch.Tensor, weight_table: torch.Tenso
         if (gather and x.shape[0] != cells) or (scatter and out.shape[0] != cells):
             raise RuntimeError("a gathered input / scattered output has one row per cell")
     if rows is None:
-        # both sides cell-major: at most one row per cell and path, and never more than the tag
-        # matrix has slots for
-        rows = out.shape[0] if not scatter else (x.shape[0] if not gather else tags.numel())
+        if gather and scatter:
+            # neither side is path-major, so nothing bounds the rows but the caller: the slots of
+            # the tag matrix would launch a grid that is almost all empty row blocks
+            raise RuntimeError("rows (an upper bound of sum(loads)) is needed when x is gathered and out scattered")
+        rows = out.shape[0] if not scatter else x.shape[0]
     elif (not gather and rows > x.shape[0]) or (not scatter and rows > out.shape[0]):
         raise RuntimeError("rows exceeds the path-major buffer")
     if not routed and x.shape[0] != out.shape[0]:

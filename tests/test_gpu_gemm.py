@@ -376,7 +376,9 @@ def test_routed_gemm_argument_checks():
     tags = torch.arange(1, 9, dtype=torch.int32, device="cuda").view(8, 1)
     with pytest.raises(RuntimeError):
         grouped_linear(x[:4], out, table, None, loads, 64, 64, tags=tags, gather=True)  # x not cell-major
-    grouped_linear(x, out, table, None, loads, 64, 64, tags=tags, gather=True, scatter=True)
+    with pytest.raises(RuntimeError):                                     # nothing bounds the rows
+        grouped_linear(x, out, table, None, loads, 64, 64, tags=tags, gather=True, scatter=True)
+    grouped_linear(x, out, table, None, loads, 64, 64, tags=tags, gather=True, scatter=True, rows=8)
     entries = torch.arange(1, 17, dtype=torch.int32, device="cuda")        # 8 cells x 2 entries
     with pytest.raises(NotImplementedError):                              # scatter needs one path per cell
         grouped_linear(x, out, table, None, loads, 64, 64, row_entries=entries, entries_per_cell=2,
