@@ -61,7 +61,110 @@ def parse():
     p.add_argument("--warmup", type=int, default=20)
     p.add_argument("--only", choices=PHASES, default="all")
     p.add_argument("--no-cpu-baseline", action="store_true")
+    p.add_argument("--summarize-pmc", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
+                   help="print the profiles/ summary of two rocprofv3 --pmc runs of this file "
+                        "(FETCH_SIZE, then WRITE_SIZE: their *_counter_collection.csv) and exit")
+    p.add_argument("--summarize-trace", nargs="+", metavar="LABEL=STATS_CSV",
+                   help="print the profiles/ summary of rocprofv3 --kernel-trace --stats runs of this "
+                        "file (their *_kernel_stats.csv, one per phase) and exit")
+    p.add_argument("--commit", default="unknown", help="commit the profiled tree was at (for the summaries)")
     return p.parse_args()
+
+
+# kernels of the benchmark step -> the names bench.py reports them under
+def _kernel_key(name):
+    if "dispatch_lean_kernel" in name or "dispatch_kernel" in name or "dispatch_small_kernel" in name:
+        return "dispatch"
+    if "combine_rows_kernel" in name:
+        return "combine"
+    if "combine_lean_kernel" in name:
+        return "combine_gather"
+    if "band_count_kernel" in name:
+        return "indexgen_count"
+    if "band_apply_kernel" in name:
+        return "indexgen_apply"
+    m = re.search(r"grouped_gemm_kernel<\s*\d+,\s*\d+,\s*\d+,\s*(\d+)", name)
+    if m:
+        return "ffn_gemm1_gelu" if m.group(1) == "1" else "ffn_gemm2"
+    return None
+
+
+def summarize_pmc(fetch_csv, write_csv, commit):
+    """Markdown summary of two counter runs: median FETCH_SIZE / WRITE_SIZE per kernel, scaled to
+    KiB by what the same counters read for the plain 12 MiB device copy the benchmark launches
+    (`y.copy_(x[:P])`), and the line bench.py reads back."""
+    import csv
+    import statistics
+
+    def medians(path):
+        per = {}
+        with open(path) as f:
+            for row in csv.DictReader(f):
+                per.setdefault(row["Kernel_Name"], []).append(float(row["Counter_Value"]))
+        return {k: (statistics.median(v), len(v)) for k, v in per.items()}
+
+    fetch, write = medians(fetch_csv), medians(write_csv)
+    copy_kib = T * D * 2 / 1024
+    copies = [k for k in fetch if "copyBuffer" in k or "copy_kernel" in k.lower() or "CopyFunctor" in k]
+    cal = {}
+    for label, table in (("fetch", fetch), ("write", write)):
+        vals = [table[k][0] for k in copies if k in table and 0.4 * copy_kib <= table[k][0] <= 1.1 * copy_kib]
+        cal[label] = copy_kib / statistics.median(vals) if vals else float("nan")
+    print("# rocprofv3 PMC: HBM traffic per launch, Switch-MoE layer hot path (bench.py default workload)\n")
+    print("Commands (one counter per run; the summary is printed by `bench.py --summarize-pmc`):\n")
+    print("    rocprofv3 --pmc FETCH_SIZE --output-format csv -d <dir_f> -o s -- python3 bench.py --steps 20 --warmup 2 --no-cpu-baseline")
+    print("    rocprofv3 --pmc WRITE_SIZE --output-format csv -d <dir_w> -o s -- python3 bench.py --steps 20 --warmup 2 --no-cpu-baseline")
+    print("    python3 bench.py --summarize-pmc <dir_f>/.../s_counter_collection.csv <dir_w>/.../s_counter_collection.csv --commit <hash>\n")
+    print(f"Calibration: the device-to-device copy of the {copy_kib:.0f} KiB of rows reads FETCH_SIZE x "
+          f"{cal['fetch']:.3f} = {copy_kib:.0f} KiB and WRITE_SIZE x {cal['write']:.3f} = {copy_kib:.0f} KiB; "
+          "every counter below is scaled by these factors.\n")
+    print("| kernel | launches | FETCH_SIZE (raw median) | WRITE_SIZE (raw median) | read KiB | written KiB |")
+    print("|---|---|---|---|---|---|")
+    traffic = {}
+    for name in sorted(set(fetch) | set(write)):
+        key = _kernel_key(name)
+        if key is None and "brt::" not in name:
+            continue
+        f, n = fetch.get(name, (float("nan"), 0))
+        w, _ = write.get(name, (float("nan"), 0))
+        rk, wk = f * cal["fetch"], w * cal["write"]
+        short = re.sub(r"^void |brt::\(anonymous namespace\)::|\(brt::\w+\)$", "", name)
+        print(f"| `{short[:90]}` | {n} | {f:.1f} | {w:.1f} | {rk:.0f} | {wk:.0f} |")
+        if key is not None:
+            traffic[key] = traffic.get(key, 0) + int(round((rk + wk) * 1024))
+    if "indexgen_count" in traffic or "indexgen_apply" in traffic:
+        traffic["indexgen"] = traffic.pop("indexgen_count", 0) + traffic.pop("indexgen_apply", 0)
+    print("\nHBM bytes per launch (read + written, scaled), as bench.py reports them in `roofline.traffic`:\n")
+    print("traffic_bytes_per_launch: " + json.dumps(traffic, sort_keys=True))
+    print(f"taken_at_commit: {commit}")
+
+
+def summarize_trace(pairs, commit):
+    """Markdown summary of kernel-trace statistics, one table per phase of the benchmark."""
+    import csv
+
+    print("# rocprofv3 kernel trace: launch durations, Switch-MoE layer hot path (bench.py default workload)\n")
+    print("One run per phase, so that launches inside the layer step (inputs as the layer leaves them) and "
+          "back-to-back launches on one buffer set (inputs in the last-level cache) are separate rows:\n")
+    for pair in pairs:
+        label = pair.split("=", 1)[0]
+        print(f"    rocprofv3 --kernel-trace --stats --output-format csv -d <dir> -o s -- python3 bench.py --only {label} --no-cpu-baseline")
+    print("    python3 bench.py --summarize-trace " + " ".join(p.split("=", 1)[0] + "=<dir>/.../s_kernel_stats.csv" for p in pairs)
+          + " --commit <hash>\n")
+    for pair in pairs:
+        label, path = pair.split("=", 1)
+        print(f"## phase `{label}`\n")
+        print("| kernel | calls | average ns | min ns | max ns |")
+        print("|---|---|---|---|---|")
+        with open(path) as f:
+            for row in csv.DictReader(f):
+                name = row["Name"]
+                if "brt::" not in name and "Cijk" not in name:
+                    continue
+                short = re.sub(r"^void |brt::\(anonymous namespace\)::|\(brt::\w+\)$", "", name)
+                print(f"| `{short[:90]}` | {row['Calls']} | {float(row['AverageNs']):.0f} | {row['MinNs']} | {row['MaxNs']} |")
+        print()
+    print(f"taken_at_commit: {commit}")
 
 
 def measured_traffic():
@@ -857,6 +960,10 @@ def cpu_baseline(layer):
 
 def main():
     args = parse()
+    if args.summarize_pmc:
+        return summarize_pmc(args.summarize_pmc[0], args.summarize_pmc[1], args.commit)
+    if args.summarize_trace:
+        return summarize_trace(args.summarize_trace, args.commit)
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: the routing hot path is built and measured on a "
                  "single MI355X (no collectives in this build); run with --gpus 1")
