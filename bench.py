@@ -61,9 +61,10 @@ def parse():
     p.add_argument("--warmup", type=int, default=20)
     p.add_argument("--only", choices=PHASES, default="all")
     p.add_argument("--no-cpu-baseline", action="store_true")
-    p.add_argument("--summarize-pmc", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
-                   help="print the profiles/ summary of two rocprofv3 --pmc runs of this file "
-                        "(FETCH_SIZE, then WRITE_SIZE: their *_counter_collection.csv) and exit")
+    p.add_argument("--summarize-pmc", nargs="+", metavar="CSV",
+                   help="print the profiles/ summary of two rocprofv3 --pmc runs of `bench.py --only step` "
+                        "(FETCH_SIZE, then WRITE_SIZE: their *_counter_collection.csv), optionally followed "
+                        "by the same two of a run of all phases (listed, not used for the traffic line), and exit")
     p.add_argument("--summarize-trace", nargs="+", metavar="LABEL=STATS_CSV",
                    help="print the profiles/ summary of rocprofv3 --kernel-trace --stats runs of this "
                         "file (their *_kernel_stats.csv, one per phase) and exit")
@@ -89,10 +90,10 @@ def _kernel_key(name):
     return None
 
 
-def summarize_pmc(fetch_csv, write_csv, commit):
-    """Markdown summary of two counter runs: median FETCH_SIZE / WRITE_SIZE per kernel, scaled to
-    KiB by what the same counters read for the plain 12 MiB device copy the benchmark launches
-    (`y.copy_(x[:P])`), and the line bench.py reads back."""
+def summarize_pmc(csvs, commit):
+    """Markdown summary of counter runs: median FETCH_SIZE / WRITE_SIZE per kernel, scaled to KiB
+    by what the same counters read for a plain device-to-device copy of the 12 MiB of rows that
+    the benchmark makes (`x.clone()`), and the line bench.py reads back (from the run of the step)."""
     import csv
     import statistics
 
@@ -103,38 +104,50 @@ def summarize_pmc(fetch_csv, write_csv, commit):
                 per.setdefault(row["Kernel_Name"], []).append(float(row["Counter_Value"]))
         return {k: (statistics.median(v), len(v)) for k, v in per.items()}
 
-    fetch, write = medians(fetch_csv), medians(write_csv)
     copy_kib = T * D * 2 / 1024
-    copies = [k for k in fetch if "copyBuffer" in k or "copy_kernel" in k.lower() or "CopyFunctor" in k]
-    cal = {}
-    for label, table in (("fetch", fetch), ("write", write)):
-        vals = [table[k][0] for k in copies if k in table and 0.4 * copy_kib <= table[k][0] <= 1.1 * copy_kib]
-        cal[label] = copy_kib / statistics.median(vals) if vals else float("nan")
+
+    def table(fetch, write, keyed):
+        copies = [k for k in fetch if "copyBuffer" in k or "copy_kernel" in k.lower() or "CopyFunctor" in k]
+        cal = {}
+        for label, counts in (("fetch", fetch), ("write", write)):
+            vals = [counts[k][0] for k in copies
+                    if k in counts and 0.4 * copy_kib <= counts[k][0] <= 1.1 * copy_kib]
+            cal[label] = copy_kib / statistics.median(vals) if vals else float("nan")
+        print(f"Calibration: a device-to-device copy of the {copy_kib:.0f} KiB of rows reads FETCH_SIZE x "
+              f"{cal['fetch']:.3f} = {copy_kib:.0f} KiB and WRITE_SIZE x {cal['write']:.3f} = {copy_kib:.0f} KiB; "
+              "the counters below are scaled by these factors.\n")
+        print("| kernel | launches | FETCH_SIZE (raw median) | WRITE_SIZE (raw median) | read KiB | written KiB |")
+        print("|---|---|---|---|---|---|")
+        traffic = {}
+        for name in sorted(set(fetch) | set(write)):
+            key = _kernel_key(name)
+            if key is None and "brt::" not in name and "Cijk" not in name:
+                continue
+            f, n = fetch.get(name, (float("nan"), 0))
+            w, _ = write.get(name, (float("nan"), 0))
+            rk, wk = f * cal["fetch"], w * cal["write"]
+            short = re.sub(r"^void |brt::\(anonymous namespace\)::|\(brt::\w+\)$", "", name)
+            print(f"| `{short[:90]}` | {n} | {f:.1f} | {w:.1f} | {rk:.0f} | {wk:.0f} |")
+            if keyed and key is not None and n >= 10:
+                traffic[key] = traffic.get(key, 0) + int(round((rk + wk) * 1024))
+        if "indexgen_count" in traffic or "indexgen_apply" in traffic:
+            traffic["indexgen"] = traffic.pop("indexgen_count", 0) + traffic.pop("indexgen_apply", 0)
+        return traffic
+
     print("# rocprofv3 PMC: HBM traffic per launch, Switch-MoE layer hot path (bench.py default workload)\n")
     print("Commands (one counter per run; the summary is printed by `bench.py --summarize-pmc`):\n")
-    print("    rocprofv3 --pmc FETCH_SIZE --output-format csv -d <dir_f> -o s -- python3 bench.py --steps 20 --warmup 2 --no-cpu-baseline")
-    print("    rocprofv3 --pmc WRITE_SIZE --output-format csv -d <dir_w> -o s -- python3 bench.py --steps 20 --warmup 2 --no-cpu-baseline")
-    print("    python3 bench.py --summarize-pmc <dir_f>/.../s_counter_collection.csv <dir_w>/.../s_counter_collection.csv --commit <hash>\n")
-    print(f"Calibration: the device-to-device copy of the {copy_kib:.0f} KiB of rows reads FETCH_SIZE x "
-          f"{cal['fetch']:.3f} = {copy_kib:.0f} KiB and WRITE_SIZE x {cal['write']:.3f} = {copy_kib:.0f} KiB; "
-          "every counter below is scaled by these factors.\n")
-    print("| kernel | launches | FETCH_SIZE (raw median) | WRITE_SIZE (raw median) | read KiB | written KiB |")
-    print("|---|---|---|---|---|---|")
-    traffic = {}
-    for name in sorted(set(fetch) | set(write)):
-        key = _kernel_key(name)
-        if key is None and "brt::" not in name:
-            continue
-        f, n = fetch.get(name, (float("nan"), 0))
-        w, _ = write.get(name, (float("nan"), 0))
-        rk, wk = f * cal["fetch"], w * cal["write"]
-        short = re.sub(r"^void |brt::\(anonymous namespace\)::|\(brt::\w+\)$", "", name)
-        print(f"| `{short[:90]}` | {n} | {f:.1f} | {w:.1f} | {rk:.0f} | {wk:.0f} |")
-        if key is not None:
-            traffic[key] = traffic.get(key, 0) + int(round((rk + wk) * 1024))
-    if "indexgen_count" in traffic or "indexgen_apply" in traffic:
-        traffic["indexgen"] = traffic.pop("indexgen_count", 0) + traffic.pop("indexgen_apply", 0)
-    print("\nHBM bytes per launch (read + written, scaled), as bench.py reports them in `roofline.traffic`:\n")
+    print("    rocprofv3 --pmc FETCH_SIZE --output-format csv -d <f> -o s -- python3 bench.py --only step --steps 20 --warmup 2 --no-cpu-baseline")
+    print("    rocprofv3 --pmc WRITE_SIZE --output-format csv -d <w> -o s -- python3 bench.py --only step --steps 20 --warmup 2 --no-cpu-baseline")
+    if len(csvs) >= 4:
+        print("    rocprofv3 --pmc FETCH_SIZE --output-format csv -d <fa> -o s -- python3 bench.py --steps 20 --warmup 2 --no-cpu-baseline")
+        print("    rocprofv3 --pmc WRITE_SIZE --output-format csv -d <wa> -o s -- python3 bench.py --steps 20 --warmup 2 --no-cpu-baseline")
+    print("    python3 bench.py --summarize-pmc <f>/.../s_counter_collection.csv <w>/... [<fa>/... <wa>/...] --commit <hash>\n")
+    print("## the kernels of the step\n")
+    traffic = table(medians(csvs[0]), medians(csvs[1]), True)
+    if len(csvs) >= 4:
+        print("\n## every kernel of the benchmark (all phases: other configurations, compact route, gate, tag-index gather, library GEMM)\n")
+        table(medians(csvs[2]), medians(csvs[3]), False)
+    print("\nHBM bytes per launch (read + written, scaled) of the kernels of the step, as bench.py reports them in `roofline.traffic`:\n")
     print("traffic_bytes_per_launch: " + json.dumps(traffic, sort_keys=True))
     print(f"taken_at_commit: {commit}")
 
@@ -616,37 +629,26 @@ def phase_configs(gpu):
 
 
 def phase_instep(gpu, layer, steps):
-    """Kernel durations inside the step: the same step launched eagerly with an event after every
-    launch.  The two GEMMs keep the GPU busy long enough for the host to stay ahead, so the
-    intervals are kernel time, not launch time; what an event record itself costs is measured in
-    the same run (events recorded back to back) and taken off.  Inputs are what the layer sees:
-    the rows dispatch reads were last touched one step (700 MB of FFN traffic) earlier, the rows
-    combine reads were just written by the second GEMM."""
-    torch = gpu.torch
+    """What each kernel costs inside the step: the graph of K whole steps against the graph of K
+    steps with that one kernel left out, per step.  No event sits between the kernels and no
+    constant is taken off; the difference holds the kernel and the boundary to its successor, which
+    is also what a kernel trace of the step shows as the kernel's duration (dependent kernels
+    run one after the other, so a kernel's end is its successor's start).  Inputs are what the
+    layer sees: the rows dispatch reads were last touched one step (700 MB of FFN traffic) earlier,
+    the rows combine reads were just written by the second GEMM."""
     order = [("indexgen", layer.indexgen), ("dispatch", layer.dispatch), ("ffn_gemm1_gelu", layer.gemm1),
              ("ffn_gemm2", layer.gemm2), ("combine", layer.combine)]
-    n_eager = max(50, min(steps, 200))
-    marks = [[torch.cuda.Event(enable_timing=True) for _ in range(len(order) + 1)] for _ in range(n_eager)]
-    with torch.cuda.stream(gpu.stream):
-        for _ in range(3):
-            layer.step(0)
-        for ev in marks:
-            ev[0].record(gpu.stream)
-            for j, (_, fn) in enumerate(order):
-                fn(0)
-                ev[j + 1].record(gpu.stream)
-        blank = [torch.cuda.Event(enable_timing=True) for _ in range(64)]
-        layer.gemm2(0)                                   # something to queue behind
-        for ev in blank:
-            ev.record(gpu.stream)
-    gpu.stream.synchronize()
-    gaps = sorted(blank[i].elapsed_time(blank[i + 1]) * 1e3 for i in range(8, 63))
-    event_us = gaps[len(gaps) // 2]                      # what an event record itself costs
-    in_step_us = {}
-    for j, (name, _) in enumerate(order):
-        spans = sorted(ev[j].elapsed_time(ev[j + 1]) * 1e3 for ev in marks)
-        in_step_us[name] = max(spans[len(spans) // 2] - event_us, 0.0)
-    return in_step_us, event_us
+    rounds = max(50, min(steps, 200))
+
+    def per_step_us(skip):
+        fns = [(lambda fn=fn: fn(0)) for name, fn in order if name != skip]
+        graph = gpu.capture(fns, rounds)
+        gpu.timed(graph, 1)
+        return min(gpu.timed(graph, 1) for _ in range(5)) * 1e3 / rounds
+
+    whole = per_step_us(None)
+    in_step_us = {name: max(whole - per_step_us(name), 0.0) for name, _ in order}
+    return in_step_us, whole
 
 
 # ------------------------------------------------------------------ extras (reported, not `value`)
@@ -961,7 +963,7 @@ def cpu_baseline(layer):
 def main():
     args = parse()
     if args.summarize_pmc:
-        return summarize_pmc(args.summarize_pmc[0], args.summarize_pmc[1], args.commit)
+        return summarize_pmc(args.summarize_pmc, args.commit)
     if args.summarize_trace:
         return summarize_trace(args.summarize_trace, args.commit)
     if args.gpus != 1:
@@ -1022,18 +1024,19 @@ def main():
         result["layer_through_router_api"] = phase_api(gpu, layer, args.steps)
 
     if want("instep"):
-        us, event_us = phase_instep(gpu, layer, args.steps)
+        us, whole_us = phase_instep(gpu, layer, args.steps)
         dc_bytes = nbytes["dispatch"] + nbytes["combine"]
         value = dc_bytes / (us["dispatch"] + us["combine"]) / 1e3
         result["value"] = round(value, 1)
         result["hbm_peak_frac"] = round(value / HBM_PEAK_GBPS, 4)
         result["value_is"] = (
             f"(bytes dispatch and the tag-driven combine have to move = {dc_bytes}) / (sum of their "
-            "durations inside the step: medians of event-to-event intervals of the eagerly launched "
-            "step minus the cost of an event record).  Inputs are as the layer leaves them: not the "
+            "costs inside the step: the graph of K steps against the graph of K steps without that "
+            "kernel, per step; the kernel trace of the same step shows the same durations).  Inputs are as the layer leaves them: not the "
             "cache-resident buffers of back-to-back launches (dispatch_combine_warm_GBps), not the "
             "never-touched ones of the ring (dispatch_combine_cold_ring_GBps)")
-        result["in_step"] = {"event_record_us": round(event_us, 2), "kernels": per_kernel(us)}
+        result["in_step"] = {"step_us": round(whole_us, 2), "sum_of_kernel_costs_us": round(sum(us.values()), 2),
+                             "kernels": per_kernel(us)}
         dominant = "combine" if us["combine"] >= us["dispatch"] else "dispatch"
         result["roofline"] = {
             "kernel": dominant, "bound": "hbm",
