@@ -102,16 +102,16 @@ def summarize_pmc(csvs, commit):
         with open(path) as f:
             for row in csv.DictReader(f):
                 per.setdefault(row["Kernel_Name"], []).append(float(row["Counter_Value"]))
-        return {k: (statistics.median(v), len(v)) for k, v in per.items()}
+        return {k: (statistics.median(v), len(v), v) for k, v in per.items()}
 
     copy_kib = T * D * 2 / 1024
 
     def table(fetch, write, keyed):
-        copies = [k for k in fetch if "copyBuffer" in k or "copy_kernel" in k.lower() or "CopyFunctor" in k]
         cal = {}
         for label, counts in (("fetch", fetch), ("write", write)):
-            vals = [counts[k][0] for k in copies
-                    if k in counts and 0.4 * copy_kib <= counts[k][0] <= 1.1 * copy_kib]
+            # the copies of the 12 MiB of rows among all device-to-device copies of the run
+            vals = [v for k in counts if "copyBuffer" in k for v in counts[k][2]
+                    if 0.4 * copy_kib <= v <= 1.1 * copy_kib]
             cal[label] = copy_kib / statistics.median(vals) if vals else float("nan")
         print(f"Calibration: a device-to-device copy of the {copy_kib:.0f} KiB of rows reads FETCH_SIZE x "
               f"{cal['fetch']:.3f} = {copy_kib:.0f} KiB and WRITE_SIZE x {cal['write']:.3f} = {copy_kib:.0f} KiB; "
@@ -123,8 +123,8 @@ def summarize_pmc(csvs, commit):
             key = _kernel_key(name)
             if key is None and "brt::" not in name and "Cijk" not in name:
                 continue
-            f, n = fetch.get(name, (float("nan"), 0))
-            w, _ = write.get(name, (float("nan"), 0))
+            f, n = fetch.get(name, (float("nan"), 0, None))[:2]
+            w = write.get(name, (float("nan"), 0, None))[0]
             rk, wk = f * cal["fetch"], w * cal["write"]
             short = re.sub(r"^void |brt::\(anonymous namespace\)::|\(brt::\w+\)$", "", name)
             print(f"| `{short[:90]}` | {n} | {f:.1f} | {w:.1f} | {rk:.0f} | {wk:.0f} |")
