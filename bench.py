@@ -68,6 +68,12 @@ def parse():
     p.add_argument("--summarize-trace", nargs="+", metavar="LABEL=STATS_CSV",
                    help="print the profiles/ summary of rocprofv3 --kernel-trace --stats runs of this "
                         "file (their *_kernel_stats.csv, one per phase) and exit")
+    p.add_argument("--config", default=None,
+                   help="with --only configs: run only the configurations whose name contains this")
+    p.add_argument("--summarize-counters", nargs="+", metavar="LABEL=COUNTER_CSV",
+                   help="print a profiles/ summary of rocprofv3 --pmc runs of `bench.py --only configs "
+                        "--config <label>` (their *_counter_collection.csv): averages per kernel, and exit")
+    p.add_argument("--counters", default="", help="the counter list of those runs (for the summary)")
     p.add_argument("--commit", default="unknown", help="commit the profiled tree was at (for the summaries)")
     return p.parse_args()
 
@@ -149,6 +155,47 @@ def summarize_pmc(csvs, commit):
         table(medians(csvs[2]), medians(csvs[3]), False)
     print("\nHBM bytes per launch (read + written, scaled) of the kernels of the step, as bench.py reports them in `roofline.traffic`:\n")
     print("traffic_bytes_per_launch: " + json.dumps(traffic, sort_keys=True))
+    print(f"taken_at_commit: {commit}")
+
+
+def summarize_counters(pairs, counters, commit):
+    """Average of every counter per grouped-GEMM kernel, one table per configuration."""
+    import csv
+
+    print("# rocprofv3 PMC: matrix-pipe and LDS counters of the grouped expert GEMM on the ragged and compute-bound shapes\n")
+    print("One run per configuration (the same kernel instantiation serves several of them):\n")
+    for pair in pairs:
+        label = pair.split("=", 1)[0]
+        print(f"    rocprofv3 --pmc {counters} --output-format csv -d <dir> -o s -- python3 bench.py --only configs --config {label} --no-cpu-baseline")
+    print("    python3 bench.py --summarize-counters " + " ".join(p.split("=", 1)[0] + "=<dir>/.../s_counter_collection.csv" for p in pairs)
+          + " --counters '<list>' --commit <hash>\n")
+    print("Averages per launch; SQ counters are summed over the chip, GRBM_GUI_ACTIVE over the 8 XCDs. "
+          "`mfma busy` = SQ_VALU_MFMA_BUSY_CYCLES / (1024 SIMDs x GRBM_GUI_ACTIVE / 8): the share of the "
+          "kernel's duration in which a SIMD's matrix pipe is busy (the counter advances by 32 per "
+          "`v_mfma_f32_32x32x16_bf16`); `flop` = SQ_INSTS_VALU_MFMA_MOPS_BF16 x 512 (every row tile of a "
+          "row block is multiplied, filled or not).\n")
+    for pair in pairs:
+        label, path = pair.split("=", 1)
+        per = {}
+        with open(path) as f:
+            for row in csv.DictReader(f):
+                name = row["Kernel_Name"]
+                if "grouped_gemm_kernel" not in name:
+                    continue
+                per.setdefault(name, {}).setdefault(row["Counter_Name"], []).append(float(row["Counter_Value"]))
+        names = sorted({c for v in per.values() for c in v})
+        print(f"## `{label}`\n")
+        print("| kernel | launches | " + " | ".join(names) + " | mfma busy | flop |")
+        print("|---|---|" + "---|" * (len(names) + 2))
+        for name, vals in sorted(per.items()):
+            avg = {c: sum(v) / len(v) for c, v in vals.items()}
+            n = max(len(v) for v in vals.values())
+            busy = avg.get("SQ_VALU_MFMA_BUSY_CYCLES", float("nan")) / (1024 * avg.get("GRBM_GUI_ACTIVE", float("nan")) / 8)
+            flop = avg.get("SQ_INSTS_VALU_MFMA_MOPS_BF16", float("nan")) * 512
+            short = re.sub(r"^void |brt::\(anonymous namespace\)::|\(brt::\w+\)$", "", name)
+            print(f"| `{short}` | {n} | " + " | ".join(f"{avg.get(c, float('nan')):.0f}" for c in names)
+                  + f" | {busy:.3f} | {flop:.3e} |")
+        print()
     print(f"taken_at_commit: {commit}")
 
 
@@ -608,23 +655,29 @@ def ffn_config(gpu, loads_np, d, dff, seed, spot_checks=3):
     return res
 
 
-def phase_configs(gpu):
+def phase_configs(gpu, only=None):
+    """`only`: a substring that selects the configurations to run (for counter runs of one of them)."""
     import numpy as np
     import workloads
 
     out = {"note": "the other BASELINE configurations at full size, same process, same timing "
                    "method (graphs of launches over a ring of buffer sets larger than the "
                    "last-level cache); bytes by the per-kernel formulas of the routing kernels"}
+    want = lambda name: only is None or only in name  # noqa: E731
     for name, c in workloads.ROUTING_CONFIGS.items():
-        out[name] = routing_config(gpu, name, c)
-    loads3 = workloads.top2_skewed_route()[3]
-    out["cfg3_ffn_32e_1024_4096"] = ffn_config(gpu, loads3.astype(np.int64), 1024, 4096, seed=3)
-    loads5 = workloads.dirichlet_loads(32768, 128, 0.3, seed=5)
-    out["cfg5_task_moe_ffn_128e_2048_8192"] = ffn_config(gpu, loads5.astype(np.int64), 2048, 8192, seed=5)
+        if want(name):
+            out[name] = routing_config(gpu, name, c)
+    if want("cfg3_ffn_32e_1024_4096"):
+        loads3 = workloads.top2_skewed_route()[3]
+        out["cfg3_ffn_32e_1024_4096"] = ffn_config(gpu, loads3.astype(np.int64), 1024, 4096, seed=3)
+    if want("cfg5_task_moe_ffn_128e_2048_8192"):
+        loads5 = workloads.dirichlet_loads(32768, 128, 0.3, seed=5)
+        out["cfg5_task_moe_ffn_128e_2048_8192"] = ffn_config(gpu, loads5.astype(np.int64), 2048, 8192, seed=5)
     # what the same kernel does when the shape lets the matrix units be the bound: the same rows
     # and feature sizes over 8 experts of 4096 rows (weights 268 MB per GEMM)
-    out["compute_bound_probe_8e_x_4096_rows_2048_8192"] = ffn_config(
-        gpu, np.full(8, 4096, dtype=np.int64), 2048, 8192, seed=6, spot_checks=1)
+    if want("compute_bound_probe_8e_x_4096_rows_2048_8192"):
+        out["compute_bound_probe_8e_x_4096_rows_2048_8192"] = ffn_config(
+            gpu, np.full(8, 4096, dtype=np.int64), 2048, 8192, seed=6, spot_checks=1)
     return out
 
 
@@ -966,6 +1019,8 @@ def main():
         return summarize_pmc(args.summarize_pmc, args.commit)
     if args.summarize_trace:
         return summarize_trace(args.summarize_trace, args.commit)
+    if args.summarize_counters:
+        return summarize_counters(args.summarize_counters, args.counters, args.commit)
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: the routing hot path is built and measured on a "
                  "single MI355X (no collectives in this build); run with --gpus 1")
@@ -1087,7 +1142,7 @@ def main():
         }
 
     if want("configs"):
-        result["configs"] = phase_configs(gpu)
+        result["configs"] = phase_configs(gpu, args.config)
 
     if want("extras"):
         result.update(phase_extras(gpu, layer, args.steps))
