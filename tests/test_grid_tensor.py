@@ -128,3 +128,22 @@ def test_protocol_masks_on_cpu():
     m = make_protocol("binary_threshold", {"threshold": 0.9, "selected_path": 1})(
         torch.tensor([[10.0, 0.0], [0.1, 0.0]]))
     assert m.tolist() == [[0, 1], [1, 0]]  # confident rows take the selected path
+
+
+def test_module_paths_of_the_reference_resolve():
+    """Code written against the reference imports its classes from the modules it keeps them in
+    (python/brt/router/fabric/fused.py, protocol/topk.py, ...)."""
+    import importlib
+
+    for path, attr in (("brt.router.fabric.fused", "FusedDispatchFabric"),
+                       ("brt.router.fabric.generic", "DispatchFabric"),
+                       ("brt.router.fabric.base", "make_fabric"),
+                       ("brt.router.fabric.distributed", "DistributedFusedCombineFabric"),
+                       ("brt.router.protocol.topk", "TopKProtocol"),
+                       ("brt.router.protocol.swin_moe", "SwinMoEProtocol"),
+                       ("brt.router.protocol.base", "make_protocol"),
+                       ("brainstorm_amd.router.protocol.hashed", "HashProtocol")):
+        module = importlib.import_module(path)
+        assert hasattr(module, attr), path
+    from brt.router.fabric.fused import FusedCombineFabric  # noqa: F401
+    from brt.router.protocol.switch import SwitchTop1Protocol  # noqa: F401
