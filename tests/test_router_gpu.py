@@ -735,3 +735,87 @@ def test_task_hash_and_label_protocols_route_on_the_gpu(brt_mod):
     assert np.array_equal(brt.to_torch_tensor(routed).cpu().numpy(), o_y)
     out = gather(routed * 2.0, torch.zeros_like(x))
     assert np.array_equal(brt.to_torch_tensor(out).cpu().numpy(), x.cpu().numpy() * 2)
+
+
+@pytest.mark.parametrize("fabric_kwargs", [{"defer_dispatch": True}, {"static_rows": True}])
+def test_deferred_and_static_rows_layers_replay_from_a_hip_graph(brt_mod, fabric_kwargs):
+    """Neither form reads the loads back, so the layer (router objects and jit kernels, written as
+    the reference's Switch layer) can be captured without max_path_padding and replayed for new
+    inputs; every replay is checked against the eager layer, with eager work in between."""
+    brt, _, ScatterRouter, GatherRouter = brt_mod
+    from brt.jit import make_jit_kernel
+
+    T, E, d, dff, cap = 3000, 8, 128, 256, 500
+    gen = torch.Generator(device="cuda").manual_seed(77)
+    x = torch.randn(T, d, device="cuda", generator=gen).to(torch.bfloat16)
+    score = torch.randn(T, E, device="cuda", generator=gen)
+    torch.manual_seed(78)
+    wi = nn.ModuleList(nn.Linear(d, dff, bias=False) for _ in range(E)).cuda().to(torch.bfloat16)
+    wo = nn.ModuleList(nn.Linear(dff, d, bias=False) for _ in range(E)).cuda().to(torch.bfloat16)
+    fused_wi = make_jit_kernel(wi, None, opt_level="homo_fuse", activation="relu")
+    fused_wo = make_jit_kernel(wo, None, opt_level="homo_fuse")
+    annotate = brt.Annotator([0])
+
+    def make_layer(kwargs):
+        scatter = ScatterRouter(protocol_type="topk", fabric_type="fused_dispatch",
+                                fabric_kwargs={"supported_capacities": [cap], **kwargs}).cuda()
+        gather = GatherRouter(fabric_type="fused_combine").cuda()
+
+        def layer(cells, scores, residual):
+            routed = scatter(annotate(cells), scores)
+            states, tags, loads, extra = brt.to_torch_tensor(routed, retrieve_attr=True)
+            h = torch.empty((states.shape[0], dff), device="cuda", dtype=torch.bfloat16)
+            fused_wi(shared_inputs=[states, h], standalone_inputs=[m.weight for m in wi], capacities=loads[-1])
+            y = torch.empty((states.shape[0], d), device="cuda", dtype=torch.bfloat16)
+            fused_wo(shared_inputs=[h, y], standalone_inputs=[m.weight for m in wo], capacities=loads[-1])
+            return brt.to_torch_tensor(gather(brt.to_grid_tensor(y, tags, loads, extra), residual))
+        return layer
+
+    layer, eager = make_layer(fabric_kwargs), make_layer({})
+    residual = torch.empty_like(x)
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        residual.copy_(x)
+        layer(x, score, residual)  # allocations and lazy initialisation happen outside the capture
+        torch.cuda.synchronize()
+        with torch.cuda.graph(graph, stream=stream):
+            residual.copy_(x)
+            layer(x, score, residual)
+    torch.cuda.synchronize()
+    for _ in range(4):
+        x.copy_(torch.randn(T, d, device="cuda", generator=gen).to(torch.bfloat16))
+        score.copy_(torch.randn(T, E, device="cuda", generator=gen))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        want = eager(x, score, x.clone())
+        assert torch.equal(residual, want)
+        assert not torch.equal(residual, x)
+
+
+def test_decoder_greedy_search_protocol_on_the_gpu(brt_mod):
+    """protocol/decoder.py:31-75: path 0 takes the sequences whose last token is not the end token,
+    path 1 the finished ones, with the loads of the hot mask; with skip_eos_check the first
+    iterations (no sequence can have ended yet) route everything to path 0 without looking."""
+    from brt.router.protocol import make_protocol
+
+    eos = 2
+    tokens = torch.tensor([[5], [2], [7], [2], [2], [9]], device="cuda")
+    proto = make_protocol("decoder_greedy_search", {"index_format": "seat_index", "pad_token_id": 0,
+                                                    "eos_token_id": eos}).cuda()
+    hot_mask, loads, loads_again = proto(tokens)
+    want = torch.tensor([[1, 0], [0, 1], [1, 0], [0, 1], [0, 1], [1, 0]], device="cuda")
+    assert torch.equal(hot_mask, want) and loads.tolist() == [3, 3] and loads_again is loads
+    skipping = make_protocol("decoder_greedy_search", {"index_format": "seat_index", "pad_token_id": 0,
+                                                       "eos_token_id": eos, "skip_eos_check": True}).cuda()
+    skipping.update(torch.tensor([4, 6, 4], device="cuda"))
+    route, loads, _ = skipping(tokens)             # iteration 1 of sequences of at least 4 tokens
+    assert route[:, 0].tolist() == list(range(6)) and int(route[:, 1].abs().sum()) == 0
+    assert loads.tolist() == [6, 0]
+    skipping(tokens)                               # iteration 2
+    hot_mask3, loads3, _ = skipping(tokens)        # iteration 3: a sequence of 4 may end now
+    assert torch.equal(hot_mask3, want) and loads3.tolist() == [3, 3]
+    with pytest.raises(NotImplementedError):
+        make_protocol("decoder_beam_search", {"index_format": "seat_index", "pad_token_id": 0,
+                                              "eos_token_id": eos}).cuda()(tokens)
