@@ -489,7 +489,8 @@ __global__ __launch_bounds__(WAVES * 64) void grouped_gemm_kernel(GemmArgs a) {
 #pragma unroll
             for (int w = 0; w < 4; ++w) v[w] = plus_zero<BRT_BF16>(v[w]);
           }
-          stream_out(v, reinterpret_cast<u32x4*>(oc + static_cast<size_t>(to) * a.N + c * 8));
+          if (a.plain_out) *reinterpret_cast<u32x4*>(oc + static_cast<size_t>(to) * a.N + c * 8) = v;  // kept in the caches
+          else stream_out(v, reinterpret_cast<u32x4*>(oc + static_cast<size_t>(to) * a.N + c * 8));
         }
       }
     }
@@ -648,6 +649,13 @@ int grouped_gemm_impl(const void* x, const void* const* weights, const void* con
   a.tag_div = entries_per_cell;
   a.E = E; a.P = P; a.K = K; a.N = N; a.T = T;
   a.gather = gather_in != 0; a.scatter = scatter_out != 0;
+  // Output stores.  A large output (the expanding GEMM of an FFN) is written with the streaming
+  // policy: it would only push the operands out of the caches.  A small one that the next kernel
+  // reads at once (the contracting GEMM: its rows go straight into the combine) is written with
+  // ordinary stores and stays in the last-level cache: the benchmark layer's combine then costs
+  // 4.9 us instead of 5.9 us and the GEMM itself nothing (measured inside the step; with ordinary
+  // stores in the expanding GEMM that GEMM takes 102 us instead of 87 us).
+  a.plain_out = N < K && static_cast<size_t>(P) * N * 2 <= (size_t{32} << 20);
   if (out_is_f32) {
     if (act == BRT_ACT_GELU) return launch_f32<BRT_ACT_GELU>(a, as_stream(stream));
     if (act == BRT_ACT_RELU) return launch_f32<BRT_ACT_RELU>(a, as_stream(stream));

@@ -18,6 +18,7 @@ struct GemmArgs {
   int tag_vector;   // tags is the row-entry vector
   int tag_div;      // entries per cell (k) of the row-entry vector
   int E, P, K, N, T;
+  int plain_out;  // ordinary output stores instead of streaming ones (a small output that is read at once)
   int gather, scatter;  // rows of x / of out are addressed through the tags
   int tiles_n, tiles_m_max;
   int walk, groups_n;  // column tiles one workgroup walks, ceil(tiles_n / walk)
