@@ -147,3 +147,48 @@ def test_module_paths_of_the_reference_resolve():
         assert hasattr(module, attr), path
     from brt.router.fabric.fused import FusedCombineFabric  # noqa: F401
     from brt.router.protocol.switch import SwitchTop1Protocol  # noqa: F401
+
+
+def test_deferred_buffer_fills_itself_before_any_read_and_not_for_metadata():
+    """Host logic of the deferred dispatch (no GPU: the dispatch itself is replaced by a counter).
+    Shape, dtype, device, data_ptr leave the buffer alone; an operator on the plain tensor or on the
+    GridTensor that wraps it fills it first; afterwards nothing is deferred any more."""
+    import brt
+    from brainstorm_amd.runtime import deferred
+
+    class State(deferred.DeferredState):
+        __slots__ = ("fills",)
+
+        def materialize(self):
+            if not self.done:
+                self.fills += 1
+                self.buffer.fill_(7.0)
+                self.done = True
+
+    def make():
+        cells = torch.zeros(4, 3)
+        state = State(cells, route=None, buffer=torch.empty(6, 3), key="brt_deferred_0")
+        state.fills = 0
+        grid = brt.to_grid_tensor(state.buffer, [torch.zeros(1)], [torch.zeros(1)], {"brt_deferred_0": state})
+        return state, grid
+
+    state, grid = make()
+    assert tuple(grid.shape) == (6, 3) and grid.dtype == torch.float32 and grid.data_ptr() == state.buffer.data_ptr()
+    plain, tags, loads, extra = brt.to_torch_tensor(grid, retrieve_attr=True)
+    assert isinstance(plain, deferred.DeferredRows) and deferred.state_of(plain) is state
+    assert plain.shape[0] == 6 and plain.device.type == "cpu" and plain.is_contiguous() and state.fills == 0
+    total = plain.sum()                      # a read: the dispatch runs first
+    assert state.fills == 1 and float(total) == 7.0 * 18 and deferred.state_of(plain) is None
+    assert type(plain + 1) is torch.Tensor   # results are ordinary tensors
+    again = brt.to_torch_tensor(grid)        # nothing pending any more: a plain tensor
+    assert type(again) is torch.Tensor and state.fills == 1
+
+    state, grid = make()
+    doubled = grid * 2                       # an operator on the GridTensor fills it too
+    assert state.fills == 1 and float(brt.to_torch_tensor(doubled).sum()) == 14.0 * 18
+    assert isinstance(doubled, brt.GridTensor) and doubled.extra_attr_dict["brt_deferred_0"] is state
+
+    state, grid = make()
+    other = torch.ones(6, 3)
+    assert deferred.pending_state(grid.extra_attr_dict, other) is None  # another tensor is not the buffer
+    assert deferred.wrap_if_pending(other, grid.extra_attr_dict) is other and state.fills == 0
