@@ -159,23 +159,38 @@ def summarize_pmc(csvs, commit):
 
 
 def summarize_counters(pairs, counters, commit):
-    """Average of every counter per grouped-GEMM kernel, one table per configuration."""
+    """Average of every counter per grouped-GEMM kernel, one table per profiled run.
+
+    A label that names a phase of the benchmark stands for `--only <label>`, any other for
+    `--only configs --config <label>`; `counters` is one list for all runs, or one per run
+    separated by `;` (a label may repeat: one run per pass over the counters).
+    """
     import csv
 
-    print("# rocprofv3 PMC: matrix-pipe and LDS counters of the grouped expert GEMM on the ragged and compute-bound shapes\n")
-    print("One run per configuration (the same kernel instantiation serves several of them):\n")
-    for pair in pairs:
+    lists = [c.strip() for c in counters.split(";")]
+    if len(lists) != len(pairs):
+        lists = [counters.strip()] * len(pairs)
+
+    def run_args(label):
+        return f"--only {label}" if label in PHASES else f"--only configs --config {label}"
+
+    print("# rocprofv3 PMC: counters of the grouped expert GEMM\n")
+    print("One run per table (the same kernel instantiation serves several configurations):\n")
+    for pair, clist in zip(pairs, lists):
         label = pair.split("=", 1)[0]
-        print(f"    rocprofv3 --pmc {counters} --output-format csv -d <dir> -o s -- python3 bench.py --only configs --config {label} --no-cpu-baseline")
+        print(f"    rocprofv3 --pmc {clist} --output-format csv -d <dir> -o s -- python3 bench.py {run_args(label)} --no-cpu-baseline")
     print("    python3 bench.py --summarize-counters " + " ".join(p.split("=", 1)[0] + "=<dir>/.../s_counter_collection.csv" for p in pairs)
-          + " --counters '<list>' --commit <hash>\n")
-    print("Averages per launch; SQ counters are summed over the chip, GRBM_GUI_ACTIVE over the 8 XCDs. "
+          + " --counters '<list>[;<list>...]' --commit <hash>\n")
+    print("Averages per launch; SQ, TCP and TCC counters are summed over the chip (SQ wave-cycle counters "
+          "advance once per 4 clocks), GRBM_GUI_ACTIVE over the 8 XCDs. "
           "`mfma busy` = SQ_VALU_MFMA_BUSY_CYCLES / (1024 SIMDs x GRBM_GUI_ACTIVE / 8): the share of the "
           "kernel's duration in which a SIMD's matrix pipe is busy (the counter advances by 32 per "
           "`v_mfma_f32_32x32x16_bf16`); `flop` = SQ_INSTS_VALU_MFMA_MOPS_BF16 x 512 (every row tile of a "
           "row block is multiplied, filled or not).\n")
+    seen = {}
     for pair in pairs:
         label, path = pair.split("=", 1)
+        seen[label] = seen.get(label, 0) + 1
         per = {}
         with open(path) as f:
             for row in csv.DictReader(f):
@@ -184,17 +199,23 @@ def summarize_counters(pairs, counters, commit):
                     continue
                 per.setdefault(name, {}).setdefault(row["Counter_Name"], []).append(float(row["Counter_Value"]))
         names = sorted({c for v in per.values() for c in v})
-        print(f"## `{label}`\n")
-        print("| kernel | launches | " + " | ".join(names) + " | mfma busy | flop |")
-        print("|---|---|" + "---|" * (len(names) + 2))
+        repeated = sum(1 for q in pairs if q.split("=", 1)[0] == label) > 1
+        print(f"## `{label}`" + (f", pass {seen[label]}" if repeated else "") + "\n")
+        with_busy = "SQ_VALU_MFMA_BUSY_CYCLES" in names and "GRBM_GUI_ACTIVE" in names
+        with_flop = "SQ_INSTS_VALU_MFMA_MOPS_BF16" in names
+        extra = (["mfma busy"] if with_busy else []) + (["flop"] if with_flop else [])
+        print("| kernel | launches | " + " | ".join(names + extra) + " |")
+        print("|---|---|" + "---|" * (len(names) + len(extra)))
         for name, vals in sorted(per.items()):
             avg = {c: sum(v) / len(v) for c, v in vals.items()}
             n = max(len(v) for v in vals.values())
-            busy = avg.get("SQ_VALU_MFMA_BUSY_CYCLES", float("nan")) / (1024 * avg.get("GRBM_GUI_ACTIVE", float("nan")) / 8)
-            flop = avg.get("SQ_INSTS_VALU_MFMA_MOPS_BF16", float("nan")) * 512
+            cells = [f"{avg.get(c, float('nan')):.0f}" for c in names]
+            if with_busy:
+                cells.append(f"{avg['SQ_VALU_MFMA_BUSY_CYCLES'] / (1024 * avg['GRBM_GUI_ACTIVE'] / 8):.3f}")
+            if with_flop:
+                cells.append(f"{avg['SQ_INSTS_VALU_MFMA_MOPS_BF16'] * 512:.3e}")
             short = re.sub(r"^void |brt::\(anonymous namespace\)::|\(brt::\w+\)$", "", name)
-            print(f"| `{short}` | {n} | " + " | ".join(f"{avg.get(c, float('nan')):.0f}" for c in names)
-                  + f" | {busy:.3f} | {flop:.3e} |")
+            print(f"| `{short}` | {n} | " + " | ".join(cells) + " |")
         print()
     print(f"taken_at_commit: {commit}")
 
