@@ -771,6 +771,50 @@ def phase_extras(gpu, layer, steps):
     extras["layer_fused_step"] = ("indexgen(tag indices)+GEMM1 gathering cells+GEMM2 scattering to "
                                   "cells; K steps in one HIP graph")
 
+    # ---- index generation and dispatch in one dependent step (two launches instead of three)
+    ws_rd = torch.empty(max(16, L.brt_hip_route_and_dispatch_workspace_bytes(T, E, D * 2)),
+                        dtype=torch.uint8, device=dev)
+    idx_rd = torch.empty_like(mask)
+    loads_counts_rd = torch.empty(2, E, dtype=torch.int32, device=dev)
+    y_rd = torch.empty(P, D, dtype=torch.bfloat16, device=dev)
+    tags_rd = torch.empty(P, dtype=torch.int32, device=dev)
+    y2_rd = torch.empty(P, D, dtype=torch.bfloat16, device=dev)
+    out_rd = x.clone()
+
+    def k_route_dispatch():
+        gpu.check(L.brt_hip_route_and_dispatch(
+            mask.data_ptr(), x.data_ptr(), y_rd.data_ptr(), idx_rd.data_ptr(),
+            loads_counts_rd[0].data_ptr(), loads_counts_rd[1].data_ptr(), tags_rd.data_ptr(), T, E, P,
+            D * 2, layer.caps.data_ptr(), 1, 0, 0, ws_rd.data_ptr(), ws_rd.numel(), gpu.sptr()))
+
+    def step_route_dispatch():
+        k_route_dispatch()
+        gpu.check(L.brt_hip_grouped_gemm(
+            y_rd.data_ptr(), layer.wi_tab.data_ptr(), None, layer.h.data_ptr(),
+            loads_counts_rd[0].data_ptr(), E, P, D, DFF, lib.ACT_GELU, gpu.sptr()))
+        gpu.check(L.brt_hip_grouped_gemm(
+            layer.h.data_ptr(), layer.wo_tab.data_ptr(), None, y2_rd.data_ptr(),
+            loads_counts_rd[0].data_ptr(), E, P, DFF, D, lib.ACT_NONE, gpu.sptr()))
+        gpu.check(L.brt_hip_combine_by_tags(
+            y2_rd.data_ptr(), out_rd.data_ptr(), tags_rd.data_ptr(), P, D, T, lib.BF16, lib.BF16,
+            gpu.sptr()))
+
+    gpu.run(lambda: layer.step(0), step_route_dispatch)
+    same = (torch.equal(b0["out"].view(torch.int16), out_rd.view(torch.int16))
+            and torch.equal(b0["idx"], idx_rd) and torch.equal(b0["y"].view(torch.int16), y_rd.view(torch.int16))
+            and torch.equal(b0["row_tags"], tags_rd) and torch.equal(layer.loads, loads_counts_rd[0]))
+    if not same:
+        sys.exit("bench.py: index generation fused with dispatch disagrees with the two calls")
+    g_rd = gpu.capture(step_route_dispatch, steps)
+    g_plain = gpu.capture(lambda: layer.step(0), steps)
+    gpu.timed(g_rd, 1), gpu.timed(g_plain, 1)
+    extras["layer_route_dispatch_us"] = round(gpu.timed(g_rd, 1) / steps * 1e3, 2)
+    extras["layer_route_dispatch_step"] = ("index generation fused with dispatch (2 launches)+ffn+"
+                                           "tag-driven combine; K steps in one HIP graph; beside it "
+                                           "the five-launch step timed the same way in the same "
+                                           "process")
+    extras["layer_route_dispatch_unfused_us"] = round(gpu.timed(g_plain, 1) / steps * 1e3, 2)
+
     # ---- gate front-end: scores -> hot mask
     gate_mask = torch.empty_like(mask)
     probs_d = layer.probs.to(dev)
@@ -913,6 +957,8 @@ def phase_extras(gpu, layer, steps):
         "compact_gate_softmax_top1": k_gate_compact, "compact_gate_switch_torch_ops": k_gate_switch_torch,
         "compact_route_by_path": k_route_compact, "compact_dispatch_by_rows": k_dispatch_rows,
         "compact_combine_by_rows": k_combine_rows, "indexgen_tags": k_indexgen_tags,
+        "route_and_dispatch": k_route_dispatch,
+        "indexgen_then_dispatch": lambda: (layer.indexgen(0), layer.dispatch(0)),
         "ffn_gemm1_gelu_gather": k_gemm1_gather, "ffn_gemm2_scatter": k_gemm2_scatter,
         "tag_gather_unique": k_tag_unique, "tag_gather_sum": k_tag_sum,
         "tag_gather_sum_torch_ops": k_tag_sum_torch,
@@ -925,6 +971,8 @@ def phase_extras(gpu, layer, steps):
     kbytes = {
         "gate_topk_mask": 2 * idx_bytes, "indexgen_tags": 2 * idx_bytes + 8 * E,
         "plain_copy_of_the_rows": 2 * min(P, T) * D * es,
+        "route_and_dispatch": 2 * idx_bytes + 8 * E + R * D * es + P * D * es + 4 * P,
+        "indexgen_then_dispatch": 3 * idx_bytes + 8 * E + R * D * es + P * D * es + 4 * P,
         "compact_gate_softmax_top1": idx_bytes + 8 * T,
         "compact_route_by_path": 2 * 4 * T + 4 * T + 4 * P + 8 * E,
         "compact_dispatch_by_rows": R * D * es + P * D * es + 4 * P,

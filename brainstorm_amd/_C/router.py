@@ -25,6 +25,7 @@ __all__ = [
     "generate_indices_and_loads",
     "convert_index_format",
     "dispatch_with_indices_and_loads",
+    "route_and_dispatch",
     "dispatch_rows_of_route",
     "combine_by_row_tags",
     "split_fused_cells_to_paths",
@@ -382,8 +383,8 @@ def dispatch_with_indices_and_loads(
             new_tags = alloc((total,), dtype=route_indices.dtype, device=device)
         hidden_tags = (pairing is not None and pairing.single_path and is_1d_routing
                        and not tag_generating)
-        if hidden_tags and new_tags is None:
-            new_tags = torch.empty((total,), dtype=torch.int32, device=device)
+        if hidden_tags and new_tags is None:  # rows past the loads have no writer: their tags start at zero
+            new_tags = alloc((total,), dtype=torch.int32, device=device)
 
         _lib.check(_lib.lib().brt_hip_dispatch(
             _ptr(in_data), _ptr(out), _ptr(dev_gates), _ptr(route_indices), _ptr(dev_loads),
@@ -394,6 +395,70 @@ def dispatch_with_indices_and_loads(
     if tag_generating:
         return [out, new_tags]
     return [out]
+
+
+def route_and_dispatch(
+    in_data: torch.Tensor,
+    hot_mask: torch.Tensor,
+    rows: int,
+    supported_capacities: Optional[torch.Tensor] = None,
+    capacity_padding: bool = False,
+    path_wise_padding: bool = False,
+    single_path: bool = False,
+) -> Tuple[Route, torch.Tensor]:
+    """Not in the reference: :func:`generate_route` (seat indices) and an unweighted 1-d
+    :func:`dispatch_with_indices_and_loads` with ``rows=`` in one dependent step -- the second pass
+    of the index scan moves the rows of its own cells (two launches instead of three, the index
+    matrix is not read back).  Returns the route and the ``[rows, ...]`` path-major tensor, every
+    row of it written (zeros where no cell owns the row); bit-identical to the two calls, which it
+    makes itself for the shapes the fused kernel does not take."""
+    _check_on_device(in_data, "in_data")
+    _check_on_device(hot_mask, "hot_mask")
+    _check_int32(hot_mask, "hot_mask")
+    T, E = hot_mask.size(0), hot_mask.size(1)
+    if in_data.size(0) != T:
+        raise RuntimeError("in_data and hot_mask must have one row per cell")
+    rows = int(rows)
+    n_caps = 0 if supported_capacities is None else supported_capacities.size(0)
+    cell_bytes = (in_data.numel() // T) * in_data.element_size() if T > 0 else 0
+    lib = _lib.lib()
+    fused = (T > 0 and in_data.dtype in _DT and lib.brt_hip_route_and_dispatch_supported(
+        T, E, cell_bytes, n_caps, int(bool(path_wise_padding and capacity_padding))) == 1)
+    if not fused:
+        route = generate_route(hot_mask, supported_capacities, capacity_padding, path_wise_padding,
+                               False, single_path)
+        out = dispatch_with_indices_and_loads(in_data, route.indices, route.loads, route=route,
+                                              rows=rows)[0]
+        return route, out
+    with _device_guard(in_data.device):
+        caps = None
+        if supported_capacities is not None:
+            _check_on_device(supported_capacities, "supported_capacities")
+            _check_int32(supported_capacities, "supported_capacities")
+            caps = supported_capacities.contiguous()
+        if capacity_padding and n_caps < 1:
+            raise RuntimeError("capacity_padding requires at least one supported capacity")
+        hot_mask = hot_mask.contiguous()
+        in_data = in_data.contiguous()
+        indices = torch.empty_like(hot_mask)
+        loads_and_counts = torch.empty((2, E), dtype=torch.int32, device=hot_mask.device)
+        loads, counts = loads_and_counts[0], loads_and_counts[1]
+        out = torch.empty([rows] + list(in_data.shape[1:]), dtype=in_data.dtype, device=in_data.device)
+        row_tags = torch.empty((rows,), dtype=torch.int32, device=in_data.device) if single_path else None
+        need = lib.brt_hip_route_and_dispatch_workspace_bytes(T, E, cell_bytes)
+        key = (in_data.device.index, _stream())
+        ws = _workspaces.get(key)
+        if ws is None or ws.numel() < need:
+            ws = torch.empty(max(need, 1 << 16), dtype=torch.uint8, device=in_data.device)
+            _workspaces[key] = ws
+        _lib.check(lib.brt_hip_route_and_dispatch(
+            _ptr(hot_mask), _ptr(in_data), _ptr(out), _ptr(indices), _ptr(loads), _ptr(counts),
+            _ptr(row_tags), T, E, rows, cell_bytes, _ptr(caps), n_caps, int(capacity_padding),
+            int(path_wise_padding), _ptr(ws), ws.numel(), _stream()))
+        route = Route(indices, loads, counts, False, single_path)
+        if single_path:
+            route.row_tags, route.row_tags_stride = row_tags, 0
+    return route, out
 
 
 def dispatch_rows_of_route(cells: torch.Tensor, route: Route, out: torch.Tensor) -> None:

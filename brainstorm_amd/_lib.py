@@ -51,6 +51,13 @@ SIGNATURES = {
         [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int,
          _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     ),
+    "brt_hip_route_and_dispatch_supported": (_c_int, [_c_int, _c_int, _c_size, _c_int, _c_int]),
+    "brt_hip_route_and_dispatch_workspace_bytes": (_c_size, [_c_int, _c_int, _c_size]),
+    "brt_hip_route_and_dispatch": (
+        _c_int,
+        [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_size,
+         _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_size, _c_ptr],
+    ),
     "brt_hip_combine": (
         _c_int,
         [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,

@@ -35,8 +35,10 @@
 #include <algorithm>
 #include <cstdlib>
 #include <mutex>
+#include <type_traits>
 
 #include "common.hpp"
+#include "rows.hpp"
 
 // Scratch of brt_hip_generate_indices_and_loads_static: the per-band column sums that the first
 // kernel of index generation hands to the second, for callers that cannot bring a workspace of
@@ -349,6 +351,276 @@ __global__ __launch_bounds__(kWavesPB * kWave) void band_apply_kernel(ScanArgs a
   }
 }
 
+// ---- index generation pass 2 and dispatch in one kernel ---------------------------------------
+// What band_apply_kernel<kSeat> writes, and in the same kernel what the dispatch of those indices
+// writes (1-d routing, unweighted, un-strided layout): the rows of the wavefront's own cells go to
+// start[path] + seat - 1 of the path-major buffer.  A wavefront's cells are one contiguous run of
+// 16-byte units; every lane requests its share of them before anything else, so the rows travel
+// while the mask words and the sums of the other bands are fetched and walked, and are stored as
+// soon as the seats are known.  Every band needs the totals of all paths (for the path starts),
+// so it adds up the bands below it as well as those above.  The rows no cell owns (padding rows
+// of a path, rows past the last path) are zero-filled by the same launch, dealt evenly to all
+// wavefronts.  E <= 64; a wavefront's cells fit kFusedUnits 16-byte units per lane (the host
+// picks the rows per wavefront for that).
+constexpr int kFusedUnits = 32;  // 16-byte units of row data a lane holds (128 registers)
+constexpr int kFusedCaps = 8;    // supported capacities held in registers
+constexpr int kFusedPartials = 64;  // band sums a lane adds up (one batch of loads)
+
+struct FusedArgs {
+  ScanArgs s;
+  const u32x4* src;  // [T, cpr]
+  u32x4* dst;        // [P, cpr]
+  int* row_tags;     // [P] or null
+  int P, cpr;
+};
+
+template <bool STREAM, int NV>
+__global__ __launch_bounds__(kBlock) void band_apply_dispatch_kernel(FusedArgs f) {
+  const ScanArgs& a = f.s;
+  __shared__ int s_above[kWavesPB][kWave];
+  __shared__ int s_own[kWavesPB][kWave];
+  __shared__ int s_below[kWavesPB][kWave];
+  __shared__ int s_n[kWavesPB][kBatch * kWave];     // per wavefront: paths that take each of its rows
+  __shared__ int s_list[kWavesPB][kBatch * kWave];  // per wavefront: their destination rows, row-major
+  const int tid = threadIdx.x, lane = tid & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int E = a.E, band = blockIdx.x;
+  const int ep = 1 << a.ep_shift, rps = kWave >> a.ep_shift;
+  const int e = lane & (ep - 1), sub = lane >> a.ep_shift;
+  const long row_w = (static_cast<long>(band) * kWavesPB + wave) * a.rows_pw;
+  const int n_ins = a.n_ins;
+  const int rows_here = static_cast<int>(max(0l, min(static_cast<long>(a.rows_pw), a.T - row_w)));
+  const int cpr = f.cpr;
+  const bool col_ok = e < E;
+
+  // Every load of the kernel's first memory round trip is a buffer load: a wave-uniform base and
+  // extent per array, a 32-bit offset per lane, and a word outside the extent (a row past the
+  // wavefront's rows, a band past the last, a lane past E) reads as zero -- no 64-bit address
+  // arithmetic, no branch and no select stands between the loads, so all of them are in flight
+  // before the first is used.
+  constexpr unsigned kOutside = 0x80000000u;
+  auto resource = [](const void* base, size_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0,
+                                             static_cast<int>(std::min<size_t>(bytes, 0x7fffffff)), 0x00020000);
+  };
+  // Issue order = order of use (the memory counter retires loads in order): band sums, own mask
+  // words, capacities, and last the wavefront's rows, which are stored at the very end.
+  // ---- sums of the other bands (the host keeps the bands within kFusedPartials loads per lane) ----
+  int part[kFusedPartials];
+  const int j_first = wave + sub * kWavesPB, j_step = kWavesPB * rps;
+  {
+    const __amdgpu_buffer_rsrc_t res_partial = resource(a.partial, static_cast<size_t>(a.bands) * E * 4);
+    const unsigned partial_off = col_ok ? (j_first * E + e) * 4 : kOutside;
+#pragma unroll
+    for (int u = 0; u < kFusedPartials; ++u)
+      part[u] = __builtin_amdgcn_raw_buffer_load_b32(res_partial, partial_off + u * j_step * E * 4, 0, 0);
+  }
+  // ---- own mask words -----------------------------------------------------------------------
+  int m0[kBatch];
+  {
+    const __amdgpu_buffer_rsrc_t res_mask =
+        resource(a.mask + (rows_here > 0 ? row_w : 0) * E, static_cast<size_t>(rows_here) * E * 4);
+    const unsigned mask_off = col_ok ? (sub * E + e) * 4 : kOutside;
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u)
+      m0[u] = __builtin_amdgcn_raw_buffer_load_b32(res_mask, mask_off + u * rps * E * 4, 0, 0);
+  }
+  // ---- capacity menu: lane i fetches entry i, lane e the path's own capacity (path-wise padding) ----
+  const __amdgpu_buffer_rsrc_t res_caps = resource(a.caps, static_cast<size_t>(a.C) * 4);
+  const int cap_lane = __builtin_amdgcn_raw_buffer_load_b32(res_caps, lane * 4, 0, 0);
+  const int cap_own = __builtin_amdgcn_raw_buffer_load_b32(res_caps, col_ok ? e * 4 : kOutside, 0, 0);
+  // ---- the wavefront's rows ------------------------------------------------------------------
+  const int n_units = rows_here * cpr;
+  const __amdgpu_buffer_rsrc_t res_rows =
+      resource(f.src + (rows_here > 0 ? row_w : 0) * cpr, static_cast<size_t>(n_units) * 16);
+  u32x4 val[NV];
+#pragma unroll
+  for (int i = 0; i < NV; ++i)
+    val[i] = __builtin_amdgcn_raw_buffer_load_b128(res_rows, (i * kWave + lane) * 16, 0, 0);
+  __builtin_amdgcn_sched_barrier(0);  // nothing below is scheduled in between the loads
+
+  int above = 0, below = 0;
+#pragma unroll
+  for (int u = 0; u < kFusedPartials; ++u) {
+    const int j = j_first + u * j_step;
+    above += j < band ? part[u] : 0;
+    below += j > band ? part[u] : 0;
+  }
+  int capv[kFusedCaps];
+#pragma unroll
+  for (int i = 0; i < kFusedCaps; ++i) capv[i] = read_lane(cap_lane, i);
+  int own = 0;
+#pragma unroll
+  for (int u = 0; u < kBatch; ++u) own += m0[u];
+  above = sum_over_rows_in_wave(above, a.ep_shift);
+  below = sum_over_rows_in_wave(below, a.ep_shift);
+  own = sum_over_rows_in_wave(own, a.ep_shift);
+  if (sub == 0) {
+    s_above[wave][e] = above;
+    s_own[wave][e] = own;
+    s_below[wave][e] = below;
+  }
+  __syncthreads();
+  int carry = 0, total = 0;
+#pragma unroll
+  for (int k = 0; k < kWavesPB; ++k) {
+    carry += s_above[k][e];
+    total += s_above[k][e] + s_own[k][e] + s_below[k][e];
+    if (k < wave) carry += s_own[k][e];
+  }
+
+  // ---- loads and path starts from the totals (every lane: those of its own path) ------------
+  int load_e = 0;
+  if (col_ok) {
+    if (a.path_wise_padding) load_e = cap_own;
+    else if (total == 0 || a.C == 0) load_e = total;
+    else {
+      load_e = capv[0];  // overwritten below; the last capacity when none holds the count
+      bool done = false;
+#pragma unroll
+      for (int i = 0; i < kFusedCaps; ++i) {
+        if (i < a.C) {
+          if (!done && total <= capv[i]) {
+            load_e = a.capacity_padding ? capv[i] : total;
+            done = true;
+          }
+          if (!done) load_e = capv[i];
+        }
+      }
+    }
+  }
+  const int incl_l = wave_inclusive_scan(sub == 0 ? load_e : 0);
+  const int start_e = __shfl(incl_l - (sub == 0 ? load_e : 0), e, kWave);
+  const int sum_loads = read_lane(incl_l, kWave - 1);
+
+  // ---- walk the rows: seats out, destination rows into the wavefront's table ----------------
+  {
+    int incl[kBatch], tot[kBatch];
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) {
+      incl[u] = m0[u];
+      tot[u] = m0[u];
+      if (rps > 1 && u < n_ins) {
+        int x = m0[u];
+        for (int d = ep; d < kWave; d <<= 1) {
+          const int t = __shfl_up(x, d, kWave);
+          if (lane >= d) x += t;
+        }
+        incl[u] = x;
+        tot[u] = __shfl(x, (rps - 1) * ep + e, kWave);
+      }
+    }
+    int* __restrict__ out_w = a.out + row_w * E;
+    const unsigned long long seg0 = ep == kWave ? ~0ull : ((1ull << ep) - 1ull);
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) {
+      if (u < n_ins) {  // wave-uniform
+        const int run = carry + incl[u];
+        carry += tot[u];
+        const int rl = u * rps + sub;
+        const bool mine = col_ok && rl < rows_here;
+        const int v = run * m0[u];
+        if (mine) out_w[static_cast<unsigned>(rl) * E + e] = v;  // location * mask, location.cu:177-178
+        const int dst_row = start_e + v - 1;
+        const bool hit = mine && v >= 1 && v <= load_e && dst_row < f.P;
+        const unsigned long long seg = (__ballot(hit) >> (sub * ep)) & seg0;
+        if (hit) {
+          s_list[wave][rl * ep + __popcll(seg & ((1ull << e) - 1ull))] = dst_row;
+          if (f.row_tags != nullptr) f.row_tags[dst_row] = static_cast<int>(row_w) + rl + 1;
+        }
+        if (e == 0) s_n[wave][rl] = __popcll(seg);
+      }
+    }
+  }
+  __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+
+  // ---- the rows leave: unit i*64 + lane of the wavefront's run belongs to row (i*64+lane)/cpr ----
+  // The table is read for all units at once (one LDS latency instead of two per unit), the first
+  // destination of every unit is stored, and only a wavefront that holds a cell on several paths
+  // walks the further destinations.
+  {
+    const int q64 = kWave / cpr, r64 = kWave - q64 * cpr;
+    const int row0 = lane / cpr, off0 = lane - row0 * cpr;
+    auto advance = [&](int& row, int& off) {
+      row += q64;
+      off += r64;
+      if (off >= cpr) off -= cpr, ++row;
+    };
+    int n_of[NV], d_of[NV];
+    {
+      int row = row0, off = off0;
+#pragma unroll
+      for (int i = 0; i < NV; ++i) {
+        const int at = i * kWave + lane < n_units ? row : 0;
+        n_of[i] = s_n[wave][at];
+        d_of[i] = s_list[wave][at * ep];
+        advance(row, off);
+      }
+    }
+    int most = 0;
+    {
+      int row = row0, off = off0;
+#pragma unroll
+      for (int i = 0; i < NV; ++i) {
+        if (i * kWave + lane >= n_units) n_of[i] = 0;
+        if (n_of[i] > 0) store_unit<STREAM>(f.dst + static_cast<size_t>(d_of[i]) * cpr + off, val[i]);
+        most = max(most, n_of[i]);
+        advance(row, off);
+      }
+    }
+    if (__ballot(most > 1) != 0) {
+      int row = row0, off = off0;
+#pragma unroll
+      for (int i = 0; i < NV; ++i) {
+        for (int j = 1; j < n_of[i]; ++j) {
+          const int d = s_list[wave][row * ep + j];
+          store_unit<STREAM>(f.dst + static_cast<size_t>(d) * cpr + off, val[i]);
+        }
+        advance(row, off);
+      }
+    }
+  }
+
+  // ---- rows no cell owns: padding rows of the paths, then the rows past the last path ----------
+  {
+    const long n_waves = static_cast<long>(gridDim.x) * kWavesPB;
+    const long me = static_cast<long>(band) * kWavesPB + wave;
+    const bool path_lane = sub == 0 && col_ok;
+    const int z = path_lane ? load_e - max(0, min(total, load_e)) : 0;
+    const int z_incl = wave_inclusive_scan(z);
+    const long Z = read_lane(z_incl, kWave - 1);
+    const long tail = max(0l, static_cast<long>(f.P) - sum_loads);
+    if (Z + tail > 0) {
+      const unsigned nw = static_cast<unsigned>(n_waves), w = static_cast<unsigned>(me);
+      const unsigned all = static_cast<unsigned>(Z + tail);
+      const unsigned q = all / nw, r = all % nw;
+      const long z0 = static_cast<long>(q) * w + min(w, r), z1 = z0 + q + (w < r ? 1 : 0);
+      for (long zi = z0; zi < z1; ++zi) {
+        long row;
+        if (zi < Z) {
+          const int pe = __builtin_ctzll(__ballot(z_incl > zi));
+          const int pad = read_lane(z, pe);
+          row = static_cast<long>(read_lane(start_e, pe)) + (read_lane(load_e, pe) - pad) +
+                (zi - (read_lane(z_incl, pe) - pad));
+        } else {
+          row = sum_loads + (zi - Z);
+        }
+        if (row < f.P) {
+          for (int o = lane; o < cpr; o += kWave) f.dst[static_cast<size_t>(row) * cpr + o] = zero_unit<16>();
+          if (f.row_tags != nullptr && lane == 0) f.row_tags[row] = 0;
+        }
+      }
+    }
+  }
+
+  // ---- totals (last band only) -----------------------------------------------------------
+  if (band == a.bands - 1 && wave == 0 && sub == 0 && col_ok) {
+    a.loads[e] = load_e;
+    if (a.counts) a.counts[e] = total;
+  }
+}
+
 __global__ void fill_int_kernel(int* p, int n, int v) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) p[i] = v;
@@ -424,6 +696,29 @@ int launch_scan(int mode, ScanArgs& a, void* workspace, size_t workspace_bytes, 
   else
     hipLaunchKernelGGL((band_apply_kernel<kThrottle, kWavesPB>), grid, dim3(kBlock), 0, st, a);
   return check_launch("band_apply_kernel");
+}
+
+// Geometry of the fused kernel: rows per wavefront so that a wavefront's cells fit the units a
+// lane holds and, where the batch allows, every CU gets a band.
+bool fused_geometry(int T, int E, int cpr, ScanGeometry* g) {
+  if (T <= 0 || E <= 0 || E > kWave || cpr <= 0) return false;
+  int shift = 0;
+  while ((1 << shift) < E) ++shift;
+  const int rps = kWave >> shift;
+  const long fit = static_cast<long>(kFusedUnits) * kWave / cpr / rps * rps;  // rows a wavefront can hold
+  if (fit < rps) return false;
+  const long most = std::min<long>(static_cast<long>(kBatch) * rps, fit);
+  constexpr long want_bands = 256;  // one per CU: half as many make the kernel a third longer at 8192 x 64
+  long rows_pw = (static_cast<long>(T) + want_bands * kWavesPB - 1) / (want_bands * kWavesPB);
+  rows_pw = std::min(most, std::max<long>((rows_pw + rps - 1) / rps * rps, rps));
+  const long per_band = rows_pw * kWavesPB;
+  const long bands = (static_cast<long>(T) + per_band - 1) / per_band;
+  if (bands > kMaxBands || bands > static_cast<long>(kFusedPartials) * kWavesPB * rps) return false;
+  g->ep_shift = shift;
+  g->rows_pw = static_cast<int>(rows_pw);
+  g->bands = static_cast<int>(bands);
+  g->waves_pb = kWavesPB;
+  return true;
 }
 
 constexpr int kMaxDevices = 64;
@@ -523,6 +818,91 @@ extern "C" int brt_hip_generate_indices_and_loads_static(const int32_t* mask, in
   return brt_hip_generate_indices_and_loads(mask, indices, loads, counts, T, E, caps, C,
                                             capacity_padding, path_wise_padding, is_tag_index, ptr,
                                             kStaticScratchInts * sizeof(int), stream);
+}
+
+extern "C" int brt_hip_route_and_dispatch_supported(int T, int E, size_t cell_bytes, int C,
+                                                    int path_wise_padding) {
+  ScanGeometry g;
+  if (cell_bytes == 0 || cell_bytes % 16 != 0 || cell_bytes / 16 > 0x7fffffffull) return 0;
+  if (!path_wise_padding && C > kFusedCaps) return 0;
+  return fused_geometry(T, E, static_cast<int>(cell_bytes / 16), &g) ? 1 : 0;
+}
+
+extern "C" size_t brt_hip_route_and_dispatch_workspace_bytes(int T, int E, size_t cell_bytes) {
+  ScanGeometry g;
+  if (cell_bytes == 0 || cell_bytes % 16 != 0 || cell_bytes / 16 > 0x7fffffffull) return 0;
+  if (!fused_geometry(T, E, static_cast<int>(cell_bytes / 16), &g)) return 0;
+  return (static_cast<size_t>(g.bands) + 1) * E * sizeof(int);
+}
+
+extern "C" int brt_hip_route_and_dispatch(const int32_t* mask, const void* cells, void* rows,
+                                          int32_t* indices, int32_t* loads, int32_t* counts,
+                                          int32_t* row_tags, int T, int E, int P, size_t cell_bytes,
+                                          const int32_t* caps, int C, int capacity_padding,
+                                          int path_wise_padding, void* workspace,
+                                          size_t workspace_bytes, void* stream) {
+  if (T < 0 || E <= 0 || P < 0) return fail(BRT_E_INVALID, "bad shape T=%d E=%d P=%d", T, E, P);
+  if (!mask || !cells || !indices || !loads || (!rows && P > 0)) return fail(BRT_E_INVALID, "null argument");
+  if (caps == nullptr) C = 0;
+  if (capacity_padding && C < 1)
+    return fail(BRT_E_INVALID, "capacity_padding needs at least one supported capacity");
+  if (!capacity_padding) path_wise_padding = 0;
+  if (path_wise_padding && C < E)
+    return fail(BRT_E_INVALID, "path_wise_padding needs one capacity per path (%d < %d)", C, E);
+  if (!aligned(cells, 16) || !aligned(rows, 16))
+    return fail(BRT_E_INVALID, "cells/rows must be 16-byte aligned");
+  ScanGeometry g;
+  if (!brt_hip_route_and_dispatch_supported(T, E, cell_bytes, C, path_wise_padding) ||
+      !fused_geometry(T, E, static_cast<int>(cell_bytes / 16), &g))
+    return fail(BRT_E_UNSUPPORTED,
+                "route_and_dispatch takes 1..64 paths, cells of a multiple of 16 bytes, at most %d "
+                "supported capacities and a batch its bands can hold (T=%d E=%d cell=%zu bytes C=%d): "
+                "use brt_hip_generate_indices_and_loads + brt_hip_dispatch",
+                kFusedCaps, T, E, cell_bytes, C);
+  const size_t need = (static_cast<size_t>(g.bands) + 1) * E * sizeof(int);
+  if (workspace == nullptr || workspace_bytes < need)
+    return fail(BRT_E_WORKSPACE, "workspace too small: %zu < %zu bytes", workspace_bytes, need);
+  if (!aligned(workspace, 4)) return fail(BRT_E_INVALID, "workspace must be 4-byte aligned");
+  FusedArgs f{};
+  ScanArgs& a = f.s;
+  a.mask = mask;
+  a.out = indices;
+  a.loads = loads;
+  a.counts = counts;
+  a.caps = caps;
+  a.C = C;
+  a.T = T;
+  a.E = E;
+  a.capacity_padding = capacity_padding;
+  a.path_wise_padding = path_wise_padding;
+  a.partial = static_cast<int*>(workspace);
+  a.prefix_in = a.partial + static_cast<size_t>(g.bands) * E;
+  a.ep_shift = g.ep_shift;
+  a.rows_pw = g.rows_pw;
+  a.n_ins = g.rows_pw >> (6 - g.ep_shift);
+  a.bands = g.bands;
+  f.src = static_cast<const u32x4*>(cells);
+  f.dst = static_cast<u32x4*>(rows);
+  f.row_tags = row_tags;
+  f.P = P;
+  f.cpr = static_cast<int>(cell_bytes / 16);
+  hipStream_t st = as_stream(stream);
+  const dim3 grid(g.bands);
+  if (g.bands > 1) hipLaunchKernelGGL(band_count_kernel, grid, dim3(kBlock), 0, st, a);
+  // rows of more than 128 bytes leave as streaming stores, shorter ones merge in the L2 (as in dispatch)
+  const int units = (g.rows_pw * f.cpr + kWave - 1) / kWave;  // per lane
+  auto go = [&](auto stream_t, auto nv_t) {
+    hipLaunchKernelGGL((band_apply_dispatch_kernel<decltype(stream_t)::value, decltype(nv_t)::value>), grid,
+                       dim3(kBlock), 0, st, f);
+  };
+  auto by_units = [&](auto stream_t) {
+    if (units <= 8) go(stream_t, std::integral_constant<int, 8>{});
+    else if (units <= 16) go(stream_t, std::integral_constant<int, 16>{});
+    else go(stream_t, std::integral_constant<int, kFusedUnits>{});
+  };
+  if (f.cpr > 8) by_units(std::true_type{});
+  else by_units(std::false_type{});
+  return check_launch("band_apply_dispatch_kernel");
 }
 
 extern "C" int brt_hip_throttle_hotmask(const int32_t* mask, int32_t* out, int32_t* prefix,

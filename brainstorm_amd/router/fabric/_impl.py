@@ -400,6 +400,35 @@ class FusedDispatchFabric(DispatchFabric):
             return paths * max(self._host_caps)
         return min(cells, paths * max(self._host_caps))
 
+    def forward(self, in_flow, hot_mask, runtime_capacities=None, score=None):
+        in_flows = [in_flow] if self.flow_num == 1 else in_flow
+        if not self._in_one_step(in_flows, runtime_capacities, hot_mask):
+            return super().forward(in_flow, hot_mask, runtime_capacities, score)
+        # static rows, one flow, single-path route: index generation moves the rows itself
+        data, tags, load_stack, extra = to_torch_tensor(in_flows[0], retrieve_attr=True)
+        assert tags[-1] is None  # fused dispatch starts from freshly annotated cells
+        self._route, routed = c_router.route_and_dispatch(
+            data, hot_mask, self._row_bound(data.shape[0], hot_mask.shape[1]),
+            supported_capacities=self.supported_capacities, capacity_padding=self.capacity_padding,
+            path_wise_padding=self.path_wise_padding, single_path=True)
+        route_indices, loads = self._route.indices, self._route.loads
+        self.capture_flow_stats(in_flows, route_indices, loads)
+        extra = dict(extra or {})
+        extra[_route_key(len(tags) - 1)] = self._route
+        out = init_grid_tensor(routed, tags[:-1] + [route_indices], load_stack[:-1] + [loads], extra)
+        return (out if self.flow_num == 1 else [out]), score
+
+    def _in_one_step(self, in_flows, runtime_capacities, hot_mask) -> bool:
+        if not (self.static_rows and getattr(hot_mask, "_brt_single_path", False)):
+            return False
+        if self.defer_dispatch and self._defers(in_flows, runtime_capacities, hot_mask):
+            return False
+        if len(in_flows) != 1 or runtime_capacities is not None or self.max_path_padding:
+            return False
+        flow = in_flows[0]
+        return (not self.transforms[0] and self.route_logics[0] == "1d" and flow.dim() >= 2
+                and flow.shape[0] > 0 and flow.is_cuda and hot_mask.dtype == torch.int32)
+
     def dispatch(self, in_flows, route_indices, loads, score):
         all_out_flows = []
         deferred = self._route.is_tag_index

@@ -154,6 +154,40 @@ int brt_hip_dispatch(const void* src, void* dst, const void* gates, const int32_
                      int is_1d_routing, int is_tag_index, int dtype, void* stream);
 
 /*
+ * Index generation and dispatch in one dependent step: what
+ * brt_hip_generate_indices_and_loads (seat indices) followed by brt_hip_dispatch (1-d routing,
+ * unweighted, counts given, max_path_load = 0) write, from two launches instead of three -- the
+ * second pass of the scan moves the rows of its own cells as soon as it knows their seats.  Fuses
+ * src/router/location.cu:212-257 with src/router/route.cu:13-103 (the reference runs them as
+ * separate kernels, router.cc:100-140,180-250); results are bit-identical to the two calls.
+ *
+ *   mask      [T,E] int32 hot mask              cells    [T, cell_bytes] rows of any dtype
+ *   rows      [P, cell_bytes] out: EVERY row is written -- routed rows, zeros for the padding
+ *             rows of a path and for the rows past the last path (P may exceed sum(loads):
+ *             a caller that cannot read the loads back allocates an upper bound)
+ *   indices   [T,E] out, loads [E] out, counts [E] out or NULL: as brt_hip_generate_indices_and_loads
+ *   row_tags  [P] out or NULL: 1-based cell of every row, 0 for rows no cell owns (the new_tags
+ *             of brt_hip_dispatch; what brt_hip_combine_by_tags reads)
+ *   caps, C, capacity_padding, path_wise_padding: the capacity rules of location.cu:222-256
+ *   workspace at least brt_hip_route_and_dispatch_workspace_bytes(T, E, cell_bytes) bytes
+ *
+ * Shapes it takes: 1 <= E <= 64, T >= 1, cell_bytes a multiple of 16, at most 8 supported
+ * capacities unless padding path-wise, and a batch whose bands can hold its cells
+ * (brt_hip_route_and_dispatch_supported() returns 1; e.g. up to 16384 cells of 1536 bytes over 64 paths, or
+ * 262144 cells of 192 bytes over 8 paths).  Anything else is refused with BRT_E_UNSUPPORTED and nothing is launched:
+ * make the two calls.
+ */
+int brt_hip_route_and_dispatch_supported(int T, int E, size_t cell_bytes, int C,
+                                         int path_wise_padding);
+size_t brt_hip_route_and_dispatch_workspace_bytes(int T, int E, size_t cell_bytes);
+int brt_hip_route_and_dispatch(const int32_t* mask, const void* cells, void* rows,
+                               int32_t* indices, int32_t* loads, int32_t* counts,
+                               int32_t* row_tags, int T, int E, int P, size_t cell_bytes,
+                               const int32_t* caps, int C, int capacity_padding,
+                               int path_wise_padding, void* workspace, size_t workspace_bytes,
+                               void* stream);
+
+/*
  * Replaces router::CombineWithIndicesAndLoads<dtype>, seat-index mode
  * (route.h:30-44, route.cu:208-282,467-518).
  *

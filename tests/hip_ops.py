@@ -134,6 +134,37 @@ def dispatch(x_bits, idx, loads, gates_bits=None, counts=None, tag_generating=Fa
     return host(d_out, True), (None if d_new is None else host(d_new))
 
 
+def route_and_dispatch_supported(T, E, cell_bytes, n_caps=0, path_wise_padding=False):
+    return _lib.lib().brt_hip_route_and_dispatch_supported(T, E, cell_bytes, n_caps, int(path_wise_padding)) == 1
+
+
+def route_and_dispatch(mask, x_bits, P, caps=None, capacity_padding=False, path_wise_padding=False,
+                       want_tags=True, dtype="f32"):
+    """Every output starts poisoned: the entry point has to write all of indices, loads, counts, rows
+    and row tags itself."""
+    mask = np.ascontiguousarray(mask, dtype=np.int32)
+    T, E = mask.shape
+    x_bits = np.ascontiguousarray(x_bits).reshape(T, -1)
+    cell_bytes = x_bits.shape[1] * x_bits.dtype.itemsize
+    d_mask, d_x = dev(mask), dev(x_bits)
+    d_idx = torch.full((T, E), -7, dtype=torch.int32, device="cuda")
+    d_loads = torch.full((E,), -1, dtype=torch.int32, device="cuda")
+    d_counts = torch.full((E,), -1, dtype=torch.int32, device="cuda")
+    d_rows = torch.full((P, x_bits.shape[1]), 0x55, dtype=_TORCH_BITS[dtype], device="cuda") if dtype != "f32" \
+        else torch.full((P, x_bits.shape[1]), float("nan"), device="cuda")
+    d_tags = torch.full((P,), -9, dtype=torch.int32, device="cuda") if want_tags else None
+    d_caps = None if caps is None else dev(np.asarray(caps, dtype=np.int32))
+    need = _lib.lib().brt_hip_route_and_dispatch_workspace_bytes(T, E, cell_bytes)
+    ws = torch.full((max(need, 16),), 0xA5, dtype=torch.uint8, device="cuda")
+    _lib.check(_lib.lib().brt_hip_route_and_dispatch(
+        ptr(d_mask), ptr(d_x), ptr(d_rows), ptr(d_idx), ptr(d_loads), ptr(d_counts), ptr(d_tags),
+        T, E, P, cell_bytes, ptr(d_caps), 0 if caps is None else len(caps), int(capacity_padding),
+        int(path_wise_padding), ptr(ws), ws.numel(), stream()))
+    torch.cuda.synchronize()
+    return (host(d_idx), host(d_loads), host(d_counts), host(d_rows, True),
+            None if d_tags is None else host(d_tags))
+
+
 def combine(y_bits, idx, loads, gates_bits=None, residual_bits=None, max_path_load=0,
             in_dtype="f32", out_dtype=None, gate_dtype=None):
     out_dtype = out_dtype or in_dtype

@@ -171,6 +171,54 @@ def test_dispatch_bit_exact(hip, T, E, k, cell, dtype):
             assert same_bits(got, want) and np.array_equal(got_tags, want_tags)
 
 
+ROUTE_DISPATCH_SHAPES = [  # T, E, k, cell elements, dtype
+    (8192, 64, 1, 768, "bf16"), (1024, 16, 1, 512, "f32"), (16384, 32, 2, 1024, "bf16"),
+    (100352, 8, 1, 96, "f16"), (777, 5, 3, 24, "f32"), (100, 3, 2, 8, "bf16"), (1, 1, 1, 8, "bf16"),
+    (3000, 64, 4, 40, "f16"), (5000, 33, 1, 264, "bf16"), (4096, 64, 2, 4096, "bf16"),
+    (2048, 2, 0, 4, "f32"), (4100, 64, 1, 1024, "f32"), (20000, 1, 1, 8, "f16"),
+]
+
+
+@pytest.mark.parametrize("T,E,k,cell,dtype", ROUTE_DISPATCH_SHAPES)
+def test_route_and_dispatch_bit_exact(hip, T, E, k, cell, dtype):
+    """Index generation fused with dispatch against the oracle's two steps: indices, loads, counts,
+    every row of a buffer longer (and shorter) than the loads add up to, and the row tags."""
+    mask, _ = topk_mask(T, E, k, seed=T + 3 * cell) if k > 0 else (np.zeros((T, E), np.int32), None)
+    mask[::7] = 0  # cells that no path takes
+    rng = np.random.default_rng(T + E)
+    x = as_dtype_bits(rng.standard_normal((T, cell)), dtype)
+    cell_bytes = cell * x.dtype.itemsize
+    cap = max(1, int(1.1 * T * max(k, 1) / E))
+    menus = [(None, False, False), ([cap], False, False), ([max(1, cap // 2), cap, 4 * cap], True, False),
+             ([cap + e for e in range(E)], True, True)]
+    for caps, pad, path_wise in menus:
+        assert hip.route_and_dispatch_supported(T, E, cell_bytes, 0 if caps is None else len(caps), path_wise)
+        want_idx, want_loads = oracle.generate_indices_and_loads(mask, caps, pad, path_wise)
+        total = int(want_loads.sum())
+        for P in (total, total + 37, max(total - 5, 0)):
+            idx, loads, counts, rows, tags = hip.route_and_dispatch(mask, x, P, caps, pad, path_wise, dtype=dtype)
+            assert np.array_equal(idx, want_idx) and np.array_equal(loads, want_loads)
+            assert np.array_equal(counts, mask.sum(0))
+            want, want_tags = oracle.dispatch(x, want_idx, want_loads, tag_generating=True, dtype=dtype)
+            n = min(P, total)
+            assert same_bits(rows[:n], want[:n]) and np.array_equal(tags[:n], want_tags[:n])
+            assert not rows[n:].any() and not tags[n:].any()  # rows past the last path are zero
+
+
+def test_route_and_dispatch_refuses_what_it_does_not_take(hip):
+    assert not hip.route_and_dispatch_supported(8192, 65, 1536)        # more than 64 paths
+    assert not hip.route_and_dispatch_supported(8192, 64, 1530)        # rows that are not 16-byte units
+    assert not hip.route_and_dispatch_supported(70000, 64, 1536)       # more cells than its bands hold
+    assert not hip.route_and_dispatch_supported(8192, 64, 1536, 9)     # a capacity menu of more than 8
+    assert hip.route_and_dispatch_supported(8192, 64, 1536, 64, True)  # ... unless it is one per path
+    assert not hip.route_and_dispatch_supported(0, 64, 1536)
+    mask, _ = topk_mask(512, 65, 1, seed=1)
+    x = np.zeros((512, 8), np.float32)
+    with pytest.raises(NotImplementedError) as err:
+        hip.route_and_dispatch(mask, x, 512)
+    assert "generate_indices_and_loads" in str(err.value)
+
+
 def test_dispatch_custom_tags_2d_and_tag_mode(hip):
     T, E, cell = 1500, 4, 6
     mask, _ = topk_mask(T, E, 2, seed=41)

@@ -487,7 +487,7 @@ def test_row_buffers_beyond_two_gib(brt_mod):
     assert torch.equal(back2.view(torch.int16), x.view(torch.int16))
 
 
-def _switch_layer(brt_mod, defer, E, d, dff, cap, pad, dtype, seed):
+def _switch_layer(brt_mod, defer, E, d, dff, cap, pad, dtype, seed, static=False):
     """ScatterRouter(fused_dispatch) -> two homo-fused kernels -> GatherRouter(fused_combine), written
     as benchmark/switch_moe/switch_transformer.py:336-380 and switch_expert.py:62-99 write it."""
     brt, _, ScatterRouter, GatherRouter = brt_mod
@@ -499,6 +499,8 @@ def _switch_layer(brt_mod, defer, E, d, dff, cap, pad, dtype, seed):
     fabric_kwargs = {"supported_capacities": [cap], "capacity_padding": pad}
     if defer:
         fabric_kwargs["defer_dispatch"] = True
+    if static:
+        fabric_kwargs["static_rows"] = True
     scatter = ScatterRouter(protocol_type="topk", fabric_type="fused_dispatch",
                             fabric_kwargs=fabric_kwargs).cuda()
     gather = GatherRouter(fabric_type="fused_combine").cuda()
@@ -544,6 +546,14 @@ def test_deferred_fused_dispatch_is_the_same_layer_in_four_launches(brt_mod, pad
     assert calls[0] == 6 + casts and calls[1] == 5 + casts, calls
     assert torch.equal(results[0], results[1])
     assert not torch.equal(results[0], hidden)
+    # static_rows=True: index generation moves the rows itself (one call for the two), nothing is
+    # read back to the host, same bits
+    layer = _switch_layer(brt_mod, False, E, d, dff, cap, pad, dtype, seed=32, static=True)
+    layer(hidden.clone(), score)
+    before = _lib.call_count()
+    out = layer(hidden.clone(), score)
+    assert _lib.call_count() - before == 5 + casts
+    assert torch.equal(out, results[0])
 
 
 def test_deferred_rows_fill_themselves_when_anything_else_reads_them(brt_mod):
