@@ -625,6 +625,19 @@ def test_static_rows_dispatch_reads_nothing_back(brt_mod):
         assert got.shape[0] == bound and torch.equal(got[:rows], want) and int(got[rows:].abs().sum()) == 0
         (plain,) = c_router.dispatch_with_indices_and_loads(x, route.indices, route.loads, rows=bound)
         assert torch.equal(plain, got)
+        # the tags of the rows past the loads are zero whatever the allocator hands out (a stale
+        # valid tag there would let the tag-driven combine overwrite that cell with a zero row)
+        stale = torch.full((bound,), 7, dtype=torch.int32, device="cuda")
+        del stale
+        route2 = c_router.generate_route(torch.from_numpy(mask).cuda(), caps, pad, single_path=True)
+        c_router.dispatch_with_indices_and_loads(x, route2.indices, route2.loads, route=route2, rows=bound)
+        assert route2.row_tags.shape[0] == bound and int(route2.row_tags[rows:].abs().sum()) == 0
+        # the one-step form: same route, same rows, same tags
+        route3, got3 = c_router.route_and_dispatch(x, torch.from_numpy(mask).cuda(), bound, caps, pad,
+                                                   single_path=True)
+        assert torch.equal(got3, got) and torch.equal(route3.row_tags, route2.row_tags)
+        assert torch.equal(route3.indices, route.indices) and torch.equal(route3.loads, route.loads)
+        assert torch.equal(route3.counts, route.counts)
     score = torch.from_numpy(softmax(logits).astype(np.float32)).cuda()
     layer_out = []
     for static in (False, True):
