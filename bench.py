@@ -1061,7 +1061,7 @@ def cpu_baseline(layer):
         yy = torch_path.dispatch(x32, m_idx, m_loads)
         torch_path.combine(yy, m_idx, m_loads, None, x32)
     reps, spent, t_dc = 0, 0.0, []
-    while (spent < 10.0 and reps < 2000) or reps < 5:
+    while (spent < 10.0 and reps < 8000) or reps < 5:
         t1 = time.perf_counter()
         yy = torch_path.dispatch(x32, m_idx, m_loads)
         torch_path.combine(yy, m_idx, m_loads, None, x32)
