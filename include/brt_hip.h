@@ -161,7 +161,8 @@ int brt_hip_dispatch(const void* src, void* dst, const void* gates, const int32_
  * src/router/location.cu:212-257 with src/router/route.cu:13-103 (the reference runs them as
  * separate kernels, router.cc:100-140,180-250); results are bit-identical to the two calls.
  *
- *   mask      [T,E] int32 hot mask              cells    [T, cell_bytes] rows of any dtype
+ *   mask      [T,E] int32 hot mask of zeros and ones (what brt_hip_dispatch assumes when it is
+ *             given counts); cells [T, cell_bytes]: rows of any dtype, 16-byte aligned
  *   rows      [P, cell_bytes] out: EVERY row is written -- routed rows, zeros for the padding
  *             rows of a path and for the rows past the last path (P may exceed sum(loads):
  *             a caller that cannot read the loads back allocates an upper bound)

@@ -139,7 +139,7 @@ def route_and_dispatch_supported(T, E, cell_bytes, n_caps=0, path_wise_padding=F
 
 
 def route_and_dispatch(mask, x_bits, P, caps=None, capacity_padding=False, path_wise_padding=False,
-                       want_tags=True, dtype="f32"):
+                       want_tags=True, dtype="f32", misalign=False):
     """Every output starts poisoned: the entry point has to write all of indices, loads, counts, rows
     and row tags itself."""
     mask = np.ascontiguousarray(mask, dtype=np.int32)
@@ -148,6 +148,12 @@ def route_and_dispatch(mask, x_bits, P, caps=None, capacity_padding=False, path_
     cell_bytes = x_bits.shape[1] * x_bits.dtype.itemsize
     d_mask, d_x = dev(mask), dev(x_bits)
     d_idx = torch.full((T, E), -7, dtype=torch.int32, device="cuda")
+    if misalign:  # int32 arrays that are only 4-byte aligned
+        mbuf = torch.zeros(T * E + 1, dtype=torch.int32, device="cuda")
+        d_mask = mbuf[1:].view(T, E)
+        d_mask.copy_(torch.from_numpy(mask))
+        ibuf = torch.full((T * E + 3,), -7, dtype=torch.int32, device="cuda")
+        d_idx = ibuf[3:].view(T, E)
     d_loads = torch.full((E,), -1, dtype=torch.int32, device="cuda")
     d_counts = torch.full((E,), -1, dtype=torch.int32, device="cuda")
     d_rows = torch.full((P, x_bits.shape[1]), 0x55, dtype=_TORCH_BITS[dtype], device="cuda") if dtype != "f32" \

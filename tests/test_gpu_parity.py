@@ -205,6 +205,19 @@ def test_route_and_dispatch_bit_exact(hip, T, E, k, cell, dtype):
             assert not rows[n:].any() and not tags[n:].any()  # rows past the last path are zero
 
 
+def test_route_and_dispatch_with_int32_arrays_that_are_only_4_byte_aligned(hip):
+    T, E, cell = 3001, 13, 72
+    mask, _ = topk_mask(T, E, 2, seed=77)
+    x = as_dtype_bits(np.random.default_rng(78).standard_normal((T, cell)), "bf16")
+    want_idx, want_loads = oracle.generate_indices_and_loads(mask, [300], False)
+    want, want_tags = oracle.dispatch(x, want_idx, want_loads, tag_generating=True, dtype="bf16")
+    P = int(want_loads.sum()) + 9
+    idx, loads, counts, rows, tags = hip.route_and_dispatch(mask, x, P, [300], dtype="bf16", misalign=True)
+    assert np.array_equal(idx, want_idx) and np.array_equal(loads, want_loads)
+    assert same_bits(rows[:P - 9], want) and np.array_equal(tags[:P - 9], want_tags)
+    assert not rows[P - 9:].any() and not tags[P - 9:].any()
+
+
 def test_route_and_dispatch_refuses_what_it_does_not_take(hip):
     assert not hip.route_and_dispatch_supported(8192, 65, 1536)        # more than 64 paths
     assert not hip.route_and_dispatch_supported(8192, 64, 1530)        # rows that are not 16-byte units
