@@ -92,7 +92,7 @@ __global__ __launch_bounds__(WAVES * 64) void grouped_gemm_kernel(GemmArgs a) {
   static_assert(BN % ROWS_PER_PASS == 0 && ROWS_PER_PASS % 8 == 0, "tile shape");
   constexpr int OUT_ROW = BN * 2 + 16;
   extern __shared__ __attribute__((aligned(16))) char smem[];
-  __shared__ int s_tile[4];  // expert, first row, valid rows, first row counted inside the expert
+  __shared__ int s_tile[5];  // expert, first row, valid rows, first row counted inside the expert, column group (patch order)
   __shared__ int s_cell[BM];  // routed forms: 0-based cell behind each row of the tile, -1 = empty slot
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -104,41 +104,97 @@ __global__ __launch_bounds__(WAVES * 64) void grouped_gemm_kernel(GemmArgs a) {
   // that really exist -- only the device knows how many -- spread evenly), and the
   // column tiles of one row block are consecutive workgroups of that XCD.
   const int xcd = blockIdx.x % kXcds, idx = blockIdx.x / kXcds;
-  const int mt = (idx / a.groups_n) * kXcds + xcd, nt_first = (idx % a.groups_n) * a.walk;
-  const int nt_end = WALKS ? min(nt_first + a.walk, a.tiles_n) : nt_first + 1;  // this workgroup's column tiles
-  if (mt >= a.tiles_m_max) return;
-  if (tid < kWave) {
-    int carry_t = 0, carry_m = 0;
-    bool found = false;
-    for (int base = 0; base < a.E && !found; base += kWave) {
-      const int e = base + lane;
-      const int m = e < a.E ? a.loads[e] : 0;
-      const int tiles = (m + BM - 1) / BM;
-      const int incl_t = wave_inclusive_scan(tiles), incl_m = wave_inclusive_scan(m);
-      const int first_tile = carry_t + incl_t - tiles;
-      const bool hit = mt >= first_tile && mt < first_tile + tiles;
-      const unsigned long long b = __ballot(hit);
-      if (b != 0) {
-        found = true;
-        if (hit) {
-          const int local = mt - first_tile;
-          s_tile[0] = e;
-          s_tile[1] = carry_m + incl_m - m + local * BM;
-          s_tile[2] = min(BM, m - local * BM);
-          s_tile[3] = local * BM;
+  int mt = 0, nt_first = 0;
+  if (a.patch == 0) {
+    mt = (idx / a.groups_n) * kXcds + xcd;
+    nt_first = (idx % a.groups_n) * a.walk;
+    if (mt >= a.tiles_m_max) return;
+    if (tid < kWave) {
+      int carry_t = 0, carry_m = 0;
+      bool found = false;
+      for (int base = 0; base < a.E && !found; base += kWave) {
+        const int e = base + lane;
+        const int m = e < a.E ? a.loads[e] : 0;
+        const int tiles = (m + BM - 1) / BM;
+        const int incl_t = wave_inclusive_scan(tiles), incl_m = wave_inclusive_scan(m);
+        const int first_tile = carry_t + incl_t - tiles;
+        const bool hit = mt >= first_tile && mt < first_tile + tiles;
+        const unsigned long long b = __ballot(hit);
+        if (b != 0) {
+          found = true;
+          if (hit) {
+            const int local = mt - first_tile;
+            s_tile[0] = e;
+            s_tile[1] = carry_m + incl_m - m + local * BM;
+            s_tile[2] = min(BM, m - local * BM);
+            s_tile[3] = local * BM;
+          }
         }
+        carry_t += __shfl(incl_t, kWave - 1, kWave);
+        carry_m += __shfl(incl_m, kWave - 1, kWave);
       }
-      carry_t += __shfl(incl_t, kWave - 1, kWave);
-      carry_m += __shfl(incl_m, kWave - 1, kWave);
+      if (!found && lane == 0) {  // beyond the last row block: how far, and where the rows end
+        s_tile[0] = -1;
+        s_tile[1] = carry_m;
+        s_tile[2] = mt - carry_t;
+      }
     }
-    if (!found && lane == 0) {  // beyond the last row block: how far, and where the rows end
-      s_tile[0] = -1;
-      s_tile[1] = carry_m;
-      s_tile[2] = mt - carry_t;
+  } else {
+    // Patch order, for experts with several row blocks (plain form only): the workgroups are an
+    // ordered list -- expert by expert; inside an expert groups of kPatchRows row blocks; inside
+    // a group the row block changes fastest, then the column group -- and the 32 workgroups an XCD
+    // runs at one time take 32 consecutive entries: kPatchRows row blocks x 8 column groups of one
+    // expert, which share the activation rows AND the weight tiles through that XCD's L2.  With
+    // the row blocks of an expert dealt round-robin over the XCDs (the order above) every row
+    // block streams the expert's weights from memory again.
+    constexpr int kPatchRows = 4, kCusPerXcd = 32;
+    const int t = ((idx / kCusPerXcd) * kXcds + xcd) * kCusPerXcd + idx % kCusPerXcd;
+    if (tid < kWave) {
+      int carry_t = 0, carry_m = 0;
+      bool found = false;
+      for (int base = 0; base < a.E && !found; base += kWave) {
+        const int e = base + lane;
+        const int m = e < a.E ? a.loads[e] : 0;
+        const int blocks = (m + BM - 1) / BM;
+        const int tiles = blocks * a.groups_n;
+        const int incl_t = wave_inclusive_scan(tiles), incl_m = wave_inclusive_scan(m);
+        const int first = carry_t + incl_t - tiles;
+        const bool hit = t >= first && t < first + tiles;
+        if (__ballot(hit) != 0) {
+          found = true;
+          if (hit) {
+            const int local = t - first, per_group = kPatchRows * a.groups_n;
+            const int full = blocks / kPatchRows;
+            const int g = local / per_group;
+            int col, block;
+            if (g < full) {
+              const int r = local - g * per_group;
+              col = r / kPatchRows;
+              block = g * kPatchRows + r % kPatchRows;
+            } else {
+              const int last = blocks - full * kPatchRows;
+              const int r = local - full * per_group;
+              col = r / last;
+              block = full * kPatchRows + r % last;
+            }
+            s_tile[0] = e;
+            s_tile[1] = carry_m + incl_m - m + block * BM;
+            s_tile[2] = min(BM, m - block * BM);
+            s_tile[3] = block * BM;
+            s_tile[4] = col;
+          }
+        }
+        carry_t += __shfl(incl_t, kWave - 1, kWave);
+        carry_m += __shfl(incl_m, kWave - 1, kWave);
+      }
+      if (!found && lane == 0) s_tile[0] = -2;  // beyond the last entry of the list
     }
   }
   __syncthreads();
   const int e = __builtin_amdgcn_readfirstlane(s_tile[0]);
+  if (e == -2) return;
+  if (a.patch != 0) nt_first = __builtin_amdgcn_readfirstlane(s_tile[4]) * a.walk;
+  const int nt_end = WALKS ? min(nt_first + a.walk, a.tiles_n) : nt_first + 1;  // this workgroup's column tiles
   if (e < 0) {
     // The row blocks past the last one clear the tags of the rows no path owns (the layout may be
     // allocated for more rows than the loads add up to): surplus block j takes rows
@@ -556,7 +612,15 @@ int launch_act(GemmArgs& a, hipStream_t st) {
   // only the 4-wavefront tiles have the registers to walk column tiles
   constexpr bool kCanWalk = WAVES == 4;
   if (!kCanWalk) a.walk = 1, a.groups_n = a.tiles_n;
-  const long grid_wgs = static_cast<long>(a.tiles_m_max) * a.groups_n;
+  // Experts with several row blocks (and no routing through tags): patch order, so that the row
+  // blocks of an expert that run side by side on an XCD share its weight tiles.  Measured against
+  // the round-robin order in one process: the ragged task-MoE shape (128 experts, Dirichlet loads)
+  // 1652 -> 1596 us and 1443 -> 1379 us, 8 experts x 4096 rows 1106 -> 1053 us and 1019 -> 999 us,
+  // the top-2 shape with three row blocks per expert the same within 2 %; 2, 8 or 16 row blocks per
+  // patch instead of 4 change these by less than 1 %.
+  a.patch = (a.tags == nullptr && !stream_weights) ? 1 : 0;
+  long grid_wgs = static_cast<long>(a.tiles_m_max) * a.groups_n;
+  if (a.patch) grid_wgs = (grid_wgs + 255) / 256 * 256;  // whole rounds of 32 workgroups per XCD
   const dim3 blocks(static_cast<unsigned>(grid_wgs)), threads(WAVES * 64);
   // more than 64 KB of dynamic LDS has to be allowed once per device and kernel
   auto run = [&](auto walks, auto wstream) -> int {

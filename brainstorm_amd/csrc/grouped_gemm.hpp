@@ -22,6 +22,7 @@ struct GemmArgs {
   int gather, scatter;  // rows of x / of out are addressed through the tags
   int tiles_n, tiles_m_max;
   int walk, groups_n;  // column tiles one workgroup walks, ceil(tiles_n / walk)
+  int patch;           // workgroups in patch order (experts with several row blocks), see the kernel
 };
 
 // GELU(v) = v * Phi(v) = max(v, 0) - |v| * Phi(-|v|), branch free.  The tail probability is

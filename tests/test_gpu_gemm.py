@@ -489,6 +489,25 @@ def test_workgroups_walking_several_column_tiles(K, N):
     run(loads, K, N, act="none", bias=False, seed=K, slack=100)
 
 
+@pytest.mark.parametrize("loads,K,N", [
+    # 1, 2, 3, 4, 5, 8 and 9 row blocks per expert (whole patches of four and remainders), empty
+    # experts in between, one column group and several
+    ([160, 320, 0, 480, 640, 1, 800, 0, 1280, 1441], 256, 256),
+    ([161, 639, 641, 0, 0, 2000, 7, 959], 512, 1536),
+    # more than 64 experts (the lookup scans them 64 at a time), every third one heavy
+    ([700 if e % 3 == 0 else (e % 5) * 40 for e in range(70)], 128, 768),
+    # more row blocks than the chip has CUs and enough column tiles to walk
+    ([4096, 0, 4000, 33, 4096], 256, 4096),
+])
+def test_experts_with_many_row_blocks_in_patch_order(loads, K, N):
+    """More rows than experts x 160: the workgroups of the plain form are laid out in patches of
+    four row blocks x eight column groups per XCD; every row of every expert is still computed once,
+    the rows behind the loads stay untouched."""
+    assert sum(loads) > 160 * len(loads)
+    run(loads, K, N, act="gelu", bias=True, seed=len(loads))
+    run(loads, K, N, act="none", bias=False, seed=K, slack=77)
+
+
 def test_grouped_gemm_random_shapes():
     """Seeded random expert counts, ragged loads (many empty), K and N that are any multiple of
     8, bias and activation at random, slack rows behind the loads."""
