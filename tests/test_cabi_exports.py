@@ -32,6 +32,22 @@ def test_workspace_size_is_monotonic_and_small():
     assert f(1 << 20, 64) < 1 << 20
 
 
+def test_one_step_front_end_says_which_shapes_it_takes_without_a_gpu():
+    """brt_hip_route_and_dispatch_supported / _workspace_bytes are host arithmetic: the shapes of the
+    benchmark configurations are taken, what the kernel cannot hold is refused, and the workspace
+    covers one row of band sums per band plus one."""
+    lib = _lib.lib()
+    ok, ws = lib.brt_hip_route_and_dispatch_supported, lib.brt_hip_route_and_dispatch_workspace_bytes
+    for T, E, cell_bytes in ((8192, 64, 1536), (1024, 16, 2048), (16384, 32, 2048), (100352, 8, 192), (1, 1, 16)):
+        assert ok(T, E, cell_bytes, 1, 0) == 1
+        assert 2 * E * 4 <= ws(T, E, cell_bytes) <= (512 + 1) * E * 4
+    assert ok(8192, 65, 1536, 0, 0) == 0 and ws(8192, 65, 1536) == 0      # more than 64 paths
+    assert ok(8192, 64, 1530, 0, 0) == 0                                  # rows that are not whole 16-byte units
+    assert ok(16385, 64, 1536, 0, 0) == 0 and ok(16384, 64, 1536, 0, 0) == 1  # what 256 bands of 64 rows hold
+    assert ok(8192, 64, 1536, 9, 0) == 0 and ok(8192, 64, 1536, 64, 1) == 1   # capacity menu
+    assert ok(0, 64, 1536, 0, 0) == 0
+
+
 def test_argument_errors_do_not_need_a_gpu():
     handle = _lib.lib()
     assert handle.brt_hip_dispatch(None, None, None, None, None, None, None, None,
