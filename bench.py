@@ -830,6 +830,27 @@ def phase_extras(gpu, layer, steps):
     if not torch.equal(gate_mask, mask):
         sys.exit("bench.py: the gate kernel does not reproduce the argmax mask")
 
+    # the layer from the scores: the gate's mask kernel in front of the step, with and without the
+    # one-step front-end
+    def ffn_and_combine_rd():
+        gpu.check(L.brt_hip_grouped_gemm(
+            y_rd.data_ptr(), layer.wi_tab.data_ptr(), None, layer.h.data_ptr(),
+            loads_counts_rd[0].data_ptr(), E, P, D, DFF, lib.ACT_GELU, gpu.sptr()))
+        gpu.check(L.brt_hip_grouped_gemm(
+            layer.h.data_ptr(), layer.wo_tab.data_ptr(), None, y2_rd.data_ptr(),
+            loads_counts_rd[0].data_ptr(), E, P, DFF, D, lib.ACT_NONE, gpu.sptr()))
+        gpu.check(L.brt_hip_combine_by_tags(
+            y2_rd.data_ptr(), out_rd.data_ptr(), tags_rd.data_ptr(), P, D, T, lib.BF16, lib.BF16,
+            gpu.sptr()))
+
+    g_b = gpu.capture(lambda: (k_gate(), k_route_dispatch(), ffn_and_combine_rd()), steps)
+    g_c = gpu.capture(lambda: (k_gate(), layer.step(0)), steps)
+    for g in (g_b, g_c):
+        gpu.timed(g, 1)
+    extras["layer_from_scores_us"] = {
+        "gate | count | apply+dispatch | ffn | combine": round(gpu.timed(g_b, 1) / steps * 1e3, 2),
+        "gate | count | apply | dispatch | ffn | combine": round(gpu.timed(g_c, 1) / steps * 1e3, 2)}
+
     # ---- the same route in the compact format (k path ids per cell instead of the [T,E] mask)
     logits_d = layer.logits.to(dev)
     c_ids = torch.empty(T, 1, dtype=torch.int32, device=dev)
