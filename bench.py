@@ -261,6 +261,25 @@ def measured_traffic():
     return (json.loads(m.group(1)) if m else {}), (c.group(1) if c else None)
 
 
+def kernel_trace_step_us():
+    """Average launch durations (us) of the step's kernels from the committed rocprofv3
+    --kernel-trace summary, phase `step`, and the commit it was taken at."""
+    path = os.path.join(os.path.dirname(TRAFFIC_FILE), "switch_moe_8k_kernel_trace.md")
+    try:
+        text = open(path).read()
+    except OSError:
+        return {}, None
+    m = re.search(r"^## phase `step`\s*$(.*?)(?=^## |\Z)", text, re.M | re.S)
+    c = re.search(r"^taken_at_commit:\s*(\S+)", text, re.M)
+    total, calls = {}, {}
+    for row in re.finditer(r"^\| `([^`]+)` \| (\d+) \| (\d+) \|", m.group(1) if m else "", re.M):
+        key = _kernel_key(row.group(1))
+        if key is not None and int(row.group(2)) > 1:
+            total[key] = total.get(key, 0.0) + int(row.group(2)) * float(row.group(3))
+            calls[key] = calls.get(key, 0) + int(row.group(2))
+    return {k: total[k] / calls[k] / 1e3 for k in total}, (c.group(1) if c else None)
+
+
 class Gpu:
     """Stream, graph capture and event timing shared by all phases."""
 
@@ -1191,6 +1210,17 @@ def main():
             "avg_us": round(us[dominant], 3), "algorithmic_bytes": nbytes[dominant],
             "launches": "inside the step (bench.py --only instep runs nothing else)",
         }
+        trace_us, trace_commit = kernel_trace_step_us()
+        if dominant in trace_us:  # the kernel's own duration in the same step, from the committed profile
+            result["roofline"]["kernel_trace_avg_us"] = round(trace_us[dominant], 3)
+            result["roofline"]["frac_by_kernel_trace"] = round(
+                nbytes[dominant] / trace_us[dominant] / 1e3 / HBM_PEAK_GBPS, 4)
+            result["roofline"]["kernel_trace_taken_at_commit"] = trace_commit
+            result["roofline"]["avg_us_is"] = (
+                "what the kernel costs the step (it and the boundary to its successor: the step graph "
+                "against the step graph without it); kernel_trace_avg_us is the launch duration of the "
+                "same kernel in the same step as rocprofv3 --kernel-trace reports it "
+                "(profiles/switch_moe_8k_kernel_trace.md, phase step)")
 
     if want("cold"):
         us = phase_routing(gpu, layer, sets, index_sets)
@@ -1230,6 +1260,12 @@ def main():
             "traffic": traffic.get(name), "traffic_taken_at_commit": traffic_commit,
             "avg_us": round(us[name], 3), "algorithmic_bytes": nbytes[name], "flop": flops[name],
         }
+        trace_us, trace_commit = kernel_trace_step_us()
+        if name in trace_us:
+            result["roofline_ffn"]["kernel_trace_avg_us"] = round(trace_us[name], 3)
+            result["roofline_ffn"]["frac_by_kernel_trace"] = round(
+                nbytes[name] / trace_us[name] / 1e3 / HBM_PEAK_GBPS, 4)
+            result["roofline_ffn"]["kernel_trace_taken_at_commit"] = trace_commit
 
     if want("configs"):
         result["configs"] = phase_configs(gpu, args.config)
