@@ -95,6 +95,11 @@ SIGNATURES = {
         [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
          _c_int, _c_int, _c_int, _c_ptr],
     ),
+    "brt_hip_grouped_gemm_accumulate": (
+        _c_int,
+        [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_int,
+         _c_int, _c_int, _c_int, _c_ptr],
+    ),
     "brt_hip_unique_tags_workspace_bytes": (_c_size, [ctypes.c_long, ctypes.c_long]),
     "brt_hip_unique_tags": (
         _c_int,

@@ -94,6 +94,7 @@ __global__ __launch_bounds__(WAVES * 64) void grouped_gemm_kernel(GemmArgs a) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   __shared__ int s_tile[5];  // expert, first row, valid rows, first row counted inside the expert, column group (patch order)
   __shared__ int s_cell[BM];  // routed forms: 0-based cell behind each row of the tile, -1 = empty slot
+  __shared__ float s_gate[BM];  // accumulate form: the weight of each row of the tile
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -235,10 +236,12 @@ __global__ __launch_bounds__(WAVES * 64) void grouped_gemm_kernel(GemmArgs a) {
   if (a.tags != nullptr) {
     for (int r = tid; r < rows; r += THREADS) {
       int cell;
+      size_t gate_at;  // accumulate form: where the row's weight stands
       if (a.tag_vector) {
         const int entry = a.tags[static_cast<size_t>(row0) + r];
         cell = a.tag_div > 1 ? (entry - 1) / a.tag_div : entry - 1;
         cell = (entry >= 1 && cell < a.T) ? cell : -1;
+        gate_at = static_cast<size_t>(max(entry, 1)) - 1;
       } else {
         // the tag matrix has T rows; a load padded beyond T (capacity above the batch size) names
         // slots that do not exist: they are empty, as in dispatch (route.cu:84-92 bounds the slot
@@ -246,8 +249,10 @@ __global__ __launch_bounds__(WAVES * 64) void grouped_gemm_kernel(GemmArgs a) {
         const int slot = seat0 + r;
         const int tag = slot < a.T ? a.tags[static_cast<size_t>(slot) * a.E + e] : 0;
         cell = (tag >= 1 && tag <= a.T) ? tag - 1 : -1;
+        gate_at = static_cast<size_t>(max(cell, 0)) * a.E + e;
       }
       s_cell[r] = cell;
+      if (a.gates != nullptr) s_gate[r] = a.gates[cell >= 0 ? gate_at : 0];  // entry 0 for an empty slot: never used
       // side output for a combine that runs later: the cell of every row, written once per row block
       if (a.row_tags_out != nullptr && nt_first == 0) a.row_tags_out[static_cast<size_t>(row0) + r] = cell + 1;
     }
@@ -532,6 +537,24 @@ __global__ __launch_bounds__(WAVES * 64) void grouped_gemm_kernel(GemmArgs a) {
       }
       __syncthreads();
       const int r_lo = i_lo * 32, r_hi = min(rows, i_hi * 32);
+      if (a.gates != nullptr) {
+        // Accumulate form: the weighted combine of a route with several paths per cell is folded
+        // into the store (route.cu:236-243: `in * gate`, then an atomic add per element).  The
+        // value is the row as the separate GEMM would have stored it (rounded to bf16), times the
+        // gate in fp32, added to the fp32 output; 64 consecutive columns of one row per wavefront
+        // and instruction.  Two addends per cell give the same bits in either order.
+        float* const of = a.acc_out + n0;
+        for (int q = tid_e; q < (r_hi - r_lo) * BN; q += THREADS) {
+          const int rl = q / BN, c = q - rl * BN;
+          const int r = r_lo + rl;
+          const int to = s_cell[r];
+          if (to >= 0 && n0 + c < a.N) {
+            const float v = static_cast<float>(*reinterpret_cast<const __bf16*>(stage_out + rl * OUT_ROW + c * 2));
+            unsafeAtomicAdd(of + static_cast<size_t>(to) * a.N + c, v * s_gate[r]);
+          }
+        }
+        continue;
+      }
       for (int q = tid_e; q < (r_hi - r_lo) * OUT_CHUNKS; q += THREADS) {
         const int rl = q / OUT_CHUNKS, c = q - rl * OUT_CHUNKS;
         const int r = r_lo + rl;
@@ -686,7 +709,8 @@ namespace {
 int grouped_gemm_impl(const void* x, const void* const* weights, const void* const* biases, void* out,
                       const int32_t* loads, const int32_t* tags, int entries_per_cell, int E, int P,
                       int T, int K, int N, int act, int gather_in, int scatter_out, void* stream,
-                      bool out_is_f32 = false, int32_t* row_tags_out = nullptr) {
+                      bool out_is_f32 = false, int32_t* row_tags_out = nullptr,
+                      const float* gates = nullptr) {
   if (E <= 0 || P < 0 || K <= 0 || N <= 0 || T < 0)
     return fail(BRT_E_INVALID, "bad shape E=%d P=%d T=%d K=%d N=%d", E, P, T, K, N);
   if (K % 8 != 0 || N % 8 != 0)
@@ -700,12 +724,16 @@ int grouped_gemm_impl(const void* x, const void* const* weights, const void* con
   if (gather_in && static_cast<size_t>(T) * K * 2 > 0x7fffffffull)
     return fail(BRT_E_UNSUPPORTED, "gathered input of %d x %d exceeds 2 GiB", T, K);
   if (!aligned(x, 16) || !aligned(out, 16)) return fail(BRT_E_INVALID, "x/out must be 16-byte aligned");
+  if (gates != nullptr && (!scatter_out || out_is_f32 || !aligned(gates, 4)))
+    return fail(BRT_E_INVALID, "the accumulate form scatters into an fp32 output and needs 4-byte aligned gates");
   GemmArgs a{};
   a.x = static_cast<const __bf16*>(x);
   a.w = reinterpret_cast<const __bf16* const*>(weights);
   a.bias = reinterpret_cast<const __bf16* const*>(biases);
-  a.out = out_is_f32 ? nullptr : static_cast<__bf16*>(out);
+  a.out = (out_is_f32 || gates != nullptr) ? nullptr : static_cast<__bf16*>(out);
   a.out_f32 = out_is_f32 ? static_cast<float*>(out) : nullptr;
+  a.gates = gates;
+  a.acc_out = gates != nullptr ? static_cast<float*>(out) : nullptr;
   a.row_tags_out = tags != nullptr ? row_tags_out : nullptr;
   a.loads = loads;
   a.tags = tags;
@@ -808,6 +836,18 @@ extern "C" int brt_hip_cast_f32_to_bf16(const float* src, void* dst, size_t n, v
   hipLaunchKernelGGL(cast_f32_to_bf16_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0,
                      as_stream(stream), src, static_cast<__bf16*>(dst), n);
   return check_launch("cast_f32_to_bf16_kernel");
+}
+
+extern "C" int brt_hip_grouped_gemm_accumulate(const void* x, const void* const* weights,
+                                               const void* const* biases, float* out,
+                                               const int32_t* loads, const int32_t* tags,
+                                               int entries_per_cell, const float* gates, int E, int P,
+                                               int T, int K, int N, int act, int gather_in,
+                                               void* stream) {
+  if (entries_per_cell < 0) return fail(BRT_E_INVALID, "entries per cell must not be negative, got %d", entries_per_cell);
+  if (!gates) return fail(BRT_E_INVALID, "the accumulate form needs the gates");
+  return grouped_gemm_impl(x, weights, biases, out, loads, tags, entries_per_cell, E, P, T, K, N, act,
+                           gather_in, 1, stream, false, nullptr, gates);
 }
 
 extern "C" int brt_hip_grouped_gemm_by_rows(const void* x, const void* const* weights,

@@ -20,6 +20,11 @@ struct GemmArgs {
   int E, P, K, N, T;
   int plain_out;  // ordinary output stores instead of streaming ones (a small output that is read at once)
   int gather, scatter;  // rows of x / of out are addressed through the tags
+  // accumulate form (scatter only): non-null gates turn the store of a row into
+  // acc_out[cell] += gate * (the row rounded to bf16), fp32 atomic adds; gate of the row's cell on
+  // this path from the [T,E] gate matrix, or by the row's entry from the [T*k] weights of the compact route
+  const float* gates;
+  float* acc_out;
   int tiles_n, tiles_m_max;
   int walk, groups_n;  // column tiles one workgroup walks, ceil(tiles_n / walk)
   int patch;           // workgroups in patch order (experts with several row blocks), see the kernel

@@ -48,7 +48,8 @@ def grouped_linear(x: torch.Tensor, out: torch.Tensor, weight_table: torch.Tenso
                    tags: Optional[torch.Tensor] = None, gather: bool = False,
                    scatter: bool = False, rows: Optional[int] = None,
                    row_entries: Optional[torch.Tensor] = None, entries_per_cell: int = 1,
-                   row_tags_out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                   row_tags_out: Optional[torch.Tensor] = None,
+                   gates: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``out[s_e : s_e + loads[e]] = act(x[s_e : s_e + loads[e]] @ W_e^T + b_e)`` for every
     branch e, ``s_e = sum(loads[:e])``, in one launch.  ``weight_table`` /
     ``bias_table`` are int64 device tensors holding the branch pointers.
@@ -66,12 +67,24 @@ def grouped_linear(x: torch.Tensor, out: torch.Tensor, weight_table: torch.Tenso
 
     ``out`` may be fp32 (tag-matrix and plain forms): it then receives the fp32 accumulator after
     bias and activation.  ``row_tags_out`` (``[rows]`` int32, tag-matrix form) receives the
-    1-based cell behind every row of the layout, which is what a later tag-driven combine needs."""
+    1-based cell behind every row of the layout, which is what a later tag-driven combine needs.
+
+    ``gates`` (fp32, ``[cells, paths]`` beside ``tags`` or ``[cells, k]`` beside ``row_entries``) with
+    ``scatter=True`` and an fp32 ``out`` folds the weighted combine of a route with several paths
+    per cell into the store (route.cu:236-243): ``out[cell] += gate * bf16(row)`` by fp32 atomic
+    adds, so ``out`` must hold zeros (or what the sums are added to) before the call.  Equal to
+    ``combine_with_indices_and_loads`` on the separate GEMM's output: bit for bit with at most two
+    paths per cell, to the last bits of an fp32 sum taken in another order with more."""
     if x.dtype != torch.bfloat16 or out.dtype not in (torch.bfloat16, torch.float32):
         raise NotImplementedError("the grouped GEMM computes in bf16 (fp32 accumulation); "
                                   "the output is bf16 or fp32")
     f32_out = out.dtype == torch.float32
-    if f32_out and row_entries is not None:
+    if gates is not None:
+        if not (scatter and f32_out):
+            raise RuntimeError("gates fold the weighted combine into the store: scatter=True and an fp32 out")
+        if not gates.is_cuda or gates.dtype != torch.float32 or not gates.is_contiguous():
+            raise RuntimeError("gates must be a contiguous fp32 device tensor")
+    elif f32_out and row_entries is not None:
         raise NotImplementedError("the row-entry form writes bf16")
     if not (x.is_cuda and out.is_cuda and loads.is_cuda):
         raise RuntimeError("grouped_linear needs device tensors")
@@ -115,7 +128,16 @@ def grouped_linear(x: torch.Tensor, out: torch.Tensor, weight_table: torch.Tenso
         lib = _lib.lib()
         stream = torch._C._cuda_getCurrentRawStream(torch._C._cuda_getDevice())
         bias_ptr = None if bias_table is None else bias_table.data_ptr()
-        if routed and row_entries is not None:
+        if gates is not None:
+            by_rows = row_entries is not None
+            k = int(entries_per_cell) if by_rows else 0
+            if gates.numel() != cells * (k if by_rows else loads.numel()):
+                raise RuntimeError("gates must hold one weight per cell and path (tags) or per entry (row_entries)")
+            _lib.check(lib.brt_hip_grouped_gemm_accumulate(
+                x.data_ptr(), weight_table.data_ptr(), bias_ptr, out.data_ptr(), loads.data_ptr(),
+                (row_entries if by_rows else tags).data_ptr(), k, gates.data_ptr(), loads.numel(), rows,
+                cells, in_features, out_features, _ACT[activation], int(gather), stream))
+        elif routed and row_entries is not None:
             _lib.check(lib.brt_hip_grouped_gemm_by_rows(
                 x.data_ptr(), weight_table.data_ptr(), bias_ptr, out.data_ptr(), loads.data_ptr(),
                 row_entries.data_ptr(), int(entries_per_cell), loads.numel(), rows, cells,

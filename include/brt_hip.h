@@ -322,6 +322,30 @@ int brt_hip_grouped_gemm_by_rows(const void* x, const void* const* weights,
                                  const int32_t* row_entries, int k, int E, int P, int T, int K,
                                  int N, int act, int gather_in, int scatter_out, void* stream);
 
+/*
+ * The routed grouped GEMM with the WEIGHTED combine of a route with several paths per cell folded
+ * into its store (the weighted branch of combine_with_seat_indices, src/router/route.cu:236-243:
+ * `in * gate`, then one atomic add per element): for every row r of the dispatched layout that a
+ * cell c owns on path e,
+ *     out[c, :] += gates(c, e) * bf16(act(x_row @ W_e^T + b_e))
+ * with fp32 atomic adds into the fp32 matrix out [T,N], which the caller has filled with zeros (or
+ * with what the sums are to be added to) before the call; cells without a row are not touched.  The
+ * addend is exactly what brt_hip_grouped_gemm_routed would store for the row (rounded to bf16)
+ * times the fp32 gate, so the result equals brt_hip_combine on that GEMM's output with fp32 gates
+ * and fp32 out: bit for bit with at most two paths per cell (an fp32 sum of two does not depend on
+ * the order), to the last bits of an fp32 sum in another order with more.
+ * entries_per_cell = 0: tags is the [T,E] tag matrix and gates the [T,E] fp32 gate matrix;
+ * entries_per_cell = k > 0: tags is the row-entry vector [P] of brt_hip_route_by_path and gates its
+ * [T,k] fp32 weights (the weight of a row is gates[entry-1]).  gather_in as in
+ * brt_hip_grouped_gemm_routed.  Calls that add into the same out on different streams at the same
+ * time are summed correctly; nothing else may write out meanwhile.
+ */
+int brt_hip_grouped_gemm_accumulate(const void* x, const void* const* weights,
+                                    const void* const* biases, float* out, const int32_t* loads,
+                                    const int32_t* tags, int entries_per_cell, const float* gates,
+                                    int E, int P, int T, int K, int N, int act, int gather_in,
+                                    void* stream);
+
 /* ---------------------------------------------------------------------------
  * Tag-index gather (the default GatherRouter path of the reference).
  *

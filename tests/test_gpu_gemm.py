@@ -354,7 +354,7 @@ def test_gathering_gemm_on_a_top2_compact_route():
     loads, counts, seat_rows, row_entries = c_router.route_by_path(ids, E, caps)
     P = int(loads.sum())
     assert int(counts.max()) > 220                      # some entries are dropped
-    _, t1 = _expert_tables(E, d, dff, 4)
+    w1, t1 = _expert_tables(E, d, dff, 4)   # the table holds addresses: the weights have to stay alive
     y = c_router.dispatch_by_rows(x, row_entries, k)
     want = torch.empty(P, dff, dtype=torch.bfloat16, device="cuda")
     grouped_linear(y[:P].contiguous(), want, t1, None, loads, d, dff, "gelu")
@@ -362,6 +362,7 @@ def test_gathering_gemm_on_a_top2_compact_route():
     grouped_linear(x, got, t1, None, loads, d, dff, "gelu", row_entries=row_entries,
                    entries_per_cell=k, gather=True, rows=P)
     assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+    del w1
 
 
 def test_routed_gemm_argument_checks():
@@ -561,3 +562,111 @@ def test_scattering_gemm_stores_plus_zero_where_the_combine_would():
     out_r = residual.clone()
     grouped_linear(y, out_r, table, None, loads, K, N, row_entries=row_entries, scatter=True, rows=T)
     assert torch.equal(out_r.view(torch.int16), want.view(torch.int16))
+
+
+@pytest.mark.parametrize("T,E,d,dff,k,cap,pad", [
+    (2048, 16, 256, 512, 2, 300, False),    # top-2, overflow dropped
+    (2048, 16, 256, 512, 2, 300, True),     # every expert padded to the capacity
+    (1000, 8, 136, 264, 2, 400, False),     # several row blocks per expert, K and N tails
+    (300, 64, 64, 128, 2, 16, False),       # most experts nearly empty
+    (1500, 12, 192, 320, 1, 200, False),    # one path per cell: a weighted scatter
+    (900, 10, 128, 448, 3, 350, False),     # three addends per cell: the order of the sum is free
+    (16, 4, 64, 128, 2, 32, True),          # capacity above the batch size
+])
+def test_weighted_combine_folded_into_the_store_of_the_second_gemm(T, E, d, dff, k, cap, pad):
+    """dispatch -> GEMM -> GEMM -> weighted combine into fp32 (route.cu:236-243) against the second
+    GEMM adding gate * row into the fp32 output itself.  The separate combine is first checked
+    against the oracle on the same rows; with at most two paths per cell the folded form must give
+    the same bits (an fp32 sum of two does not depend on the order), with three the same sum in
+    another order (2e-6 relative to the largest value)."""
+    import hip_ops
+    import oracle
+    from brainstorm_amd._C import router as c_router
+    from brainstorm_amd.jit import grouped_linear
+    from routing_cases import topk_mask
+
+    mask, logits = topk_mask(T, E, k, seed=T + E + k)
+    p = np.exp(logits - logits.max(1, keepdims=True)) * mask
+    gates_np = (p / p.sum(1, keepdims=True)).astype(np.float32)
+    d_mask, gates = torch.from_numpy(mask).cuda(), torch.from_numpy(gates_np).cuda()
+    caps = torch.tensor([cap], dtype=torch.int32, device="cuda")
+    x = torch.randn(T, d, generator=torch.Generator().manual_seed(T)).to(torch.bfloat16).cuda()
+    w1, t1 = _expert_tables(E, d, dff, 1)   # the tables hold addresses: the weights have to stay alive
+    w2, t2 = _expert_tables(E, dff, d, 2)
+
+    # the separate kernels, through the C ABI
+    idx, loads = c_router.generate_indices_and_loads(d_mask, caps, pad)
+    (y,) = c_router.dispatch_with_indices_and_loads(x, idx, loads)
+    P = y.shape[0]
+    h = torch.empty(P, dff, dtype=torch.bfloat16, device="cuda")
+    y2 = torch.empty(P, d, dtype=torch.bfloat16, device="cuda")
+    grouped_linear(y, h, t1, None, loads, d, dff, "gelu")
+    grouped_linear(h, y2, t2, None, loads, dff, d)
+    y2_bits = y2.view(torch.int16).cpu().numpy().view(np.uint16)
+    want = hip_ops.combine(y2_bits, idx.cpu().numpy(), loads.cpu().numpy(), gates_np,
+                           in_dtype="bf16", out_dtype="f32", gate_dtype="f32")
+    want_oracle = oracle.combine(y2_bits, idx.cpu().numpy(), loads.cpu().numpy(), gates_np,
+                                 in_dtype="bf16", out_dtype="f32", gate_dtype="f32")
+    assert np.array_equal(want.view(np.uint32), want_oracle.view(np.uint32))
+    want = torch.from_numpy(want.view(np.float32).reshape(T, d)).cuda()
+
+    def check(got):
+        if k <= 2:
+            assert torch.equal(got.view(torch.int32), want.view(torch.int32))
+        else:
+            assert (got - want).abs().max() <= 2e-6 * want.abs().max()
+
+    # the tag matrix names the rows
+    tags, loads_t = c_router.generate_indices_and_loads(d_mask, caps, pad, False, True)
+    assert torch.equal(loads_t, loads)
+    out = torch.zeros(T, d, dtype=torch.float32, device="cuda")
+    grouped_linear(h, out, t2, None, loads, dff, d, tags=tags, scatter=True, rows=P, gates=gates)
+    check(out)
+    # twice into the same output: the call adds to what is there
+    if k == 1:
+        grouped_linear(h, out, t2, None, loads, dff, d, tags=tags, scatter=True, rows=P, gates=gates)
+        assert torch.equal(out, want + want)
+
+    # the row-entry vector of the compact route names the rows; its weights are [T, k]
+    ids = torch.from_numpy(np.argsort(-mask, axis=1, kind="stable")[:, :k].astype(np.int32)).cuda()
+    ids = torch.sort(ids, dim=1).values.contiguous()
+    weights = torch.gather(gates, 1, ids.long()).contiguous()
+    loads_c, _, _, row_entries = c_router.route_by_path(ids, E, caps, pad, rows=P)
+    assert torch.equal(loads_c, loads)
+    out_r = torch.zeros(T, d, dtype=torch.float32, device="cuda")
+    grouped_linear(h, out_r, t2, None, loads, dff, d, row_entries=row_entries, entries_per_cell=k,
+                   scatter=True, rows=P, gates=weights)
+    check(out_r)
+
+    # gathering and accumulating in one call each: no dispatched rows, no combine
+    hf = torch.empty(P, dff, dtype=torch.bfloat16, device="cuda")
+    grouped_linear(x, hf, t1, None, loads, d, dff, "gelu", tags=tags, gather=True, rows=P)
+    assert torch.equal(hf.view(torch.int16), h.view(torch.int16))
+    out_f = torch.zeros(T, d, dtype=torch.float32, device="cuda")
+    grouped_linear(hf, out_f, t2, None, loads, dff, d, tags=tags, scatter=True, rows=P, gates=gates)
+    check(out_f)
+    del w1, w2
+
+
+def test_accumulate_form_argument_checks():
+    from brainstorm_amd.jit import grouped_linear
+
+    T, E, d = 64, 4, 64
+    x = torch.zeros(T, d, dtype=torch.bfloat16, device="cuda")
+    w, t = _expert_tables(E, d, d, 1)
+    loads = torch.full((E,), 16, dtype=torch.int32, device="cuda")
+    tags = torch.zeros(T, E, dtype=torch.int32, device="cuda")
+    gates = torch.ones(T, E, device="cuda")
+    with pytest.raises(RuntimeError):   # bf16 output
+        grouped_linear(x, torch.zeros(T, d, dtype=torch.bfloat16, device="cuda"), t, None, loads, d, d,
+                       tags=tags, scatter=True, rows=T, gates=gates)
+    with pytest.raises(RuntimeError):   # no scatter
+        grouped_linear(x, torch.zeros(T, d, device="cuda"), t, None, loads, d, d, tags=tags, gather=True,
+                       rows=T, gates=gates)
+    with pytest.raises(RuntimeError):   # gates of the wrong size
+        grouped_linear(x, torch.zeros(T, d, device="cuda"), t, None, loads, d, d, tags=tags, scatter=True,
+                       rows=T, gates=gates[:, :2].contiguous())
+    out = torch.zeros(T, d, device="cuda")
+    grouped_linear(x, out, t, None, loads, d, d, tags=tags, scatter=True, rows=T, gates=gates)
+    assert not out.any()                # an empty tag matrix adds nothing
+    del w
