@@ -695,6 +695,70 @@ def ffn_config(gpu, loads_np, d, dff, seed, spot_checks=3):
     return res
 
 
+def accumulate_config(gpu):
+    """The tail of configuration 3's layer (top-2, fp32 result): the contracting GEMM followed by
+    the weighted combine, against the GEMM that adds gate * row into the fp32 result itself
+    (after a fill kernel has zeroed it).  Both orders of kernels are timed as graphs of launches;
+    the results must agree bit for bit (two paths per cell)."""
+    import numpy as np
+    import workloads
+
+    torch, L, lib, dev = gpu.torch, gpu.L, gpu._lib, gpu.dev
+    _, throttled, gates_np, loads_np = workloads.top2_skewed_route()
+    Tn, En = throttled.shape
+    d, dff = 1024, 4096
+    routed = torch.from_numpy(throttled).cuda()
+    gates = torch.from_numpy(gates_np).cuda()
+    ws = torch.empty(max(16, L.brt_hip_scan_workspace_bytes(Tn, En)), dtype=torch.uint8, device=dev)
+    idx, tags = torch.empty_like(routed), torch.zeros_like(routed)
+    loads_counts = torch.empty(2, En, dtype=torch.int32, device=dev)
+    loads = loads_counts[0]
+    for out_idx, is_tag in ((idx, 0), (tags, 1)):
+        gpu.run(lambda: gpu.check(L.brt_hip_generate_indices_and_loads(
+            routed.data_ptr(), out_idx.data_ptr(), loads.data_ptr(), loads_counts[1].data_ptr(), Tn, En,
+            None, 0, 0, 0, is_tag, ws.data_ptr(), ws.numel(), gpu.sptr())))
+    if not np.array_equal(loads.cpu().numpy(), loads_np):
+        sys.exit("bench.py: configuration 3: the loads of the route differ from the workload's")
+    P = int(loads_np.sum())
+    g = torch.Generator(device="cuda").manual_seed(33)
+    h = torch.randn(P, dff, generator=g, device=dev).to(torch.bfloat16)
+    w2 = (torch.randn(En, d, dff, generator=g, device=dev) * 0.02).to(torch.bfloat16)
+    t2 = torch.tensor([w2[e].data_ptr() for e in range(En)], dtype=torch.int64, device=dev)
+    y2 = torch.empty(P, d, dtype=torch.bfloat16, device=dev)
+    out_sep = torch.empty(Tn, d, dtype=torch.float32, device=dev)
+    out_acc = torch.empty(Tn, d, dtype=torch.float32, device=dev)
+
+    def k_gemm2():
+        gpu.check(L.brt_hip_grouped_gemm(h.data_ptr(), t2.data_ptr(), None, y2.data_ptr(), loads.data_ptr(),
+                                         En, P, dff, d, lib.ACT_NONE, gpu.sptr()))
+
+    def k_combine():
+        gpu.check(L.brt_hip_combine(y2.data_ptr(), out_sep.data_ptr(), gates.data_ptr(), idx.data_ptr(),
+                                    loads.data_ptr(), Tn, d, En, P, 0, 0, lib.BF16, lib.F32, lib.F32,
+                                    gpu.sptr()))
+
+    def k_zero():
+        out_acc.zero_()
+
+    def k_accumulate():
+        gpu.check(L.brt_hip_grouped_gemm_accumulate(
+            h.data_ptr(), t2.data_ptr(), None, out_acc.data_ptr(), loads.data_ptr(), tags.data_ptr(), 0,
+            gates.data_ptr(), En, P, Tn, dff, d, lib.ACT_NONE, 0, gpu.sptr()))
+
+    gpu.run(k_gemm2, k_combine, k_zero, k_accumulate)
+    if not torch.equal(out_sep.view(torch.int32), out_acc.view(torch.int32)):
+        sys.exit("bench.py: configuration 3: the accumulating GEMM and GEMM + combine disagree")
+    res = {"cells": Tn, "paths": En, "rows": P, "d": d, "d_ff": dff}
+    for name, fns in (("gemm2_us", [k_gemm2]), ("combine_us", [k_combine]), ("zero_fill_us", [k_zero]),
+                      ("gemm2_accumulate_us", [k_accumulate]),
+                      ("gemm2_then_combine_us", [k_gemm2, k_combine]),
+                      ("zero_fill_then_gemm2_accumulate_us", [k_zero, k_accumulate])):
+        res[name] = round(gpu.launch_us(fns, launches=24) * len(fns), 1)
+    res["note"] = ("each figure is one pass over the named kernels, launched back to back in a graph; the two "
+                   "orders give bit-identical fp32 results (checked)")
+    return res
+
+
 def phase_configs(gpu, only=None):
     """`only`: a substring that selects the configurations to run (for counter runs of one of them)."""
     import numpy as np
@@ -713,6 +777,8 @@ def phase_configs(gpu, only=None):
     if want("cfg5_task_moe_ffn_128e_2048_8192"):
         loads5 = workloads.dirichlet_loads(32768, 128, 0.3, seed=5)
         out["cfg5_task_moe_ffn_128e_2048_8192"] = ffn_config(gpu, loads5.astype(np.int64), 2048, 8192, seed=5)
+    if want("cfg3_top2_combine_folded_into_gemm2"):
+        out["cfg3_top2_combine_folded_into_gemm2"] = accumulate_config(gpu)
     # what the same kernel does when the shape lets the matrix units be the bound: the same rows
     # and feature sizes over 8 experts of 4096 rows (weights 268 MB per GEMM)
     if want("compute_bound_probe_8e_x_4096_rows_2048_8192"):

@@ -670,3 +670,41 @@ def test_accumulate_form_argument_checks():
     grouped_linear(x, out, t, None, loads, d, d, tags=tags, scatter=True, rows=T, gates=gates)
     assert not out.any()                # an empty tag matrix adds nothing
     del w
+
+
+def test_top2_weighted_combine_folded_at_full_size():
+    """BASELINE configuration 3 (16384 cells, 32 paths, top-2 under a Zipf bias, throttled to 2048
+    cells per path, renormalised gates): the contracting GEMM 4096 -> 1024 adding gate * row into
+    the fp32 result against the same GEMM followed by the weighted combine, bit for bit."""
+    from workloads import top2_skewed_route
+    from brainstorm_amd._C import router as c_router
+    from brainstorm_amd.jit import grouped_linear
+
+    _, throttled, gates_np, loads_np = top2_skewed_route()
+    T, E = throttled.shape
+    d, dff = 1024, 4096
+    routed, gates = torch.from_numpy(throttled).cuda(), torch.from_numpy(gates_np).cuda()
+    idx, loads = c_router.generate_indices_and_loads(routed)
+    tags, loads_t = c_router.generate_indices_and_loads(routed, None, False, False, True)
+    assert np.array_equal(loads.cpu().numpy(), loads_np) and torch.equal(loads, loads_t)
+    P = int(loads_np.sum())
+    g = torch.Generator().manual_seed(33)
+    h = torch.randn(P, dff, generator=g).to(torch.bfloat16).cuda()
+    w2, t2 = _expert_tables(E, dff, d, 7)
+    y2 = torch.empty(P, d, dtype=torch.bfloat16, device="cuda")
+    grouped_linear(h, y2, t2, None, loads, dff, d)
+    (want,) = c_router.combine_with_indices_and_loads(y2, idx, loads, gates, out_dtype=torch.float32)
+    out = torch.zeros(T, d, dtype=torch.float32, device="cuda")
+    grouped_linear(h, out, t2, None, loads, dff, d, tags=tags, scatter=True, rows=P, gates=gates)
+    assert torch.equal(out.view(torch.int32), want.view(torch.int32))
+    # every cell's sum against fp64 on the rows the separate GEMM stored
+    cells = torch.from_numpy(np.nonzero(throttled.any(1))[0][:64]).cuda()
+    ref = torch.zeros(len(cells), d, dtype=torch.float64, device="cuda")
+    starts = np.concatenate([[0], np.cumsum(loads_np)])
+    idx_h = idx.cpu().numpy()
+    for j, c in enumerate(cells.tolist()):
+        for e in np.nonzero(throttled[c])[0]:
+            row = int(starts[e]) + int(idx_h[c, e]) - 1
+            ref[j] += y2[row].double() * float(gates_np[c, e])
+    assert (out[cells].double() - ref).abs().max() <= 1e-6 * ref.abs().max()
+    del w2
