@@ -1153,7 +1153,14 @@ def phase_api(gpu, layer, steps):
         graph = gpu.capture(step, steps)
         gpu.timed(graph, 1)
         us = min(gpu.timed(graph, 1) for _ in range(3)) * 1e3 / steps
-        out[name] = {"layer_us": round(us, 2), "library_calls_per_layer": calls}
+        # the same step issued by the interpreter, launch after launch (no graph): wall clock
+        eager_steps = 200
+        gpu.run(*([step] * 20))
+        t_wall = time.perf_counter()
+        gpu.run(*([step] * eager_steps))
+        eager_us = (time.perf_counter() - t_wall) * 1e6 / eager_steps
+        out[name] = {"layer_us": round(us, 2), "library_calls_per_layer": calls,
+                     "layer_us_eager_wall_clock": round(eager_us, 1)}
     if not torch.equal(results["static_rows"], results["defer_dispatch"]):
         raise SystemExit("bench: the deferred dispatch changed the layer's result")
     out["note"] = ("library calls per layer include the gate's top-k mask kernel; index generation is "
