@@ -11,6 +11,10 @@ namespace brt {
 // ---- host side: per-thread error text -------------------------------------
 int fail(int code, const char* fmt, ...);  // records the message, returns code
 int check_launch(const char* what);        // hipGetLastError -> BRT_E_LAUNCH
+// More than 64 KB of dynamic LDS has to be allowed once per kernel and device.  Thread-safe; the
+// first call for a kernel on a device changes a function attribute, so it must not happen while a
+// stream is being captured into a graph (make the first call of each op outside the capture).
+int allow_dynamic_lds(const void* kernel, int bytes);
 
 inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
 inline bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }

@@ -645,18 +645,9 @@ int launch_act(GemmArgs& a, hipStream_t st) {
   long grid_wgs = static_cast<long>(a.tiles_m_max) * a.groups_n;
   if (a.patch) grid_wgs = (grid_wgs + 255) / 256 * 256;  // whole rounds of 32 workgroups per XCD
   const dim3 blocks(static_cast<unsigned>(grid_wgs)), threads(WAVES * 64);
-  // more than 64 KB of dynamic LDS has to be allowed once per device and kernel
   auto run = [&](auto walks, auto wstream) -> int {
     auto* fn = &grouped_gemm_kernel<MT, NT, WAVES, ACT, decltype(walks)::value, decltype(wstream)::value>;
-    static bool configured[64] = {};
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 63;
-    if (!configured[dev] || dev == 63) {
-      if (hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize,
-                              static_cast<int>(lds)) != hipSuccess)
-        return fail(BRT_E_LAUNCH, "cannot reserve %zu bytes of LDS", lds);
-      configured[dev] = true;
-    }
+    if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(fn), static_cast<int>(lds)); rc != BRT_OK) return rc;
     hipLaunchKernelGGL(fn, blocks, threads, lds, st, a);
     return check_launch("grouped_gemm_kernel");
   };
@@ -678,15 +669,7 @@ int launch_f32(GemmArgs& a, hipStream_t st) {
   a.walk = 1;
   a.groups_n = a.tiles_n;
   auto* fn = &grouped_gemm_kernel<MT, NT, WAVES, ACT, false, false, true>;
-  static bool configured[64] = {};
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 63;
-  if (!configured[dev] || dev == 63) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            2 * STAGE) != hipSuccess)
-      return fail(BRT_E_LAUNCH, "cannot reserve %d bytes of LDS", 2 * STAGE);
-    configured[dev] = true;
-  }
+  if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(fn), 2 * STAGE); rc != BRT_OK) return rc;
   const long grid_wgs = static_cast<long>(a.tiles_m_max) * a.groups_n;
   hipLaunchKernelGGL(fn, dim3(static_cast<unsigned>(grid_wgs)), dim3(WAVES * 64), 2 * STAGE, st, a);
   return check_launch("grouped_gemm_kernel (fp32 output)");
@@ -753,6 +736,16 @@ int grouped_gemm_impl(const void* x, const void* const* weights, const void* con
     if (act == BRT_ACT_RELU) return launch_f32<BRT_ACT_RELU>(a, as_stream(stream));
     return launch_f32<BRT_ACT_NONE>(a, as_stream(stream));
   }
+  // Kernel choice.  Experts that average more than one row block, and enough 256 x 256 tiles for two
+  // full rounds over the CUs: the ping-pong kernel (grouped_gemm_pingpong.hip), whose tile moves a
+  // third fewer operand bytes per flop.  Measured in one process against the 160-row kernel: 8
+  // experts x 4096 rows 2048 -> 8192 -> 2048 1165 / 993 -> 994 / 831 us, the ragged task-MoE shape
+  // 1585 / 1374 -> 1401 / 1263 us, the top-2 shape's expanding GEMM (912 tiles) 212 -> 174 us; its
+  // contracting GEMM (228 tiles on 256 CUs) 156 -> 177 us, which is why few tiles stay with the
+  // 160-row kernel, like every weight-streaming shape.
+  if (pingpong_gemm_applies(a) && static_cast<long>(P) > static_cast<long>(E) * 160 &&
+      static_cast<long>((P + 255) / 256) * ((N + 255) / 256) >= 2L * device_cus())
+    return launch_pingpong_gemm(a, act, as_stream(stream));
   // Tile choice.  A wavefront owns 160 x 64 outputs (7 LDS fragment reads feed 10 MFMAs); a
   // workgroup is 2, 3 or 4 of them side by side.  The kernel is bound by how fast a CU can fill
   // its L1 (about 29 KB/us, L2 hits included), so the shape is the one that gives the busiest CU

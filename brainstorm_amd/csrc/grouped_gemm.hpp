@@ -30,6 +30,10 @@ struct GemmArgs {
   int patch;           // workgroups in patch order (experts with several row blocks), see the kernel
 };
 
+// The 256 x 256 ping-pong kernel (grouped_gemm_pingpong.hip): the shapes it takes, and its launch.
+bool pingpong_gemm_applies(const GemmArgs& a);
+int launch_pingpong_gemm(GemmArgs& a, int act, hipStream_t st);
+
 // GELU(v) = v * Phi(v) = max(v, 0) - |v| * Phi(-|v|), branch free.  The tail probability is
 // exp2(Q(|v|)) with Q a degree-7 fit of log2 Phi(-x) on [0, 8] (|Q - log2 Phi| < 5e-5 there, so the
 // tail is good to 3.5e-5 relative; beyond 8 the product is below 5e-15 and Q keeps falling to -inf).

@@ -509,6 +509,23 @@ def test_experts_with_many_row_blocks_in_patch_order(loads, K, N):
     run(loads, K, N, act="none", bias=False, seed=K, slack=77)
 
 
+@pytest.mark.parametrize("loads,K,N", [
+    ([1024] * 8, 128, 4096),                                  # two K-steps: the shortest K loop
+    ([3000, 0, 1, 2900, 257, 255, 1500, 700], 256, 4096),     # ragged: empty, one-row and 255/257-row experts
+    ([5000, 31, 4000, 129], 192, 4104),                       # N tail (8 columns in the last tile), odd K-step count
+    ([100] * 60 + [4000], 320, 3584),                         # many experts of one part-filled row block
+    ([70] * 70 + [6000, 3000, 5000], 128, 4096),               # more than 64 experts
+])
+def test_ping_pong_tiles(loads, K, N):
+    """Shapes the host sends to the 256 x 256 ping-pong kernel: experts that average more than 160
+    rows and at least two rounds of tiles over the CUs."""
+    P = sum(loads)
+    assert P > len(loads) * 160 and ((P + 255) // 256) * ((N + 255) // 256) >= 512, "not a ping-pong shape"
+    run(loads, K, N)
+    run(loads, K, N, act="gelu", bias=True, seed=1)
+    run(loads, K, N, act="relu", bias=True, seed=2, slack=300)
+
+
 def test_grouped_gemm_random_shapes():
     """Seeded random expert counts, ragged loads (many empty), K and N that are any multiple of
     8, bias and activation at random, slack rows behind the loads."""
