@@ -422,7 +422,9 @@ def route_and_dispatch(
     n_caps = 0 if supported_capacities is None else supported_capacities.size(0)
     cell_bytes = (in_data.numel() // T) * in_data.element_size() if T > 0 else 0
     lib = _lib.lib()
-    fused = (T > 0 and in_data.dtype in _DT and lib.brt_hip_route_and_dispatch_supported(
+    # (a contiguous view whose storage offset breaks the 16-byte alignment takes the two calls)
+    fused = (T > 0 and in_data.dtype in _DT and in_data.data_ptr() % 16 == 0
+             and lib.brt_hip_route_and_dispatch_supported(
         T, E, cell_bytes, n_caps, int(bool(path_wise_padding and capacity_padding))) == 1)
     if not fused:
         route = generate_route(hot_mask, supported_capacities, capacity_padding, path_wise_padding,

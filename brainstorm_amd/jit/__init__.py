@@ -78,6 +78,9 @@ def grouped_linear(x: torch.Tensor, out: torch.Tensor, weight_table: torch.Tenso
     if x.dtype != torch.bfloat16 or out.dtype not in (torch.bfloat16, torch.float32):
         raise NotImplementedError("the grouped GEMM computes in bf16 (fp32 accumulation); "
                                   "the output is bf16 or fp32")
+    pending = deferred.pending_of(x)
+    if pending is not None:
+        pending.materialize()  # an unfilled deferred buffer handed over as it is: the rows are dispatched first
     f32_out = out.dtype == torch.float32
     if gates is not None:
         if not (scatter and f32_out):
@@ -162,6 +165,8 @@ def grouped_linear(x: torch.Tensor, out: torch.Tensor, weight_table: torch.Tenso
 
 def _to_bf16(t: torch.Tensor) -> torch.Tensor:
     """fp32 -> bf16 (round to nearest even) with the library's cast kernel."""
+    if t.dtype != torch.float32:
+        raise RuntimeError(f"the cast kernel reads fp32, got {t.dtype}")
     t = t.contiguous()
     out = torch.empty(t.shape, dtype=torch.bfloat16, device=t.device)
     if t.numel():
@@ -176,12 +181,16 @@ class _Bf16Weights:
 
     def __init__(self):
         self.keys = None
+        self.sources = None  # the converted tensors are held, so their addresses cannot be reused unnoticed
         self.copies = None
 
     def get(self, tensors: Sequence[torch.Tensor]) -> List[torch.Tensor]:
-        keys = tuple((t.data_ptr(), t._version) for t in tensors)
+        # `.data = ...` swaps the storage without touching the version counter: the storage's own
+        # address and the tensor's identity are part of the key
+        keys = tuple((id(t), t.data_ptr(), t._version, t.untyped_storage().data_ptr()) for t in tensors)
         if keys != self.keys:
             self.copies = [_to_bf16(t.detach()) for t in tensors]
+            self.sources = list(tensors)
             self.keys = keys
         return self.copies
 
@@ -222,8 +231,11 @@ class GroupedLinearKernel:
         if biases:
             biases = self._branch_operands(biases, capacities.numel(), self._biases_bf16, "biases")
         loads = capacities.to(device=out.device, dtype=torch.int32)
-        state = deferred.state_of(x)
-        if state is not None and self._can_gather(state, out):
+        state = deferred.pending_of(x)  # a DeferredRows, or the routed GridTensor itself
+        if state is not None and not self._can_gather(state, out):
+            state.materialize()
+            state = None
+        if state is not None:
             # the rows of a deferred dispatch: read from the cells through the route's tag indices
             route = state.route
             cells = state.cells if state.cells.dtype == torch.bfloat16 else _to_bf16(state.cells)
@@ -244,7 +256,7 @@ class GroupedLinearKernel:
     def _branch_operands(self, tensors, used: int, cache: _Bf16Weights, what: str):
         dtypes = {t.dtype for t in tensors[:used]}
         if dtypes == {torch.float32}:
-            return cache.get(tensors)
+            return cache.get(tensors[:used])  # branches past the capacities are never read, nor converted
         for t in tensors[:used]:
             if t.dtype != torch.bfloat16 or not t.is_contiguous():
                 raise NotImplementedError(f"branch {what} must be contiguous bf16 or fp32 tensors of one dtype")

@@ -363,11 +363,24 @@ class FusedDispatchFabric(DispatchFabric):
         kwargs["index_format"] = "seat_index"
         defer = bool(kwargs.pop("defer_dispatch", False))
         static_rows = bool(kwargs.pop("static_rows", False))
-        caps = kwargs.get("supported_capacities")
         super().__init__(flow_num, route_logic=route_logic, transform=transform, **kwargs)
         self.defer_dispatch = defer
         self.static_rows = static_rows
-        self._host_caps = [caps] if isinstance(caps, int) else list(caps) if caps is not None else None
+        self._host_caps_key = ()   # the capacity buffer the host copy below was read from
+        self._host_caps_list = None
+
+    @property
+    def _host_caps(self) -> Optional[List[int]]:
+        """The capacity menu on the host.  Read back from the buffer once, and again whenever the
+        buffer is replaced or written (``supported_capacities`` is an ordinary module buffer)."""
+        caps = self.supported_capacities
+        if caps is None:
+            return None
+        key = (id(caps), caps._version, caps.data_ptr())
+        if key != self._host_caps_key:
+            self._host_caps_list = [int(c) for c in caps.detach().cpu().tolist()]
+            self._host_caps_key = key
+        return self._host_caps_list
 
     def _defers(self, in_flows, runtime_capacities, hot_mask) -> bool:
         if not (self.defer_dispatch and getattr(hot_mask, "_brt_single_path", False)):
@@ -392,13 +405,14 @@ class FusedDispatchFabric(DispatchFabric):
 
     def _row_bound(self, cells: int, paths: int) -> int:
         """Rows the path-major layout of a single-path route can need, known without reading the loads back."""
-        if self._host_caps is None:
+        caps = self._host_caps
+        if caps is None:
             return cells
         if self.path_wise_padding:
-            return sum(self._host_caps)
+            return sum(caps)
         if self.capacity_padding:
-            return paths * max(self._host_caps)
-        return min(cells, paths * max(self._host_caps))
+            return paths * max(caps)
+        return min(cells, paths * max(caps))
 
     def forward(self, in_flow, hot_mask, runtime_capacities=None, score=None):
         in_flows = [in_flow] if self.flow_num == 1 else in_flow

@@ -8,13 +8,16 @@ activations never happen.  Anything else that touches the tensor -- any torch op
 conversion, a print -- first runs the dispatch it stands for (:meth:`DeferredState.materialize`),
 so code that knows nothing about this sees an ordinary dispatched tensor.
 
-Shape, dtype, device and the data pointer can be read without filling the buffer.
+Shape, dtype and device can be read without filling the buffer.  Anything that yields an
+address or a layout a foreign kernel could read through -- ``data_ptr``, ``stride``,
+``storage_offset``, ``__cuda_array_interface__``, ``__dlpack__`` -- fills it first: a ctypes or
+C-extension consumer of ``routed.data_ptr()`` sees dispatched rows.
 """
 from typing import Any, Optional
 
 import torch
 
-__all__ = ["DeferredState", "DeferredRows", "pending_state", "wrap_if_pending", "settle"]
+__all__ = ["DeferredState", "DeferredRows", "pending_state", "pending_of", "wrap_if_pending", "settle"]
 
 
 class DeferredState:
@@ -52,8 +55,8 @@ for _name in ("shape", "device", "dtype", "ndim", "is_cuda", "requires_grad", "l
     _descr = getattr(torch.Tensor, _name, None)
     if _descr is not None:
         _METADATA.add(_descr.__get__)
-for _name in ("size", "dim", "numel", "nelement", "stride", "is_contiguous", "data_ptr", "element_size",
-              "storage_offset", "is_floating_point", "is_complex", "get_device", "__len__"):
+for _name in ("size", "dim", "numel", "nelement", "is_contiguous", "element_size",
+              "is_floating_point", "is_complex", "get_device", "__len__"):
     _method = getattr(torch.Tensor, _name, None)
     if _method is not None:
         _METADATA.add(_method)
@@ -103,6 +106,22 @@ def state_of(t: torch.Tensor) -> Optional[DeferredState]:
         if state is not None and state.pending:
             return state
     return None
+
+
+# key of a GridTensor's extra attributes in its instance dictionary (runtime/grid_tensor.py)
+_GRID_EXTRA = "cell_extra_attr_dict"
+
+
+def pending_of(t: torch.Tensor) -> Optional[DeferredState]:
+    """The pending state behind ``t``, whether it arrives as a :class:`DeferredRows` or as the
+    GridTensor itself (its extra attributes carry the state); None for any other tensor."""
+    state = state_of(t)
+    if state is None and isinstance(t, torch.Tensor):
+        extra = getattr(t, "__dict__", {}).get(_GRID_EXTRA)
+        if extra:
+            with torch._C.DisableTorchFunctionSubclass():
+                state = pending_state(extra, t)
+    return state
 
 
 def pending_state(extra: Optional[dict], t: torch.Tensor) -> Optional[DeferredState]:

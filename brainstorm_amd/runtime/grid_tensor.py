@@ -183,10 +183,15 @@ class GridTensor(torch.Tensor):
     def __torch_function__(cls, func, types, args=(), kwargs=None):
         # Only plain attribute reads happen before the super() call, so no torch
         # function is re-entered here.
+        kwargs = kwargs or {}
         tags, loads, extra = collect_cell_attr(args)
+        if tags is None and kwargs:  # operands passed by keyword only: torch.matmul(input=..., other=...)
+            tags, loads, extra = collect_cell_attr(list(kwargs.values()))
         if extra and not deferred.is_metadata_read(func):
-            _settle_deferred(args, extra)  # an unfilled dispatch buffer is filled before it is read
-        ret = super().__torch_function__(func, types, args, kwargs or {})
+            # an unfilled dispatch buffer is filled before it is read
+            _settle_deferred(args, extra)
+            _settle_deferred(list(kwargs.values()), extra)
+        ret = super().__torch_function__(func, types, args, kwargs)
         attach_cell_attr(ret, tags, loads, extra)
         return ret
 

@@ -252,6 +252,9 @@ int brt_hip_topk_hot_mask(const void* scores, int32_t* hot_mask, int T, int E, i
  *   K and N must be multiples of 8 (16-byte rows; BRT_E_UNSUPPORTED otherwise), x and out
  *   16-byte aligned.  `act` is one of BRT_ACT_*; GELU is the erf form
  *   (v * Phi(v), to 4.3e-6 absolute before the rounding to bf16).
+ *   The GEMM kernels use more than 64 KB of LDS, which has to be allowed once per kernel and
+ *   device (a function attribute, set under a lock on the first launch): make the first call of
+ *   every GEMM entry point on a device outside a graph capture, as for the static scratch above.
  */
 int brt_hip_grouped_gemm(const void* x, const void* const* weights, const void* const* biases,
                          void* out, const int32_t* loads, int E, int P, int K, int N, int act,

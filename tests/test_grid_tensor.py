@@ -151,8 +151,10 @@ def test_module_paths_of_the_reference_resolve():
 
 def test_deferred_buffer_fills_itself_before_any_read_and_not_for_metadata():
     """Host logic of the deferred dispatch (no GPU: the dispatch itself is replaced by a counter).
-    Shape, dtype, device, data_ptr leave the buffer alone; an operator on the plain tensor or on the
-    GridTensor that wraps it fills it first; afterwards nothing is deferred any more."""
+    Shape, dtype, device leave the buffer alone; an operator on the plain tensor or on the
+    GridTensor that wraps it fills it first, and so does anything that hands out its address
+    (data_ptr, stride, storage_offset: a foreign kernel could read through them); afterwards
+    nothing is deferred any more."""
     import brt
     from brainstorm_amd.runtime import deferred
 
@@ -173,7 +175,7 @@ def test_deferred_buffer_fills_itself_before_any_read_and_not_for_metadata():
         return state, grid
 
     state, grid = make()
-    assert tuple(grid.shape) == (6, 3) and grid.dtype == torch.float32 and grid.data_ptr() == state.buffer.data_ptr()
+    assert tuple(grid.shape) == (6, 3) and grid.dtype == torch.float32 and state.fills == 0
     plain, tags, loads, extra = brt.to_torch_tensor(grid, retrieve_attr=True)
     assert isinstance(plain, deferred.DeferredRows) and deferred.state_of(plain) is state
     assert plain.shape[0] == 6 and plain.device.type == "cpu" and plain.is_contiguous() and state.fills == 0
@@ -187,6 +189,24 @@ def test_deferred_buffer_fills_itself_before_any_read_and_not_for_metadata():
     doubled = grid * 2                       # an operator on the GridTensor fills it too
     assert state.fills == 1 and float(brt.to_torch_tensor(doubled).sum()) == 14.0 * 18
     assert isinstance(doubled, brt.GridTensor) and doubled.extra_attr_dict["brt_deferred_0"] is state
+
+    for read in (lambda t: t.data_ptr(), lambda t: t.stride(), lambda t: t.storage_offset()):
+        state, grid = make()
+        read(grid)                           # the address of the GridTensor: filled first
+        assert state.fills == 1
+        state, grid = make()
+        plain = brt.to_torch_tensor(grid)
+        assert state.fills == 0
+        read(plain)                          # ... and of the plain tensor
+        assert state.fills == 1
+    state, grid = make()
+    assert deferred.pending_of(grid) is state and deferred.pending_of(brt.to_torch_tensor(grid)) is state
+    assert deferred.pending_of(torch.ones(2)) is None and state.fills == 0
+
+    state, grid = make()
+    product = torch.matmul(input=grid, other=torch.ones(3, 2))  # operands passed by keyword only
+    assert state.fills == 1 and float(product.sum()) == 7.0 * 3 * 12
+    assert isinstance(product, brt.GridTensor) and product.extra_attr_dict["brt_deferred_0"] is state
 
     state, grid = make()
     other = torch.ones(6, 3)

@@ -588,6 +588,65 @@ def test_deferred_rows_fill_themselves_when_anything_else_reads_them(brt_mod):
     assert torch.allclose(total, want.float().sum())
 
 
+def test_foreign_consumers_of_a_deferred_buffer_see_dispatched_rows(brt_mod):
+    """What a deferred buffer hands to code that knows nothing of it: a consumer of its address (a
+    ctypes / C-extension kernel taking ``data_ptr()``) finds the rows dispatched, and the grouped
+    GEMM gives the same result whether it receives the plain tensor, the routed GridTensor itself,
+    or the tensor through ``grouped_linear``."""
+    import ctypes
+    from brainstorm_amd.jit import grouped_linear, make_jit_kernel
+
+    brt, c_router, ScatterRouter, GatherRouter = brt_mod
+    T, E, d, n = 1500, 6, 64, 128
+    g = torch.Generator().manual_seed(43)
+    x = torch.randn(T, d, generator=g).to(torch.bfloat16).cuda()
+    score = torch.randn(T, E, generator=g).cuda()
+    deferring = ScatterRouter(protocol_type="topk", fabric_type="fused_dispatch",
+                              fabric_kwargs={"defer_dispatch": True}).cuda()
+    plain = ScatterRouter(protocol_type="topk", fabric_type="fused_dispatch").cuda()
+    want = brt.to_torch_tensor(plain(brt.Annotator([0])(x), score))
+    rows = want.shape[0]
+
+    # the address, read from the plain tensor and from the GridTensor, is the address of filled rows
+    hip = ctypes.CDLL("libamdhip64.so")
+    hip.hipMemcpy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int]
+    for through_grid in (False, True):
+        routed = deferring(brt.Annotator([0])(x), score)
+        state = routed.extra_attr_dict["brt_deferred_0"]
+        assert state.pending
+        address = routed.data_ptr() if through_grid else brt.to_torch_tensor(routed).data_ptr()
+        assert not state.pending
+        torch.cuda.synchronize()
+        host = torch.empty(rows, d, dtype=torch.bfloat16)
+        assert hip.hipMemcpy(host.data_ptr(), address, rows * d * 2, 2) == 0  # device to host
+        assert torch.equal(host.view(torch.int16), want.cpu().view(torch.int16))
+
+    # the grouped GEMM: same rows out, whichever way the unfilled buffer reaches it
+    torch.manual_seed(44)
+    branches = nn.ModuleList(nn.Linear(d, n, bias=False) for _ in range(E)).cuda().to(torch.bfloat16)
+    kernel = make_jit_kernel(branches, None, opt_level="homo_fuse")
+    weights = [m.weight for m in branches]
+    table = torch.tensor([w.data_ptr() for w in weights], dtype=torch.int64, device="cuda")
+    loads = brt.to_torch_tensor(plain(brt.Annotator([0])(x), score), retrieve_attr=True)[2][-1]
+    reference_out = torch.zeros(T, n, dtype=torch.bfloat16, device="cuda")
+    grouped_linear(want, reference_out[:rows], table, None, loads, d, n)
+    for how in ("plain", "grid", "grouped_linear"):
+        routed = deferring(brt.Annotator([0])(x), score)
+        state = routed.extra_attr_dict["brt_deferred_0"]
+        out = torch.zeros(T, n, dtype=torch.bfloat16, device="cuda")
+        if how == "plain":
+            kernel(shared_inputs=[brt.to_torch_tensor(routed), out], standalone_inputs=weights,
+                   capacities=routed.load_stack[-1])
+            assert state.pending  # gathered from the cells: the dispatch never ran
+        elif how == "grid":
+            kernel(shared_inputs=[routed, out], standalone_inputs=weights, capacities=routed.load_stack[-1])
+            assert state.pending
+        else:
+            grouped_linear(routed, out, table, None, routed.load_stack[-1], d, n)
+            assert not state.pending  # the plain operator reads the buffer: filled first
+        assert torch.equal(out[:rows], reference_out[:rows]), how
+
+
 def test_switch_top1_sums_a_cell_that_is_on_two_paths(brt_mod):
     """switch_top1 takes the caller's mask as it is: without one_hot=True a row with two ones goes
     to both paths and the combine adds the two rows (fused path, as the reference does)."""

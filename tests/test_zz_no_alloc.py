@@ -31,9 +31,13 @@ def _both(mask, caps, capacity_padding, is_tag_index):
                 None if d_caps is None else d_caps.data_ptr(), 0 if caps is None else len(caps),
                 int(capacity_padding), 0, int(is_tag_index)]
         if static:
-            before = torch.cuda.memory_allocated()
+            # free device memory as the runtime reports it (hipMemGetInfo): a hipMalloc inside the
+            # library would show here, which the counters of torch's caching allocator would not
+            torch.cuda.synchronize()
+            free_before = torch.cuda.mem_get_info()[0]
             _lib.check(lib.brt_hip_generate_indices_and_loads_static(*head, st))
-            assert torch.cuda.memory_allocated() == before
+            torch.cuda.synchronize()
+            assert torch.cuda.mem_get_info()[0] == free_before
         else:
             _lib.check(lib.brt_hip_generate_indices_and_loads(*head, ws.data_ptr(), ws.numel(), st))
         torch.cuda.synchronize()
@@ -53,6 +57,58 @@ def test_static_scratch_form_equals_workspace_form_on_two_calls_in_a_row(is_tag_
         (i0, l0, c0), (i1, l1, c1) = _both(mask, caps, pad, is_tag_index)
         assert np.array_equal(c0, mask.sum(0))
         assert np.array_equal(i0, i1) and np.array_equal(l0, l1) and np.array_equal(c0, c1)
+
+
+@pytest.mark.parametrize("is_tag_index", [False, True])
+def test_static_scratch_form_in_a_captured_graph_on_another_stream(is_tag_index):
+    """What the entry point is for: after one call outside (which looks the buffer's address up),
+    a call is captured into a HIP graph on a stream of its own and replayed for new masks, with
+    eager work and synchronisations between the replays; every replay equals the workspace form."""
+    rng = np.random.default_rng(12)
+    T, E, caps = 4096, 32, [200]
+    lib = _lib.lib()
+    d_mask = torch.zeros((T, E), dtype=torch.int32, device="cuda")
+    d_caps = torch.tensor(caps, dtype=torch.int32, device="cuda")
+    idx = torch.empty((T, E), dtype=torch.int32, device="cuda")
+    loads = torch.empty((E,), dtype=torch.int32, device="cuda")
+    counts = torch.empty((E,), dtype=torch.int32, device="cuda")
+    ws = torch.empty((max(lib.brt_hip_scan_workspace_bytes(T, E), 4),), dtype=torch.uint8, device="cuda")
+
+    def call_static(stream_ptr):
+        _lib.check(lib.brt_hip_generate_indices_and_loads_static(
+            d_mask.data_ptr(), idx.data_ptr(), loads.data_ptr(), counts.data_ptr(), T, E,
+            d_caps.data_ptr(), len(caps), 0, 0, int(is_tag_index), stream_ptr))
+
+    call_static(torch.cuda.current_stream().cuda_stream)  # set-up happens outside the capture
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            call_static(side.cuda_stream)
+    for replay in range(3):
+        mask = np.zeros((T, E), dtype=np.int32)
+        mask[np.arange(T), rng.integers(0, E, T)] = 1
+        d_mask.copy_(torch.from_numpy(mask).cuda())
+        idx.fill_(-3)
+        loads.fill_(-3)
+        torch.cuda.synchronize()
+        free_before = torch.cuda.mem_get_info()[0]
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.cuda.mem_get_info()[0] == free_before
+        got = (idx.cpu().numpy().copy(), loads.cpu().numpy().copy(), counts.cpu().numpy().copy())
+        want_idx = torch.full((T, E), -7, dtype=torch.int32, device="cuda")
+        want_loads = torch.empty((E,), dtype=torch.int32, device="cuda")
+        want_counts = torch.empty((E,), dtype=torch.int32, device="cuda")
+        _lib.check(lib.brt_hip_generate_indices_and_loads(
+            d_mask.data_ptr(), want_idx.data_ptr(), want_loads.data_ptr(), want_counts.data_ptr(), T, E,
+            d_caps.data_ptr(), len(caps), 0, 0, int(is_tag_index), ws.data_ptr(), ws.numel(),
+            torch.cuda.current_stream().cuda_stream))
+        torch.cuda.synchronize()
+        assert np.array_equal(got[0], want_idx.cpu().numpy()), replay
+        assert np.array_equal(got[1], want_loads.cpu().numpy()) and np.array_equal(got[2], want_counts.cpu().numpy())
+        assert np.array_equal(got[2], mask.sum(0))
 
 
 def test_static_scratch_form_refuses_what_does_not_fit():
