@@ -50,7 +50,7 @@ RING_BYTES = 768 << 20      # what one kernel touches going once round a ring of
 T, D, E, DFF = 8192, 768, 64, 3072
 CAPACITY = int(1.25 * (T // E))  # 160
 SEED = 2
-PHASES = ("all", "step", "instep", "cold", "warm", "ffn", "configs", "extras", "api")
+PHASES = ("all", "step", "instep", "cold", "warm", "ffn", "configs", "extras", "api", "ceilings")
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "switch_moe_8k_pmc_traffic.md")
 
 
@@ -477,7 +477,11 @@ def check_switch_layer(gpu, layer):
 
 def phase_step(gpu, layer, steps, warmup):
     """The K steps are one HIP graph (as the layers of a model would be), launched once, so the
-    time per step holds no launch gaps between graphs; the warm-up replays a one-step graph."""
+    time per step holds no launch gaps between graphs.  The warm-up replays a one-step graph
+    `warmup` times and then keeps going until at least 50 ms of steps have run (clocks, caches and
+    the first-use costs of a fresh box settle); the K-step graph is then timed 11 times, each replay
+    between its own pair of events, and the median is the step time (BASELINE.md asks for a median
+    of repeats).  Smallest and largest replay are reported beside it."""
     torch = gpu.torch
     g_step = gpu.capture(lambda: layer.step(0))
     g_steps = gpu.capture(lambda: layer.step(0), steps)
@@ -485,14 +489,68 @@ def phase_step(gpu, layer, steps, warmup):
         for _ in range(warmup):
             g_step.replay()
     gpu.stream.synchronize()
+    warm_ms, warm_steps = 0.0, warmup
+    while warm_ms < 50.0:
+        warm_ms += gpu.timed(g_step, 50)
+        warm_steps += 50
+    gpu.timed(g_steps, 1)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    ms_total = gpu.timed(g_steps, 1)
+    replays = sorted(gpu.timed(g_steps, 1) for _ in range(11))
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3
     per_graph_launch_us = gpu.timed(g_step, steps) / steps * 1e3  # one graph launch per step
-    return {"ms_per_step": ms_total / steps, "wall_ms": wall_ms,
+    return {"ms_per_step": replays[len(replays) // 2] / steps, "ms_per_step_min": replays[0] / steps,
+            "ms_per_step_max": replays[-1] / steps, "timed_replays": len(replays),
+            "warmup_steps_run": warm_steps, "wall_ms": wall_ms,
             "layer_us_one_graph_launch_per_step": per_graph_launch_us}
+
+
+def phase_ceilings(gpu):
+    """What the machine gives the same run, for the figures of this line to be read against: the
+    library's dense bf16 GEMM (torch.matmul, a hipBLASLt kernel) on the two shapes of the
+    compute-bound probe, on the same N(0,1) x N(0,0.02) data, and the runtime's device-to-device
+    copy of 512 MiB (read + written: 1 GiB of traffic).  Eager launches between two events on the
+    benchmark's stream, 10 per interval, best of 3 intervals; none of it goes into a graph."""
+    torch, dev = gpu.torch, gpu.dev
+    g = torch.Generator(device="cuda").manual_seed(6)
+    out = {"note": "eager launches of library routines, 10 per event interval, best of 3; not part of any step"}
+
+    def eager_us(fn, per=10):
+        best = None
+        with torch.cuda.stream(gpu.stream):
+            for _ in range(3):
+                fn()
+            for _ in range(3):
+                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a.record(gpu.stream)
+                for _ in range(per):
+                    fn()
+                b.record(gpu.stream)
+                gpu.stream.synchronize()
+                t = a.elapsed_time(b) * 1e3 / per
+                best = t if best is None or t < best else best
+        return best
+
+    rows = 32768
+    for name, (k, n) in (("matmul_32768x2048x8192", (2048, 8192)), ("matmul_32768x8192x2048", (8192, 2048))):
+        x = torch.randn(rows, k, generator=g, device=dev).to(torch.bfloat16)
+        w = (torch.randn(n, k, generator=g, device=dev) * 0.02).to(torch.bfloat16)
+        y = torch.empty(rows, n, dtype=torch.bfloat16, device=dev)
+        t_us = eager_us(lambda: torch.matmul(x, w.t(), out=y))
+        flop = 2.0 * rows * k * n
+        out[name] = {"us": round(t_us, 1), "TFLOPs": round(flop / t_us / 1e6, 1),
+                     "mfma_frac": round(flop / t_us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4)}
+        del x, w, y
+    src = torch.empty(512 << 20, dtype=torch.uint8, device=dev).random_(0, 255)
+    dst = torch.empty_like(src)
+    t_us = eager_us(lambda: dst.copy_(src))
+    out["device_copy_512MiB"] = {"us": round(t_us, 1), "bytes": 2 * src.numel(),
+                                 "GBps": round(2 * src.numel() / t_us / 1e3, 1),
+                                 "hbm_frac": round(2 * src.numel() / t_us / 1e3 / HBM_PEAK_GBPS, 4)}
+    del src, dst
+    torch.cuda.empty_cache()
+    return out
 
 
 ROUTING_KERNELS = ("indexgen", "dispatch", "combine", "combine_gather")
@@ -623,9 +681,24 @@ def routing_config(gpu, name, c):
         t_us = gpu.launch_us([(lambda b=b: fn(b)) for b in ring], launches=240)
         res[kname] = {"us": round(t_us, 2), "bytes": nbytes, "GBps": round(nbytes / t_us / 1e3, 1),
                       "hbm_frac": round(nbytes / t_us / 1e3 / HBM_PEAK_GBPS, 4)}
+    # the yardstick: the runtime's own device-to-device copy of as many row bytes as dispatch
+    # moves (R rows read, P rows written), timed on the same ring in the same way
+    copy_rows = min(R, P, Tn)
+    copy_bytes = 2 * copy_rows * d * es
+    t_copy = gpu.launch_us([(lambda b=b: b["y"][:copy_rows].copy_(b["x"][:copy_rows])) for b in ring], launches=240)
+    res["plain_copy"] = {"us": round(t_copy, 2), "bytes": copy_bytes, "GBps": round(copy_bytes / t_copy / 1e3, 1),
+                         "hbm_frac": round(copy_bytes / t_copy / 1e3 / HBM_PEAK_GBPS, 4),
+                         "is": "torch's copy_ of the same number of rows, same ring, same graph timing"}
+    for kname in ("dispatch", "combine"):
+        res[kname]["vs_plain_copy"] = round(res[kname]["GBps"] / res["plain_copy"]["GBps"], 3)
     dc_bytes = entries["dispatch"][1] + entries["combine"][1]
     dc_us = res["dispatch"]["us"] + res["combine"]["us"]
     res["dispatch_combine_GBps"] = round(dc_bytes / dc_us / 1e3, 1)
+    res["dispatch_combine_hbm_frac"] = round(dc_bytes / dc_us / 1e3 / HBM_PEAK_GBPS, 4)
+    for b in ring:
+        b.clear()
+    del ring
+    torch.cuda.empty_cache()
     return res
 
 
@@ -1248,6 +1321,10 @@ def main():
     if want("step"):
         st = phase_step(gpu, layer, args.steps, args.warmup)
         result["ms_per_step"] = round(st["ms_per_step"], 5)
+        result["ms_per_step_min"] = round(st["ms_per_step_min"], 5)
+        result["ms_per_step_max"] = round(st["ms_per_step_max"], 5)
+        result["ms_per_step_is"] = (f"median of {st['timed_replays']} replays of the graph of {args.steps} steps, each "
+                                    f"between its own events, after {st['warmup_steps_run']} warm-up steps (at least 50 ms)")
         result["layer_us"] = round(st["ms_per_step"] * 1e3, 2)
         result["layer_us_one_graph_launch_per_step"] = round(st["layer_us_one_graph_launch_per_step"], 2)
         result["wall_ms_timed_region"] = round(st["wall_ms"], 3)
@@ -1281,6 +1358,16 @@ def main():
             "never-touched ones of the ring (dispatch_combine_cold_ring_GBps)")
         result["in_step"] = {"step_us": round(whole_us, 2), "sum_of_kernel_costs_us": round(sum(us.values()), 2),
                              "kernels": per_kernel(us)}
+        if result.get("layer_us") is not None:
+            # the headline step against the sum of what its kernels cost: two readings of one thing
+            off = abs(result["layer_us"] - sum(us.values())) / sum(us.values())
+            result["in_step"]["layer_us_vs_sum_of_kernel_costs"] = round(off, 4)
+            result["in_step"]["consistent_within_8_percent"] = off <= 0.08
+            if off > 0.08:
+                print(f"bench.py: WARNING: the timed step ({result['layer_us']} us) and the sum of its kernels' costs "
+                      f"({sum(us.values()):.2f} us) differ by {off:.1%}: one of the two measurements is off "
+                      "(the costs are differences of two graphs each, and hold the boundary to the next kernel "
+                      "five times where the step holds it four times)", file=sys.stderr)
         if after_producer["dispatch_us"] > 0:
             result["in_step_input_just_written"] = {
                 "dispatch_us": round(after_producer["dispatch_us"], 3),
@@ -1357,8 +1444,18 @@ def main():
                 nbytes[name] / trace_us[name] / 1e3 / HBM_PEAK_GBPS, 4)
             result["roofline_ffn"]["kernel_trace_taken_at_commit"] = trace_commit
 
+    if want("ceilings"):
+        result["ceilings"] = phase_ceilings(gpu)
+
     if want("configs"):
         result["configs"] = phase_configs(gpu, args.config)
+        probe = result["configs"].get("compute_bound_probe_8e_x_4096_rows_2048_8192")
+        if probe and "ceilings" in result:
+            # the grouped GEMM over 8 experts of 4096 rows against the library's dense GEMM of the same size
+            probe["gemm1_gelu"]["vs_library_matmul"] = round(
+                probe["gemm1_gelu"]["TFLOPs"] / result["ceilings"]["matmul_32768x2048x8192"]["TFLOPs"], 3)
+            probe["gemm2"]["vs_library_matmul"] = round(
+                probe["gemm2"]["TFLOPs"] / result["ceilings"]["matmul_32768x8192x2048"]["TFLOPs"], 3)
 
     if want("extras"):
         result.update(phase_extras(gpu, layer, args.steps))

@@ -56,6 +56,9 @@ ROUTING_CONFIGS = {
     "cfg1_top1_1024x512_f32_16e": dict(T=1024, E=16, d=512, dtype="f32", k=1, cap=64, seed=1),
     "cfg3_top2_16384x1024_bf16_32e": dict(T=16384, E=32, d=1024, dtype="bf16", k=2, cap=2048, seed=3),
     "cfg4_swin_100352x96_f16_8e": dict(T=100352, E=8, d=96, dtype="f16", k=1, cap=12544, seed=4),
+    # the benchmark layer's route shape at eight times the cells: 100 MB of rows per launch, so the
+    # launch ramp of a 25 MB kernel is no longer what is measured (capacity 1.25 x the mean load)
+    "hbm_resident_top1_65536x768_bf16_64e": dict(T=65536, E=64, d=768, dtype="bf16", k=1, cap=1280, seed=7),
 }
 
 
