@@ -1204,7 +1204,13 @@ def phase_api(gpu, layer, steps):
     annotator = brt.Annotator([0])
     out = {}
     results = {}
-    for name, kwargs in (("static_rows", {"static_rows": True}), ("defer_dispatch", {"defer_dispatch": True})):
+    forms = (("static_rows", {"static_rows": True}, False),
+             ("defer_dispatch", {"defer_dispatch": True}, False),
+             # the route carried as path ids from the gate to the combine (no [cells, paths] mask or seat matrix)
+             ("compact_route_defer_dispatch", {"compact_route": True, "defer_dispatch": True}, False),
+             # ... and the last kernel given the residual: it stores its rows straight to their cells
+             ("compact_route_defer_dispatch_folded_combine", {"compact_route": True, "defer_dispatch": True}, True))
+    for name, kwargs, fold in forms:
         scatter = ScatterRouter(protocol_type="topk", fabric_type="fused_dispatch",
                                 fabric_kwargs={"supported_capacities": [CAPACITY], **kwargs}).to(gpu.dev)
         gather = GatherRouter(fabric_type="fused_combine").to(gpu.dev)
@@ -1216,7 +1222,8 @@ def phase_api(gpu, layer, steps):
             h = torch.empty((states.shape[0], DFF), device=states.device, dtype=states.dtype)
             fused_wi(shared_inputs=[states, h], standalone_inputs=wi_w, capacities=loads[-1])
             y = torch.empty((states.shape[0], D), device=states.device, dtype=states.dtype)
-            fused_wo(shared_inputs=[h, y], standalone_inputs=wo_w, capacities=loads[-1])
+            fused_wo(shared_inputs=[h, y], standalone_inputs=wo_w, capacities=loads[-1],
+                     **({"residual": residual} if fold else {}))
             gather(brt.to_grid_tensor(y, tags, loads, extra), residual)
 
         before = gpu._lib.call_count()
@@ -1234,10 +1241,13 @@ def phase_api(gpu, layer, steps):
         eager_us = (time.perf_counter() - t_wall) * 1e6 / eager_steps
         out[name] = {"layer_us": round(us, 2), "library_calls_per_layer": calls,
                      "layer_us_eager_wall_clock": round(eager_us, 1)}
-    if not torch.equal(results["static_rows"], results["defer_dispatch"]):
-        raise SystemExit("bench: the deferred dispatch changed the layer's result")
-    out["note"] = ("library calls per layer include the gate's top-k mask kernel; index generation is "
-                   "two kernels in one call.  Both forms give bit-identical results (checked here)")
+    for name, _, _ in forms[1:]:
+        if not torch.equal(results["static_rows"], results[name]):
+            raise SystemExit(f"bench: the {name} form changed the layer's result")
+    out["note"] = ("library calls per layer include the gate kernel (top-k mask, or path ids for the compact "
+                   "route); index generation and route_by_path are two kernels in one call.  All forms give "
+                   "bit-identical results (checked here); only the last one changes the caller's code (the "
+                   "residual is handed to the expert's last kernel)")
     return out
 
 

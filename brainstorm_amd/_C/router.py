@@ -21,6 +21,9 @@ __all__ = [
     "topk_hot_mask",
     "throttle_hotmask",
     "Route",
+    "CompactRoute",
+    "remember_route",
+    "route_of_loads",
     "generate_route",
     "generate_indices_and_loads",
     "convert_index_format",
@@ -118,6 +121,55 @@ class Route:
         """True when the pair is the one this route was generated with, unmodified since."""
         return (route_indices is self.indices and loads is self.loads
                 and self._versions == (route_indices._version, loads._version))
+
+
+class CompactRoute:
+    """A route kept as ``k`` path ids per cell from the gate to the combine (an extension; the
+    reference carries a ``[cells, paths]`` hot mask and seat matrix, python/brt/router/fabric/fused.py:32-75):
+    what ``gate_topk`` chose and ``route_by_path`` laid out.  ``seat_rows[t, j]`` is the 1-based
+    row of the path-major layout that entry ``(t, j)`` owns (0: dropped), ``row_entries[r]`` the
+    1-based entry ``t * k + j + 1`` behind row ``r`` (0: padding).  ``indices`` is the dense seat
+    matrix the reference would have produced, generated on first read."""
+
+    __slots__ = ("path_ids", "weights", "loads", "counts", "seat_rows", "row_entries", "k", "cells",
+                 "paths", "single_path", "indices", "combined_into", "__weakref__")
+
+    def __init__(self, path_ids, weights, loads, counts, seat_rows, row_entries, paths, indices):
+        self.path_ids, self.weights = path_ids, weights
+        self.loads, self.counts, self.seat_rows, self.row_entries = loads, counts, seat_rows, row_entries
+        self.cells, self.k = path_ids.shape
+        self.paths = int(paths)
+        self.single_path = self.k == 1
+        self.indices = indices       # lazily filled [cells, paths] seat indices (what the stacks carry)
+        self.combined_into = None    # the tensor an expert kernel already stored the combined rows to
+
+    def owns(self, route_indices, loads) -> bool:
+        return route_indices is self.indices and loads is self.loads
+
+
+# Routes by the identity of their loads tensor: an expert kernel receives the loads as its
+# capacities and finds the route of its rows through them.  Both sides are held weakly: the route
+# lives as long as the routed GridTensor carries it, and the entry goes when the loads tensor does.
+_routes_by_loads = {}
+
+
+def remember_route(loads: torch.Tensor, route) -> None:
+    import weakref
+
+    key = id(loads)
+
+    def forget(_ref, key=key, table=_routes_by_loads):
+        table.pop(key, None)
+
+    _routes_by_loads[key] = (weakref.ref(loads, forget), weakref.ref(route))
+
+
+def route_of_loads(loads: torch.Tensor):
+    """The route that was generated with this very loads tensor, or None."""
+    entry = _routes_by_loads.get(id(loads))
+    if entry is not None and entry[0]() is loads:
+        return entry[1]()
+    return None
 
 
 _fallback_logged = set()
@@ -826,7 +878,8 @@ def route_by_path(
 
 
 def dispatch_by_rows(in_data: torch.Tensor, row_entries: torch.Tensor, k: int,
-                     weights: Optional[torch.Tensor] = None) -> torch.Tensor:
+                     weights: Optional[torch.Tensor] = None,
+                     out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``out[r] = in_data[(row_entries[r]-1) // k]`` (times ``weights.view(-1)[row_entries[r]-1]``,
     rounded once), zero rows where ``row_entries[r] == 0``: what ``dispatch_with_indices_and_loads``
     (router.cc:131-273) writes for the same route, every row written by the kernel."""
@@ -844,7 +897,11 @@ def dispatch_by_rows(in_data: torch.Tensor, row_entries: torch.Tensor, k: int,
             raise RuntimeError("weights must be fp32 [cells, k]")
         weights = weights.contiguous()
     with _device_guard(in_data.device):
-        out = torch.empty((P,) + tuple(in_data.shape[1:]), dtype=in_data.dtype, device=in_data.device)
+        if out is None:
+            out = torch.empty((P,) + tuple(in_data.shape[1:]), dtype=in_data.dtype, device=in_data.device)
+        elif (out.dtype != in_data.dtype or not out.is_contiguous() or out.numel() != P * cell
+              or out.device != in_data.device):
+            raise RuntimeError("out must be a contiguous [rows, *cell_shape] tensor of the input's type")
         _lib.check(_lib.lib().brt_hip_dispatch_by_rows(
             _ptr(in_data), _ptr(out), _ptr(weights), _ptr(row_entries.contiguous()), P, T, int(k),
             cell, _DT[in_data.dtype], _stream()))

@@ -20,6 +20,7 @@ import torch
 import torch.nn as nn
 
 from brainstorm_amd import _lib
+from brainstorm_amd._C import router as c_router
 from brainstorm_amd.runtime import deferred
 
 __all__ = ["make_jit_kernel", "grouped_linear", "GroupedLinearKernel"]
@@ -217,7 +218,15 @@ class GroupedLinearKernel:
         self._biases_bf16 = _Bf16Weights()
 
     def __call__(self, shared_inputs: List[torch.Tensor], standalone_inputs: Sequence[torch.Tensor],
-                 capacities: Union[torch.Tensor, Sequence[int]] = ()):
+                 capacities: Union[torch.Tensor, Sequence[int]] = (), *,
+                 residual: Optional[torch.Tensor] = None):
+        """``residual`` (an extension, for the last kernel of an expert on a route with one path
+        per cell): the cell-major tensor the gather router will be given as its residual.  The
+        rows are then stored straight to their cells in it -- the combine folded into the store --
+        and ``out`` is NOT written; the fused combine fabric recognises the tensor and launches
+        nothing.  It needs the route of the rows, which is found through ``capacities`` (the loads
+        tensor of the routed GridTensor, as it came off the load stack) and must stem from a fused
+        dispatch fabric built with ``compact_route=True``."""
         x, out = shared_inputs
         standalone_inputs = list(standalone_inputs)
         step = 2 if self.has_bias else 1
@@ -230,7 +239,10 @@ class GroupedLinearKernel:
         weights = self._branch_operands(weights, capacities.numel(), self._weights_bf16, "weights")
         if biases:
             biases = self._branch_operands(biases, capacities.numel(), self._biases_bf16, "biases")
+        route_loads = capacities
         loads = capacities.to(device=out.device, dtype=torch.int32)
+        if residual is not None:
+            return self._store_to_cells(x, weights, biases, loads, route_loads, residual)
         state = deferred.pending_of(x)  # a DeferredRows, or the routed GridTensor itself
         if state is not None and not self._can_gather(state, out):
             state.materialize()
@@ -239,6 +251,12 @@ class GroupedLinearKernel:
             # the rows of a deferred dispatch: read from the cells through the route's tag indices
             route = state.route
             cells = state.cells if state.cells.dtype == torch.bfloat16 else _to_bf16(state.cells)
+            if isinstance(route, c_router.CompactRoute):  # rows named by the row-entry vector
+                grouped_linear(cells, out, self._weights.get(weights),
+                               self._biases.get(biases) if biases else None, loads, self.in_features,
+                               self.out_features, self.activation, row_entries=route.row_entries,
+                               entries_per_cell=route.k, gather=True, rows=out.shape[0])
+                return
             row_tags = torch.empty((out.shape[0],), dtype=torch.int32, device=out.device)
             grouped_linear(cells, out, self._weights.get(weights),
                            self._biases.get(biases) if biases else None, loads, self.in_features,
@@ -252,6 +270,28 @@ class GroupedLinearKernel:
             x, out, self._weights.get(weights),
             self._biases.get(biases) if biases else None,
             loads, self.in_features, self.out_features, self.activation)
+
+    def _store_to_cells(self, x, weights, biases, loads, route_loads, residual):
+        """The GEMM whose rows go straight to their cells in ``residual`` (combine folded in)."""
+        route = c_router.route_of_loads(route_loads) if torch.is_tensor(route_loads) else None
+        if not isinstance(route, c_router.CompactRoute) or route.k != 1:
+            raise RuntimeError("residual= needs the loads tensor of a route with one path per cell from a "
+                               "fused dispatch fabric built with compact_route=True")
+        if (residual.dtype != torch.bfloat16 or not residual.is_contiguous() or residual.dim() != 2
+                or residual.shape != (route.cells, self.out_features) or not residual.is_cuda):
+            raise RuntimeError("the residual must be a contiguous bf16 [cells, out_features] device tensor")
+        pending = deferred.pending_of(x)
+        if pending is not None:
+            pending.materialize()
+        if x.dtype == torch.float32:
+            x = _to_bf16(x)
+        if x.shape[0] != route.row_entries.numel():
+            raise RuntimeError("the input does not have the rows of the dispatched layout")
+        grouped_linear(x, residual, self._weights.get(weights),
+                       self._biases.get(biases) if biases else None, loads, self.in_features,
+                       self.out_features, self.activation, row_entries=route.row_entries,
+                       entries_per_cell=1, scatter=True, rows=x.shape[0])
+        route.combined_into = residual
 
     def _branch_operands(self, tensors, used: int, cache: _Bf16Weights, what: str):
         dtypes = {t.dtype for t in tensors[:used]}

@@ -13,6 +13,8 @@ import torch
 import torch.nn as nn
 
 from brainstorm_amd._C import router as c_router
+from brainstorm_amd.router.protocol._impl import CompactHotMask
+from brainstorm_amd.runtime.deferred import lazy_tensor
 from brainstorm_amd.router.utils import make_kwargs
 from brainstorm_amd.runtime import Registry
 from brainstorm_amd.runtime.deferred import DeferredState
@@ -357,15 +359,23 @@ class FusedDispatchFabric(DispatchFabric):
     grouped GEMM of ``brt.jit`` gathers its rows from the cells directly; the stacks then carry
     tag-format indices.  Any other use of the tensor runs the dispatch first.
     ``static_rows=True`` (an extension) keeps the dispatch but sizes its output the same way, so
-    that nothing is read back to the host."""
+    that nothing is read back to the host.
+    ``compact_route=True`` (an extension) takes the decision of a ``topk`` protocol as ``k`` path
+    ids per cell (the ScatterRouter tells the protocol) and lays the route out from them
+    (``route_by_path``): no ``[cells, paths]`` mask or seat matrix is written or read; the matrix on
+    the tag stack is generated only if something reads it.  The rows are sized as with
+    ``static_rows`` and moved by ``dispatch_by_rows``, or with ``defer_dispatch`` gathered by the
+    expert's first grouped GEMM; top-k routes with k > 1 are taken as well."""
 
     def __init__(self, flow_num: int, route_logic="1d", transform=False, **kwargs):
         kwargs["index_format"] = "seat_index"
         defer = bool(kwargs.pop("defer_dispatch", False))
         static_rows = bool(kwargs.pop("static_rows", False))
+        compact = bool(kwargs.pop("compact_route", False))
         super().__init__(flow_num, route_logic=route_logic, transform=transform, **kwargs)
         self.defer_dispatch = defer
         self.static_rows = static_rows
+        self.compact_route = compact
         self._host_caps_key = ()   # the capacity buffer the host copy below was read from
         self._host_caps_list = None
 
@@ -403,19 +413,70 @@ class FusedDispatchFabric(DispatchFabric):
             return None
         return self._row_bound(flow_data.shape[0], route_indices.shape[1])
 
-    def _row_bound(self, cells: int, paths: int) -> int:
-        """Rows the path-major layout of a single-path route can need, known without reading the loads back."""
+    def _row_bound(self, cells: int, paths: int, k: int = 1) -> int:
+        """Rows the path-major layout of a route with ``k`` paths per cell can need, known without
+        reading the loads back."""
         caps = self._host_caps
         if caps is None:
-            return cells
+            return cells * k
         if self.path_wise_padding:
             return sum(caps)
         if self.capacity_padding:
             return paths * max(caps)
-        return min(cells, paths * max(caps))
+        return min(cells * k, paths * max(caps))
+
+    def _takes_compact(self, in_flows, runtime_capacities) -> bool:
+        if len(in_flows) != 1 or runtime_capacities is not None or self.transforms[0]:
+            return False
+        flow = in_flows[0]
+        return (self.route_logics[0] == "1d" and flow.dim() >= 2 and flow.shape[0] > 0 and flow.is_cuda
+                and flow.dtype in (torch.float32, torch.float16, torch.bfloat16))
+
+    def _forward_compact(self, in_flows, decision, score):
+        """The route from path ids: ``route_by_path`` lays it out (loads by the capacity rules of
+        location.cu:222-256, the row of every entry, the entry of every row), the rows are moved by
+        ``dispatch_by_rows`` or left to the expert's first GEMM."""
+        data, tags, load_stack, extra = to_torch_tensor(in_flows[0], retrieve_attr=True)
+        assert tags[-1] is None  # fused dispatch starts from freshly annotated cells
+        data = data.contiguous()
+        cells, paths = decision.shape
+        k = decision.path_ids.shape[1]
+        mpl = int(self.max_path_load) if self.max_path_padding else 0
+        rows = paths * mpl if mpl else self._row_bound(cells, paths, k)
+        caps = self.supported_capacities
+        loads, counts, seat_rows, row_entries = c_router.route_by_path(
+            decision.path_ids, paths, caps, self.capacity_padding, self.path_wise_padding, mpl, rows)
+
+        def fill_dense(buffer):  # the seat matrix of the reference, for whoever reads the tag stack
+            indices, _ = c_router.generate_indices_and_loads(
+                decision.dense(), caps, self.capacity_padding, self.path_wise_padding, False)
+            buffer.copy_(indices)
+
+        indices = lazy_tensor(torch.empty((cells, paths), dtype=torch.int32, device=data.device), fill_dense)
+        route = c_router.CompactRoute(decision.path_ids, decision.scores, loads, counts, seat_rows,
+                                      row_entries, paths, indices)
+        c_router.remember_route(loads, route)
+        self._route = route
+        self.capture_flow_stats(in_flows, indices, loads)  # (reads the dense matrix when capturing)
+        level = len(tags) - 1
+        extra = dict(extra or {})
+        extra[_route_key(level)] = route
+        flat = data.view(cells, -1)
+        if (self.defer_dispatch and flat.shape[1] % 8 == 0
+                and data.dtype in (torch.bfloat16, torch.float32) and data.dim() == 2):
+            routed = torch.empty((rows, flat.shape[1]), dtype=data.dtype, device=data.device)
+            extra[_deferred_key(level)] = DeferredState(flat, route, routed, _deferred_key(level))
+        else:
+            routed = c_router.dispatch_by_rows(data, row_entries, k)
+        out = init_grid_tensor(routed, tags[:-1] + [indices], load_stack[:-1] + [loads], extra)
+        return (out if self.flow_num == 1 else [out]), score
 
     def forward(self, in_flow, hot_mask, runtime_capacities=None, score=None):
         in_flows = [in_flow] if self.flow_num == 1 else in_flow
+        if isinstance(hot_mask, CompactHotMask):
+            if self._takes_compact(in_flows, runtime_capacities):
+                return self._forward_compact(in_flows, hot_mask, score)
+            hot_mask = hot_mask.dense()  # a shape this path does not take: the mask, as the reference
         if not self._in_one_step(in_flows, runtime_capacities, hot_mask):
             return super().forward(in_flow, hot_mask, runtime_capacities, score)
         # static rows, one flow, single-path route: index generation moves the rows itself
@@ -483,7 +544,9 @@ class FusedCombineFabric(CombineFabric):
             route = extra.pop(_route_key(len(tags)), None)
             state = extra.pop(_deferred_key(len(tags)), None)
             gates = score if self.transform else None
-            if route is not None and route.is_tag_index and route.owns(route_indices, loads):
+            if isinstance(route, c_router.CompactRoute) and route.owns(route_indices, loads):
+                out = self._combine_compact(data, route, state, gates, residual)
+            elif route is not None and route.is_tag_index and route.owns(route_indices, loads):
                 out = self._combine_deferred(data, route, state, gates, residual)
             else:
                 (out,) = c_router.combine_with_indices_and_loads(
@@ -491,6 +554,29 @@ class FusedCombineFabric(CombineFabric):
                     max_path_padding=self.max_path_padding, ever_padded=self.ever_padded, route=route)
             out_flows.append(init_grid_tensor(out, tags, load_stack, extra))
         return out_flows
+
+    def _combine_compact(self, data, route, state, gates, residual):
+        """Combine of a route carried as path ids: the tag-driven scatter for one path per cell (the
+        row-entry vector then is the row-tag vector), else the gather over the k entries of a cell
+        in ascending path order; both bit-identical to ``combine_with_indices_and_loads`` on the
+        dense route."""
+        if route.combined_into is not None:
+            # an expert kernel that was handed the residual has stored the combined rows already
+            if residual is None or residual.data_ptr() != route.combined_into.data_ptr():
+                raise RuntimeError("the expert kernel combined into another tensor than this residual")
+            return residual
+        if data.size(0) != route.row_entries.numel():
+            raise RuntimeError("the expert output does not have the rows of the dispatched layout")
+        if residual is not None and not residual.is_contiguous():
+            raise RuntimeError("the residual must be contiguous (it is updated in place)")
+        if route.k == 1 and gates is None:
+            if residual is not None:
+                return c_router.combine_by_row_tags(data, route.row_entries, route.cells, residual)
+            return c_router.combine_by_row_tags(data, route.row_entries, route.cells)
+        weights = None
+        if gates is not None:  # the weight of every entry: the score of its cell on its path
+            weights = torch.gather(gates, 1, route.path_ids.long()).to(torch.float32)
+        return c_router.combine_by_rows(data, route.path_ids, route.seat_rows, weights, residual)
 
     def _combine_deferred(self, data, route, state, gates, residual):
         """Combine of a route whose dispatch was deferred: tag-format indices; the row tags were

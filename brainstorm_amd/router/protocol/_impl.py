@@ -59,6 +59,41 @@ def make_protocol(protocol_type: str, kwargs: Dict[str, Any]) -> ProtocolBase:
     return protocol_cls(**make_kwargs(kwargs))
 
 
+class CompactHotMask:
+    """The decision of a top-k protocol kept as ``k`` path ids per cell instead of a
+    ``[cells, paths]`` int32 mask (an extension: python/brt/router/protocol/topk.py:26-31 builds the
+    mask with ``topk`` + ``zeros_like`` + ``scatter_``).  Only a fused dispatch fabric built with
+    ``compact_route=True`` receives one; it reads ``path_ids`` and never needs the mask.
+    ``dense()`` is the mask the reference would have built."""
+
+    dtype = torch.int32
+
+    def __init__(self, path_ids: torch.Tensor, scores: torch.Tensor, path_num: int):
+        self.path_ids = path_ids   # [cells, k] int32, in the order of torch.topk
+        self.scores = scores       # [cells, k] fp32: the scores of the chosen paths
+        self.shape = torch.Size((path_ids.shape[0], int(path_num)))
+        self.device = path_ids.device
+        self.is_cuda = path_ids.is_cuda
+        self._dense = None
+
+    def size(self, dim=None):
+        return self.shape if dim is None else self.shape[dim]
+
+    def dim(self):
+        return 2
+
+    def numel(self):
+        return self.shape[0] * self.shape[1]
+
+    def dense(self) -> torch.Tensor:
+        if self._dense is None:
+            self._dense = torch.zeros(tuple(self.shape), dtype=torch.int32, device=self.device).scatter_(
+                1, self.path_ids.long(), 1)
+            if getattr(self, "_brt_single_path", False):
+                self._dense._brt_single_path = True
+        return self._dense
+
+
 def _one_hot_int32(indices: torch.Tensor, like: torch.Tensor) -> torch.Tensor:
     """int32 mask with ones at ``indices`` (``[cells, k]``) along dim 1."""
     return torch.zeros(like.shape, dtype=torch.int32, device=like.device).scatter_(1, indices, 1)
@@ -82,8 +117,15 @@ class TopKProtocol(ProtocolBase):
         super().__init__()
         self.top_k = top_k
         self.single_path = top_k == 1
+        #: set by a ScatterRouter whose fabric takes the compact route: the decision is handed
+        #: over as path ids (one kernel, k words per cell) instead of the [cells, paths] mask
+        self.compact = False
 
     def make_route_decision(self, score):
+        if (self.compact and score.is_cuda and score.dim() == 2 and 0 < self.top_k <= score.shape[1] <= 1024
+                and score.dtype in (torch.float32, torch.float16, torch.bfloat16)):
+            path_ids, scores = c_router.gate_topk(score, self.top_k)
+            return CompactHotMask(path_ids, scores, score.shape[1])
         return _topk_hot_mask(score, self.top_k)
 
 

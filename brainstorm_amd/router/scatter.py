@@ -52,6 +52,10 @@ class ScatterRouter(RouterBase):
                 defaults = {"flow_num": 2, "route_logic": ["1d", "2d"], "transform": [False, False]}
         self.fabric_kwargs = _merged(defaults, fabric_kwargs)
         self.fabric = make_fabric(fabric_type, self.fabric_kwargs)
+        # a fused fabric built with compact_route=True takes the decision of a top-k protocol as
+        # path ids (an extension; off unless asked for)
+        if getattr(self.fabric, "compact_route", False) and hasattr(self.protocol, "compact"):
+            self.protocol.compact = True
 
     def _route(self, in_flows, score: torch.Tensor):
         hot_mask = self.protocol(score)

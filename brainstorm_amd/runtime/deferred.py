@@ -17,7 +17,8 @@ from typing import Any, Optional
 
 import torch
 
-__all__ = ["DeferredState", "DeferredRows", "pending_state", "pending_of", "wrap_if_pending", "settle"]
+__all__ = ["DeferredState", "DeferredRows", "LazyFill", "lazy_tensor", "pending_state", "pending_of",
+           "wrap_if_pending", "settle"]
 
 
 class DeferredState:
@@ -44,8 +45,39 @@ class DeferredState:
         if self.done:
             return
         from brainstorm_amd._C import router as c_router
-        c_router.dispatch_rows_of_route(self.cells, self.route, self.buffer)
+        if isinstance(self.route, c_router.CompactRoute):
+            c_router.dispatch_by_rows(self.cells, self.route.row_entries, self.route.k, out=self.buffer)
+        else:
+            c_router.dispatch_rows_of_route(self.cells, self.route, self.buffer)
         self.done = True
+
+
+class LazyFill:
+    """A buffer whose contents are produced by ``fill(buffer)`` the first time anything reads it
+    (the dense seat-index matrix of a route that is carried in compact form)."""
+
+    __slots__ = ("buffer", "fill", "done")
+
+    def __init__(self, buffer: torch.Tensor, fill):
+        self.buffer, self.fill, self.done = buffer, fill, False
+
+    @property
+    def pending(self) -> bool:
+        return not self.done
+
+    def materialize(self) -> None:
+        if not self.done:
+            self.fill(self.buffer)
+            self.done = True
+
+
+def lazy_tensor(buffer: torch.Tensor, fill) -> torch.Tensor:
+    """``buffer`` as a tensor that runs ``fill(buffer)`` before its first read; shape, dtype and
+    device can be read without filling it."""
+    with torch._C.DisableTorchFunctionSubclass():
+        wrapped = buffer.as_subclass(DeferredRows)
+    wrapped.__dict__["_brt_state"] = LazyFill(buffer, fill)
+    return wrapped
 
 
 # reads that say nothing about the rows: allowed on an unfilled buffer
@@ -103,7 +135,7 @@ def state_of(t: torch.Tensor) -> Optional[DeferredState]:
     """The pending state behind ``t`` when it is an unfilled deferred buffer, else None."""
     if isinstance(t, DeferredRows):
         state = t.__dict__.get("_brt_state")
-        if state is not None and state.pending:
+        if isinstance(state, DeferredState) and state.pending:
             return state
     return None
 

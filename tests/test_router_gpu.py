@@ -588,6 +588,128 @@ def test_deferred_rows_fill_themselves_when_anything_else_reads_them(brt_mod):
     assert torch.allclose(total, want.float().sum())
 
 
+def _moe_layer(brt_mod, E, d, dff, top_k, dtype, seed, fabric_kwargs, weighted=False, fold_combine=False):
+    """ScatterRouter(topk, fused_dispatch) -> two homo-fused kernels -> GatherRouter(fused_combine),
+    the caller code of benchmark/switch_moe/switch_expert.py:62-99; ``fold_combine`` hands the last
+    kernel the residual (the one caller-visible extension)."""
+    brt, _, ScatterRouter, GatherRouter = brt_mod
+    from brt.jit import make_jit_kernel
+
+    torch.manual_seed(seed)
+    wi = nn.ModuleList(nn.Linear(d, dff, bias=False) for _ in range(E)).cuda().to(dtype)
+    wo = nn.ModuleList(nn.Linear(dff, d, bias=False) for _ in range(E)).cuda().to(dtype)
+    scatter = ScatterRouter(protocol_type="topk", protocol_kwargs={"top_k": top_k},
+                            fabric_type="fused_dispatch", fabric_kwargs=dict(fabric_kwargs)).cuda()
+    gather = GatherRouter(fabric_type="fused_combine", fabric_kwargs={"transform": weighted}).cuda()
+    fused_wi = make_jit_kernel(wi, None, opt_level="homo_fuse", activation="gelu")
+    fused_wo = make_jit_kernel(wo, None, opt_level="homo_fuse")
+    annotator = brt.Annotator([0])
+
+    def layer(hidden, score):
+        routed = scatter(annotator(hidden), score)
+        states, tags, loads, extra = brt.to_torch_tensor(routed, retrieve_attr=True)
+        wi_out = torch.empty((states.shape[0], dff), device=states.device, dtype=states.dtype)
+        fused_wi(shared_inputs=[states, wi_out], standalone_inputs=[m.weight for m in wi], capacities=loads[-1])
+        wo_out = torch.empty((states.shape[0], d), device=states.device, dtype=states.dtype)
+        fused_wo(shared_inputs=[wi_out, wo_out], standalone_inputs=[m.weight for m in wo], capacities=loads[-1],
+                 **({"residual": hidden} if fold_combine else {}))
+        routed_out = brt.to_grid_tensor(wo_out, tags, loads, extra)
+        combined = gather(routed_out, hidden, score) if weighted else gather(routed_out, hidden)
+        return brt.to_torch_tensor(combined)
+
+    return layer
+
+
+@pytest.mark.parametrize("caps", [None, {"supported_capacities": [160]},
+                                  {"supported_capacities": [160], "capacity_padding": True}])
+def test_compact_route_through_the_router_objects_top1(brt_mod, caps):
+    """compact_route=True: the topk protocol hands the fabric path ids, route_by_path lays the route
+    out, the first GEMM gathers its rows by the row-entry vector, the tag-driven combine (or, given
+    the residual, the last GEMM itself) puts them back.  Same caller code as the dense layer, the
+    same bits, five calls into the library (four with the folded combine) against six."""
+    from brainstorm_amd import _lib
+
+    T, E, d, dff = 2048, 16, 256, 512
+    g = torch.Generator().manual_seed(51)
+    hidden = torch.randn(T, d, generator=g).to(torch.bfloat16).cuda()
+    score = torch.randn(T, E, generator=g).cuda()
+    caps = caps or {}
+    variants = [
+        (dict(caps), False, 6),                                                   # mask, indexgen, dispatch, 2 GEMMs, combine
+        (dict(caps, compact_route=True), False, 6),                               # gate, route, dispatch_by_rows, 2 GEMMs, combine
+        (dict(caps, compact_route=True, defer_dispatch=True), False, 5),          # gate, route, gathering GEMM, GEMM, combine
+        (dict(caps, compact_route=True, defer_dispatch=True), True, 4),           # gate, route, gathering GEMM, scattering GEMM
+    ]
+    results = []
+    for fabric_kwargs, fold, want_calls in variants:
+        layer = _moe_layer(brt_mod, E, d, dff, 1, torch.bfloat16, 52, fabric_kwargs, fold_combine=fold)
+        layer(hidden.clone(), score)  # pointer tables, workspaces
+        residual = hidden.clone()
+        before = _lib.call_count()
+        results.append(layer(residual, score))
+        assert _lib.call_count() - before == want_calls, (fabric_kwargs, fold, _lib.call_count() - before)
+        assert results[-1].data_ptr() == residual.data_ptr()  # combined in place, as the reference does
+    for other in results[1:]:
+        assert torch.equal(results[0], other)
+    assert not torch.equal(results[0], hidden)
+
+
+@pytest.mark.parametrize("weighted", [False, True])
+def test_compact_route_through_the_router_objects_top2(brt_mod, weighted):
+    """The same for two paths per cell (with and without gate-weighted combine): path ids to
+    route_by_path, rows by dispatch_by_rows or gathered by the first GEMM, combine over the two
+    entries of a cell in ascending path order -- bit-identical to the dense layer."""
+    from brainstorm_amd import _lib
+
+    brt = brt_mod[0]
+    T, E, d, dff = 1536, 8, 128, 256
+    g = torch.Generator().manual_seed(53)
+    hidden = torch.randn(T, d, generator=g).to(torch.bfloat16).cuda()
+    score = torch.softmax(torch.randn(T, E, generator=g), dim=1).cuda()
+    caps = {"supported_capacities": [450]}  # some cells lose a path, a few both
+    results = []
+    for fabric_kwargs, want_calls in ((dict(caps), 6), (dict(caps, compact_route=True), 6),
+                                      (dict(caps, compact_route=True, defer_dispatch=True), 5)):
+        layer = _moe_layer(brt_mod, E, d, dff, 2, torch.bfloat16, 54, fabric_kwargs, weighted=weighted)
+        layer(hidden.clone(), score)
+        before = _lib.call_count()
+        results.append(layer(hidden.clone(), score))
+        assert _lib.call_count() - before == want_calls, (fabric_kwargs, _lib.call_count() - before)
+    for other in results[1:]:
+        assert torch.equal(results[0], other)
+
+
+def test_compact_route_keeps_the_reference_format_for_whoever_reads_it(brt_mod):
+    """The tag stack of a compact route carries the dense seat matrix of the reference, generated
+    only when something reads it; the loads are the reference's; a fabric that does not take the
+    compact form gets the mask."""
+    brt, c_router, ScatterRouter, GatherRouter = brt_mod
+    T, E, d = 999, 7, 64
+    g = torch.Generator().manual_seed(55)
+    x = torch.randn(T, d, generator=g).to(torch.bfloat16).cuda()
+    score = torch.randn(T, E, generator=g).cuda()
+    for top_k in (1, 2):
+        kw = {"supported_capacities": [200], "capacity_padding": top_k == 2}
+        dense = ScatterRouter(protocol_type="topk", protocol_kwargs={"top_k": top_k},
+                              fabric_type="fused_dispatch", fabric_kwargs=dict(kw)).cuda()
+        compact = ScatterRouter(protocol_type="topk", protocol_kwargs={"top_k": top_k},
+                                fabric_type="fused_dispatch", fabric_kwargs=dict(kw, compact_route=True)).cuda()
+        want = dense(brt.Annotator([0])(x), score)
+        got = compact(brt.Annotator([0])(x), score)
+        state = got.tag_stack[-1].__dict__["_brt_state"]
+        assert state.pending                                     # nobody has read the matrix yet
+        assert torch.equal(got.load_stack[-1], want.load_stack[-1])
+        rows = int(want.load_stack[-1].sum())
+        assert torch.equal(brt.to_torch_tensor(got)[:rows], brt.to_torch_tensor(want)[:rows])
+        assert not bool(brt.to_torch_tensor(got)[rows:].any())   # rows behind the loads are zero
+        assert state.pending
+        assert torch.equal(got.tag_stack[-1] + 0, want.tag_stack[-1])  # a read: the reference's seat indices
+        assert not state.pending
+    # a plain dispatch fabric never sees a compact decision
+    plain = ScatterRouter(protocol_type="topk", fabric_type="dispatch").cuda()
+    assert plain.protocol.compact is False
+
+
 def test_foreign_consumers_of_a_deferred_buffer_see_dispatched_rows(brt_mod):
     """What a deferred buffer hands to code that knows nothing of it: a consumer of its address (a
     ctypes / C-extension kernel taking ``data_ptr()``) finds the rows dispatched, and the grouped
