@@ -29,6 +29,7 @@ constexpr int kWholeWaves = 8;    // a small route: one workgroup of 8 wavefront
 constexpr int kWholeChunks = 32;  // ... up to this many chunks of 64 entries
 constexpr int kSplitWaves = 4;    // larger routes: workgroups of 4 wavefronts, two launches
 constexpr int kSplitGroups = 32;  // ... in at most this many workgroups
+constexpr int kSoloEntries = 65536;  // routes up to this many entries: one launch, every workgroup counts the whole route
 constexpr int kSplitWavesLarge = 16;  // ... of 16 wavefronts for routes beyond 32768 entries
 constexpr int kBatch = 4;        // chunks of 64 entries a wavefront keeps in flight
 constexpr int kMaxK = 8;         // paths per cell in combine_by_rows
@@ -148,18 +149,26 @@ __device__ __forceinline__ void sum_rows(Ptr cnt, int rows, int mine, int E, int
 // its contiguous range of entries.  The counters travel through `ws`: [groups][E] sums per
 // workgroup, then [units][E] per unit, so that a unit finds its first seats with one round of
 // loads: the sums of the workgroups before its own plus the units before it in its own.
-enum RouteMode { kWhole = 0, kCount = 1, kEmit = 2 };
+// kSolo: middle-sized routes in ONE launch over several workgroups.  A workgroup needs two things from
+// the entries it does not own: how many of each path lie before its range (its first seats) and how
+// many there are in all (loads and first rows).  Neither depends on the order of those entries, so
+// every workgroup takes them from a histogram of the whole id vector (at most 256 KB, read from
+// the L2) built with LDS atomics, one add per entry, instead of waiting for a counting kernel; only
+// its own range is ranked with the ballots.  No workgroup waits for another.
+enum RouteMode { kWhole = 0, kCount = 1, kEmit = 2, kSolo = 3 };
 
 template <int MODE, int WAVES>
 __global__ __launch_bounds__(WAVES * kWave) void route_kernel(RouteArgs a) {
   extern __shared__ int lds[];
   const int E = a.E;
+  constexpr bool kOwnCounts = MODE == kWhole || MODE == kSolo;  // counters of its wavefronts stay in LDS
   int* s_cnt = lds;                                         // [WAVES][E] counters
-  int* s_seat = MODE == kWhole ? lds + WAVES * E : lds;     // [WAVES][E] running seats of pass 2
+  int* s_seat = kOwnCounts ? lds + WAVES * E : lds;         // [WAVES][E] running seats of pass 2
   int* s_load = s_seat + WAVES * E;                         // [E]
   int* s_start = s_load + E;                                // [E]
   int* s_kept = s_start + E;                                // [E] rows a path really fills
-  int* s_caps = s_kept + E;                                 // [caps_in_lds]
+  int* s_hist = s_kept + E;                                 // kSolo: [2][E] entries before this workgroup's range / from it on
+  int* s_caps = s_hist + (MODE == kSolo ? 2 * E : 0);       // [caps_in_lds]
   const int lane = threadIdx.x & (kWave - 1), w = threadIdx.x >> 6;
   const int unit = blockIdx.x * WAVES + w;
   constexpr int kStep = kWave * kBatch;
@@ -169,7 +178,7 @@ __global__ __launch_bounds__(WAVES * kWave) void route_kernel(RouteArgs a) {
   // the first batch of ids is fetched once, ahead of everything else, and serves both passes
   const Batch first = load_batch(a.ids, lo, hi, lane);
   // per-unit counters lie behind the workgroup sums (two-launch form only)
-  int* unit_rows = MODE == kWhole ? nullptr : a.ws + static_cast<size_t>(gridDim.x) * E;
+  int* unit_rows = kOwnCounts ? nullptr : a.ws + static_cast<size_t>(gridDim.x) * E;
   // kEmit: the counters of the first 64 paths are fetched in the same round trip as the ids and
   // the capacities
   int before0 = 0, total0 = 0;
@@ -182,8 +191,43 @@ __global__ __launch_bounds__(WAVES * kWave) void route_kernel(RouteArgs a) {
     for (int i = threadIdx.x; i < a.caps_in_lds; i += WAVES * kWave) s_caps[i] = a.caps[i];
   if (MODE != kEmit)
     for (int i = threadIdx.x; i < WAVES * E; i += WAVES * kWave) s_cnt[i] = 0;
+  if (MODE == kSolo)
+    for (int i = threadIdx.x; i < 2 * E; i += WAVES * kWave) s_hist[i] = 0;
   __syncthreads();
   const int* caps = a.caps_in_lds != 0 ? s_caps : a.caps;
+
+  if constexpr (MODE == kSolo) {
+    // histogram of every entry, split at the start of this workgroup's range: 16 ids per lane in
+    // flight, one LDS add each (the adds of a wavefront to one counter are serialised by the
+    // LDS, which for ids spread over the paths is a handful of passes)
+    const int own_lo = static_cast<int>(min(static_cast<long>(a.n), static_cast<long>(blockIdx.x) * WAVES * a.per_wave));
+    constexpr int kFlight = 8, kThreads = WAVES * kWave;
+    typedef int i32x4 __attribute__((ext_vector_type(4)));
+    const bool quads = (reinterpret_cast<uintptr_t>(a.ids) & 15) == 0;  // 16-byte loads of 4 ids
+    const int nq = quads ? a.n >> 2 : 0;
+    const i32x4* ids4 = reinterpret_cast<const i32x4*>(a.ids);
+#pragma unroll 1
+    for (int base = 0; base < nq; base += kFlight * kThreads) {
+      i32x4 id[kFlight];
+#pragma unroll
+      for (int q = 0; q < kFlight; ++q) id[q] = ids4[min(base + q * kThreads + static_cast<int>(threadIdx.x), nq - 1)];
+#pragma unroll
+      for (int q = 0; q < kFlight; ++q) {
+        const int i4 = base + q * kThreads + threadIdx.x;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          const int i = i4 * 4 + c, e = id[q][c];
+          if (i4 < nq && e >= 0 && e < E)
+            __hip_atomic_fetch_add(&s_hist[(i < own_lo ? 0 : E) + e], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        }
+      }
+    }
+    for (int i = nq * 4 + threadIdx.x; i < a.n; i += kThreads) {  // the tail, or everything behind a misaligned pointer
+      const int e = a.ids[i];
+      if (e >= 0 && e < E)
+        __hip_atomic_fetch_add(&s_hist[(i < own_lo ? 0 : E) + e], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+  }
 
   if (MODE != kEmit) {
     int* mine = s_cnt + w * E;
@@ -206,7 +250,7 @@ __global__ __launch_bounds__(WAVES * kWave) void route_kernel(RouteArgs a) {
     }
     return;
   }
-  if (MODE == kWhole) __syncthreads();
+  if (kOwnCounts) __syncthreads();
 
   // first seat of this unit in every path; the first wavefront also finishes the columns
   int* mine = s_seat + w * E;
@@ -217,6 +261,11 @@ __global__ __launch_bounds__(WAVES * kWave) void route_kernel(RouteArgs a) {
     int before = 0, total = 0;
     if constexpr (MODE == kWhole) {
       sum_rows<WAVES>(s_cnt, WAVES, w, E, e, &before, &total);
+    } else if constexpr (MODE == kSolo) {
+      int own = 0;
+      sum_rows<WAVES>(s_cnt, WAVES, w, E, e, &before, &own);
+      before += e < E ? s_hist[e] : 0;
+      total = e < E ? s_hist[e] + s_hist[E + e] : 0;
     } else if (e0 == 0) {
       before = before0;
       total = total0;
@@ -509,6 +558,14 @@ extern "C" int brt_hip_route_by_path(const int32_t* path_ids, int T, int k, int 
     a.per_wave = (chunks + kWholeWaves - 1) / kWholeWaves * kWave;
     const size_t lds_bytes = (static_cast<size_t>(2 * kWholeWaves + 3) * E + a.caps_in_lds) * sizeof(int);
     hipLaunchKernelGGL((route_kernel<kWhole, kWholeWaves>), dim3(1), dim3(kWholeWaves * kWave), lds_bytes, st, a);
+    return check_launch("route_kernel");
+  }
+  if (n <= kSoloEntries) {
+    // one launch: workgroups of 4 wavefronts, each wavefront a whole number of chunks of its own
+    const int groups = std::min(kSplitGroups, (chunks + kSplitWaves - 1) / kSplitWaves);
+    a.per_wave = (chunks + groups * kSplitWaves - 1) / (groups * kSplitWaves) * kWave;
+    const size_t lds_bytes = (static_cast<size_t>(2 * kSplitWaves + 5) * E + a.caps_in_lds) * sizeof(int);
+    hipLaunchKernelGGL((route_kernel<kSolo, kSplitWaves>), dim3(groups), dim3(kSplitWaves * kWave), lds_bytes, st, a);
     return check_launch("route_kernel");
   }
   int waves;
