@@ -478,7 +478,13 @@ __global__ __launch_bounds__(kBlock) void combine_by_rows_kernel(RowsArgs a) {
           }
         }
       }
-      if (live && (use[0] || !a.is_residual)) {
+      if constexpr (IN_DT != OUT_DT && LS == 6) {
+        // 16-bit rows into an fp32 result, a whole wavefront per row: whole-line streaming stores
+        const bool row_ok = live && (use[0] || !a.is_residual);  // the same for the whole wavefront
+#pragma unroll
+        for (int u = 0; u < UPR; ++u)
+          store_widened_spread(dst + to * OUT_BYTES, off0 + u * LPR, cpr, row_ok, acc[u]);
+      } else if (live && (use[0] || !a.is_residual)) {
 #pragma unroll
         for (int u = 0; u < UPR; ++u) {
           const int off = off0 + u * LPR + glane;

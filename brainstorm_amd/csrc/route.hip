@@ -895,23 +895,66 @@ __global__ __launch_bounds__(kBlock) void combine_lean_kernel(CombineArgs a) {
   const U* __restrict__ src = static_cast<const U*>(a.src);
   char* __restrict__ dst = static_cast<char*>(a.dst);
 
-  int v_next = (sub < nt && e < E) ? idx0[sub * E + e] : 0;
+  // Index words are fetched two steps ahead and the first row of a step one step ahead: while
+  // the rows of step s are added up and stored, the row loads of step s + 1 (which need its index
+  // words) are already in flight, so a wavefront keeps two rows' worth of loads outstanding
+  // instead of waiting out the index round trip and the row round trip of every cell in turn.
+  auto index_word = [&](int step) {
+    const int r = step * rps + sub;
+    return (step < n_steps && r < nt && e < E) ? idx0[r * E + e] : 0;
+  };
+  int v_ahead1 = index_word(1);
+  const int v_first = index_word(0);
   const SmallTables tab = small_tables(a.loads, E, a.mpl, ep_shift, lane);
 
-  for (int step = 0; step < n_steps; ++step) {
-    const int v = v_next;
+  struct Step {
+    unsigned long long m;  // (cell, path) pairs of the step that own a row
+    int src_row;
+    float gate;
+    int tokens;
+  };
+  auto prepare = [&](int step, int v) {
+    Step s;
     const int row = step * rps + sub;
-    {
-      const int nrow = row + rps;
-      v_next = (step + 1 < n_steps && nrow < nt && e < E) ? idx0[nrow * E + e] : 0;
-    }
-    const int src_row = tab.start_e + v - 1;
-    const bool ok = row < nt && e < E && v >= 1 && v <= tab.load_e && src_row < a.P;
-    float gate = 1.0f;
+    s.src_row = tab.start_e + v - 1;
+    const bool ok = row < nt && e < E && v >= 1 && v <= tab.load_e && s.src_row < a.P;
+    s.gate = 1.0f;
     if (ok && a.gates != nullptr)
-      gate = load_gate(a.gates, a.gate_dtype, static_cast<size_t>(t0 + row) * E + e);
-    const unsigned long long m = __ballot(ok);
-    const int tokens = min(rps, nt - step * rps);
+      s.gate = load_gate(a.gates, a.gate_dtype, static_cast<size_t>(t0 + row) * E + e);
+    s.m = __ballot(ok);
+    s.tokens = min(rps, nt - step * rps);
+    return s;
+  };
+  // the units of the first row of this lane group's first cell of the step (lowest path)
+  auto first_row = [&](const Step& s, U (&val)[UPR]) {
+    const int i = gidx;
+    const unsigned long long mine = i < s.tokens ? (s.m >> (i * ep)) & seg0 : 0ull;
+    const bool has = mine != 0;
+    const int b = i * ep + __builtin_ctzll(mine | (1ull << 63));
+    const int sr = __builtin_amdgcn_ds_bpermute(b << 2, s.src_row);
+#pragma unroll
+    for (int u = 0; u < UPR; ++u) {
+      const int off = u * LPR + glane;
+      if (has && off < cpr) val[u] = src[static_cast<size_t>(sr) * cpr + off];
+    }
+  };
+
+  Step cur = prepare(0, v_first);
+  U val_cur[UPR];
+  first_row(cur, val_cur);
+  for (int step = 0; step < n_steps; ++step) {
+    Step nxt = cur;
+    U val_nxt[UPR];
+    if (step + 1 < n_steps) {
+      const int v = v_ahead1;
+      v_ahead1 = index_word(step + 2);
+      nxt = prepare(step + 1, v);
+      first_row(nxt, val_nxt);
+    }
+    const unsigned long long m = cur.m;
+    const int src_row = cur.src_row;
+    const float gate = cur.gate;
+    const int tokens = cur.tokens;
     for (int tb = 0; tb < tokens; tb += GROUPS) {
       const int i = tb + gidx;
       const unsigned long long mine = i < tokens ? (m >> (i * ep)) & seg0 : 0ull;
@@ -923,6 +966,7 @@ __global__ __launch_bounds__(kBlock) void combine_lean_kernel(CombineArgs a) {
 #pragma unroll
           for (int q = 0; q < NE; ++q) acc[u][q] = 0.0f;
         unsigned long long rem = mine;
+        bool fetched = tb == 0 && off0 == 0;  // the first row of the first cell is in val_cur already
         while (__ballot(rem != 0) != 0) {  // ascending path order: lowest set bit first
           const bool has = rem != 0;
           const int b = i * ep + __builtin_ctzll(rem | (1ull << 63));
@@ -930,11 +974,17 @@ __global__ __launch_bounds__(kBlock) void combine_lean_kernel(CombineArgs a) {
           const int sr = __builtin_amdgcn_ds_bpermute(b << 2, src_row);
           const float g = __int_as_float(__builtin_amdgcn_ds_bpermute(b << 2, __float_as_int(gate)));
           U val[UPR];
+          if (fetched) {
 #pragma unroll
-          for (int u = 0; u < UPR; ++u) {
-            const int off = off0 + u * LPR + glane;
-            if (has && off < cpr) val[u] = src[static_cast<size_t>(sr) * cpr + off];
+            for (int u = 0; u < UPR; ++u) val[u] = val_cur[u];
+          } else {
+#pragma unroll
+            for (int u = 0; u < UPR; ++u) {
+              const int off = off0 + u * LPR + glane;
+              if (has && off < cpr) val[u] = src[static_cast<size_t>(sr) * cpr + off];
+            }
           }
+          fetched = false;
 #pragma unroll
           for (int u = 0; u < UPR; ++u) {
             const int off = off0 + u * LPR + glane;
@@ -947,12 +997,18 @@ __global__ __launch_bounds__(kBlock) void combine_lean_kernel(CombineArgs a) {
             }
           }
         }
-        if (i < tokens && (mine != 0 || !a.is_residual)) {
+        if constexpr (IN_DT != OUT_DT && LS == 6) {
+          // 16-bit rows into an fp32 result, a whole wavefront per row: whole-line streaming stores
+          const bool row_ok = i < tokens && (mine != 0 || !a.is_residual);  // the same for the whole wavefront
+#pragma unroll
+          for (int u = 0; u < UPR; ++u)
+            store_widened_spread(dst + to * OUT_BYTES, off0 + u * LPR, cpr, row_ok, acc[u]);
+        } else if (i < tokens && (mine != 0 || !a.is_residual)) {
 #pragma unroll
           for (int u = 0; u < UPR; ++u) {
             const int off = off0 + u * LPR + glane;
-            // streamed only when a wavefront's store covers whole lines: a widening store writes two
-            // 16-byte halves per lane, which have to meet in the L2 first, and so do rows of up to 128 bytes
+            // streamed only when a wavefront's store covers whole lines: rows of up to 128 bytes are
+            // scattered partial lines, which are faster merged in the L2
             if (off < cpr) {
               pack_store<OUT_DT, NE, IN_DT == OUT_DT && LS >= 4>(dst + (to + off) * OUT_BYTES, acc[u]);
             }
@@ -960,6 +1016,9 @@ __global__ __launch_bounds__(kBlock) void combine_lean_kernel(CombineArgs a) {
         }
       }
     }
+    cur = nxt;
+#pragma unroll
+    for (int u = 0; u < UPR; ++u) val_cur[u] = val_nxt[u];
   }
 }
 

@@ -106,6 +106,32 @@ __device__ __forceinline__ void pack_store(void* p, const float (&x)[N]) {
   }
 }
 
+// Widening store of a whole wavefront's row segment (16-bit input units, fp32 output): lane l
+// holds the 8 fp32 values of unit `first_unit + l`, i.e. 32 contiguous bytes of the output row, so
+// two plain 16-byte stores per lane would each write every other 16 bytes of the segment (halves
+// that have to meet in the L2).  The values are spread over the lanes first -- lane l takes half
+// l & 1 of lane l / 2 (first store) and of lane 32 + l / 2 (second store) -- and each store then
+// covers 1 KB of whole lines, streamed.  All 64 lanes must call it; `row_ok` (the row is written at
+// all) must be the same for the whole wavefront, units at or past `units_in_row` are not written.
+__device__ __forceinline__ void store_widened_spread(char* row_base, int first_unit, int units_in_row,
+                                                     bool row_ok, const float (&x)[8]) {
+  const int lane = lane_id();
+#pragma unroll
+  for (int half = 0; half < 2; ++half) {
+    const int from = 32 * half + (lane >> 1);
+    f32x4 o;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int lo = __builtin_amdgcn_ds_bpermute(from << 2, __float_as_int(x[q]));
+      const int hi = __builtin_amdgcn_ds_bpermute(from << 2, __float_as_int(x[4 + q]));
+      o[q] = __int_as_float((lane & 1) ? hi : lo);
+    }
+    const int unit = first_unit + from;
+    if (row_ok && unit < units_in_row)
+      store_unit<true>(reinterpret_cast<f32x4*>(row_base + static_cast<size_t>(unit) * 32 + (lane & 1) * 16), o);
+  }
+}
+
 template <int BYTES>
 __device__ __forceinline__ typename Unit<BYTES>::type zero_unit() {
   typename Unit<BYTES>::type z = {};
