@@ -195,7 +195,7 @@ def summarize_counters(pairs, counters, commit):
         with open(path) as f:
             for row in csv.DictReader(f):
                 name = row["Kernel_Name"]
-                if "grouped_gemm_kernel" not in name:
+                if "grouped_gemm" not in name:
                     continue
                 per.setdefault(name, {}).setdefault(row["Counter_Name"], []).append(float(row["Counter_Value"]))
         names = sorted({c for v in per.values() for c in v})
@@ -224,12 +224,20 @@ def summarize_trace(pairs, commit):
     """Markdown summary of kernel-trace statistics, one table per phase of the benchmark."""
     import csv
 
-    print("# rocprofv3 kernel trace: launch durations, Switch-MoE layer hot path (bench.py default workload)\n")
-    print("One run per phase, so that launches inside the layer step (inputs as the layer leaves them) and "
-          "back-to-back launches on one buffer set (inputs in the last-level cache) are separate rows:\n")
+    def run_args(label):
+        return f"--only {label}" if label in PHASES else f"--only configs --config {label}"
+
+    if all(pair.split("=", 1)[0] in PHASES for pair in pairs):
+        print("# rocprofv3 kernel trace: launch durations, Switch-MoE layer hot path (bench.py default workload)\n")
+        print("One run per phase, so that launches inside the layer step (inputs as the layer leaves them) and "
+              "back-to-back launches on one buffer set (inputs in the last-level cache) are separate rows:\n")
+    else:
+        print("# rocprofv3 kernel trace: launch durations of the grouped expert GEMM on the other configurations\n")
+        print("One run per configuration of `bench.py --only configs` (a label that is not a phase of the "
+              "benchmark stands for `--config <label>`):\n")
     for pair in pairs:
         label = pair.split("=", 1)[0]
-        print(f"    rocprofv3 --kernel-trace --stats --output-format csv -d <dir> -o s -- python3 bench.py --only {label} --no-cpu-baseline")
+        print(f"    rocprofv3 --kernel-trace --stats --output-format csv -d <dir> -o s -- python3 bench.py {run_args(label)} --no-cpu-baseline")
     print("    python3 bench.py --summarize-trace " + " ".join(p.split("=", 1)[0] + "=<dir>/.../s_kernel_stats.csv" for p in pairs)
           + " --commit <hash>\n")
     for pair in pairs:
