@@ -880,21 +880,35 @@ def phase_instep(gpu, layer, steps):
              ("ffn_gemm2", layer.gemm2), ("combine", layer.combine)]
     rounds = max(50, min(steps, 200))
 
-    def per_step_us(skip):
+    def graph_without(order, skip):
         fns = [(lambda fn=fn: fn(0)) for name, fn in order if name != skip]
-        graph = gpu.capture(fns, rounds)
-        gpu.timed(graph, 1)
-        return min(gpu.timed(graph, 1) for _ in range(5)) * 1e3 / rounds
+        return gpu.capture(fns, rounds)
 
-    whole = per_step_us(None)
-    in_step_us = {name: max(whole - per_step_us(name), 0.0) for name, _ in order}
+    def per_step_us(graphs, repeats=7):
+        """Median time per step of every graph, the graphs replayed in turn (whole, without the
+        first kernel, without the second, ... and round again) so that a drift of the clocks
+        during the measurement falls on all of them alike and cancels in the differences."""
+        for g in graphs.values():
+            gpu.timed(g, 1)
+        runs = {k: [] for k in graphs}
+        for _ in range(repeats):
+            for k, g in graphs.items():
+                runs[k].append(gpu.timed(g, 1) * 1e3 / rounds)
+        return {k: sorted(v)[len(v) // 2] for k, v in runs.items()}
+
+    graphs = {None: graph_without(order, None)}
+    graphs.update({name: graph_without(order, name) for name, _ in order})
+    us = per_step_us(graphs)
+    whole = us[None]
+    in_step_us = {name: max(whole - us[name], 0.0) for name, _ in order}
     # The same difference for dispatch when the cells were written just before the step, as the
     # layer in front of a MoE layer leaves them (here: an elementwise kernel that writes the input buffer).
     x = layer.sets[0]["x"]
     x_src = x.clone()
     order = [("producer", lambda s: gpu.torch.mul(x_src, 1.0, out=x))] + order
-    after_producer = {"step_with_producer_us": per_step_us(None)}
-    after_producer["dispatch_us"] = max(after_producer["step_with_producer_us"] - per_step_us("dispatch"), 0.0)
+    us = per_step_us({None: graph_without(order, None), "dispatch": graph_without(order, "dispatch")})
+    after_producer = {"step_with_producer_us": us[None]}
+    after_producer["dispatch_us"] = max(us[None] - us["dispatch"], 0.0)
     return in_step_us, whole, after_producer
 
 
