@@ -314,6 +314,46 @@ def test_combine_bit_exact(hip, T, E, k, cell, in_dtype, out_dtype, gate_dtype):
     assert np.allclose(got, ref, rtol=tol, atol=tol)
 
 
+@pytest.mark.parametrize("dtype,cell", [("bf16", 768), ("f16", 1024), ("f32", 512), ("bf16", 96)])
+def test_combine_moves_or_sums_rows_of_any_bit_pattern(hip, dtype, cell):
+    """Unweighted gather combine on a route where some cells are on one path, some on two and some on
+    none: a pass whose cells all have at most one row may move the rows instead of summing them, and
+    must still give what the sum gives -- every -0 comes out as +0, denormals and infinities as they
+    are, a cell without a row zero or the residual (NaN patterns are left out: their payload is not
+    part of the bar)."""
+    T, E = 1536, 8
+    rng = np.random.default_rng(cell)
+    mask = np.zeros((T, E), dtype=np.int32)
+    first = rng.integers(0, E, T)
+    mask[np.arange(T), first] = 1
+    twice = np.arange(T) % 193 == 5                     # a few cells on two paths, far apart
+    mask[twice, (first[twice] + 3) % E] = 1
+    mask[np.arange(T) % 7 == 3] = 0                     # cells on no path
+    idx, loads = oracle.generate_indices_and_loads(mask, [int(0.9 * T / E)])  # some overflow is dropped
+    P = int(loads.sum())
+    word = np.uint32 if dtype == "f32" else np.uint16
+    bits = rng.integers(0, 256, (P, cell * np.dtype(word).itemsize), dtype=np.uint8).view(word).copy()
+    sign = word(0x80000000 if dtype == "f32" else 0x8000)
+    bits[rng.random(bits.shape) < 0.05] = sign          # -0
+    bits[rng.random(bits.shape) < 0.02] = 1             # the smallest denormal
+    y = bits.view(np.float32) if dtype == "f32" else bits
+    bits[np.isnan(bits_to_f32(y, dtype))] = 0
+    res = as_dtype_bits(rng.standard_normal((T, cell)), dtype)
+    for r in (None, res):
+        want = oracle.combine(y, idx, loads, out_data=r, in_dtype=dtype, out_dtype=dtype)
+        got = hip.combine(y, idx, loads, None, r, in_dtype=dtype, out_dtype=dtype)
+        assert same_bits(got, want), r is None
+    # the cells on exactly one path hold their row, -0 turned into +0, whatever the oracle says
+    live = (idx >= 1) & (idx <= loads[None, :])
+    single = live.sum(1) == 1
+    start = np.concatenate([[0], np.cumsum(loads)[:-1]])
+    e = live.argmax(1)
+    rows = start[e] + idx[np.arange(T), e] - 1
+    moved = np.ascontiguousarray(hip.combine(y, idx, loads, None, None, in_dtype=dtype, out_dtype=dtype)).view(word)
+    src = bits[rows[single]]
+    assert np.array_equal(moved[single], np.where(src == sign, word(0), src))
+
+
 def test_combine_max_path_padding_and_odd_rows(hip):
     T, E = 300, 4
     mask, logits = topk_mask(T, E, 2, seed=91)
