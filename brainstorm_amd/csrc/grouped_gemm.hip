@@ -736,16 +736,22 @@ int grouped_gemm_impl(const void* x, const void* const* weights, const void* con
     if (act == BRT_ACT_RELU) return launch_f32<BRT_ACT_RELU>(a, as_stream(stream));
     return launch_f32<BRT_ACT_NONE>(a, as_stream(stream));
   }
-  // Kernel choice.  Experts that average more than one row block, and enough 256 x 256 tiles for two
-  // full rounds over the CUs: the ping-pong kernel (grouped_gemm_pingpong.hip), whose tile moves a
-  // third fewer operand bytes per flop.  Measured in one process against the 160-row kernel: 8
-  // experts x 4096 rows 2048 -> 8192 -> 2048 1165 / 993 -> 994 / 831 us, the ragged task-MoE shape
-  // 1585 / 1374 -> 1401 / 1263 us, the top-2 shape's expanding GEMM (912 tiles) 212 -> 174 us; its
-  // contracting GEMM (228 tiles on 256 CUs) 156 -> 177 us, which is why few tiles stay with the
-  // 160-row kernel, like every weight-streaming shape.
-  if (pingpong_gemm_applies(a) && static_cast<long>(P) > static_cast<long>(E) * 160 &&
-      static_cast<long>((P + 255) / 256) * ((N + 255) / 256) >= 2L * device_cus())
-    return launch_pingpong_gemm(a, act, as_stream(stream));
+  // Kernel choice.  Experts that average more than one row block take the ping-pong kernel
+  // (grouped_gemm_pingpong.hip), whose 256 x 256 tile moves a third fewer operand bytes per flop,
+  // when its tiles come in whole rounds over the CUs: at least two rounds, or one round that most
+  // CUs take part in.  In between (one to two tiles per CU) a CU with two tiles sets the time and
+  // the smaller tiles of the 160-row kernel spread better.  The tile count is an estimate: the
+  // loads are on the device; an expert's last row block is taken as half full.  Measured in one
+  // process against the 160-row kernel: 8 experts x 4096 rows 2048 -> 8192 -> 2048 1165 / 993 ->
+  // 962 / 793 us, the ragged task-MoE shape 1585 / 1374 -> 1355 / 1211 us, the top-2 shape's
+  // expanding GEMM (1232 tiles) 212 -> 166 us, 8 x 1824 rows 4096 -> 1024 (256 tiles) 146 -> 99 us;
+  // the top-2 shape's contracting GEMM (308 tiles on 256 CUs) 162 -> 173 us.
+  if (pingpong_gemm_applies(a) && static_cast<long>(P) > static_cast<long>(E) * 160) {
+    const long tiles = (static_cast<long>(P + 255) / 256 + (E + 1) / 2) * ((N + 255) / 256);
+    const long cus = device_cus();
+    if (tiles >= 2 * cus || (4 * tiles >= 3 * cus && tiles <= cus))
+      return launch_pingpong_gemm(a, act, as_stream(stream));
+  }
   // Tile choice.  A wavefront owns 160 x 64 outputs (7 LDS fragment reads feed 10 MFMAs); a
   // workgroup is 2, 3 or 4 of them side by side.  The kernel is bound by how fast a CU can fill
   // its L1 (about 29 KB/us, L2 hits included), so the shape is the one that gives the busiest CU

@@ -515,12 +515,15 @@ def test_experts_with_many_row_blocks_in_patch_order(loads, K, N):
     ([5000, 31, 4000, 129], 192, 4104),                       # N tail (8 columns in the last tile), odd K-step count
     ([100] * 60 + [4000], 320, 3584),                         # many experts of one part-filled row block
     ([70] * 70 + [6000, 3000, 5000], 128, 4096),               # more than 64 experts
+    ([1824] * 8, 256, 1024),                                  # one round: 256 tiles for 256 CUs
+    ([2000, 1700, 300, 1900, 1, 1800, 2047, 1500], 128, 1000),  # one round, ragged, N tail
 ])
 def test_ping_pong_tiles(loads, K, N):
     """Shapes the host sends to the 256 x 256 ping-pong kernel: experts that average more than 160
-    rows and at least two rounds of tiles over the CUs."""
-    P = sum(loads)
-    assert P > len(loads) * 160 and ((P + 255) // 256) * ((N + 255) // 256) >= 512, "not a ping-pong shape"
+    rows, and tiles for at least two rounds over the CUs or for one round that most CUs join."""
+    P, E = sum(loads), len(loads)
+    tiles = ((P + 255) // 256 + (E + 1) // 2) * ((N + 255) // 256)
+    assert P > E * 160 and (tiles >= 512 or 192 <= tiles <= 256), "not a ping-pong shape"
     run(loads, K, N)
     run(loads, K, N, act="gelu", bias=True, seed=1)
     run(loads, K, N, act="relu", bias=True, seed=2, slack=300)
