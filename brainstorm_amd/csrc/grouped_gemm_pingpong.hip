@@ -339,6 +339,16 @@ __global__ __launch_bounds__(kWaves * 64) void grouped_gemm_pingpong_kernel(Gemm
   const int col_w = n0 + wn * kNT * 32;   // first column of this wavefront
   __bf16* const out_w = a.out + (static_cast<size_t>(row0) + wm * kMT * 32) * a.N + col_w;
   constexpr int kChunksPerRow = kNT * 32 / 8;  // 8 chunks of 16 bytes
+  // the bias of this lane's columns, all eight loads in one round trip
+  bf16x4 bv[kNT][4];
+#pragma unroll
+  for (int j = 0; j < kNT; ++j)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int col = col_w + j * 32 + 8 * g + 4 * frag_k;
+      bv[j][g] = bf16x4{};
+      if (bias != nullptr && col < a.N) bv[j][g] = *(global_bf16x4)(bias + col);
+    }
 #pragma unroll
   for (int i = 0; i < kMT; ++i) {
     if (i * 32 >= mine) break;  // wave-uniform
@@ -347,8 +357,7 @@ __global__ __launch_bounds__(kWaves * 64) void grouped_gemm_pingpong_kernel(Gemm
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         const int col = j * 32 + 8 * g + 4 * frag_k;  // inside the wavefront's 64 columns
-        bf16x4 b4 = {};
-        if (bias != nullptr && col_w + col < a.N) b4 = *(global_bf16x4)(bias + col_w + col);
+        const bf16x4 b4 = bv[j][g];
         bf16x4 o;
 #pragma unroll
         for (int q = 0; q < 4; ++q)
