@@ -488,7 +488,7 @@ def phase_step(gpu, layer, steps, warmup):
     time per step holds no launch gaps between graphs.  The warm-up replays a one-step graph
     `warmup` times and then keeps going until at least 50 ms of steps have run (clocks, caches and
     the first-use costs of a fresh box settle); the K-step graph is then timed 11 times, each replay
-    between its own pair of events, and the median is the step time (BASELINE.md asks for a median
+    between its own pair of events, and the median is the step time (the metric is defined as a median
     of repeats).  Smallest and largest replay are reported beside it."""
     torch = gpu.torch
     g_step = gpu.capture(lambda: layer.step(0))
