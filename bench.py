@@ -232,7 +232,7 @@ def summarize_trace(pairs, commit):
         print("One run per phase, so that launches inside the layer step (inputs as the layer leaves them) and "
               "back-to-back launches on one buffer set (inputs in the last-level cache) are separate rows:\n")
     else:
-        print("# rocprofv3 kernel trace: launch durations of the grouped expert GEMM on the other configurations\n")
+        print("# rocprofv3 kernel trace: launch durations on the other configurations\n")
         print("One run per configuration of `bench.py --only configs` (a label that is not a phase of the "
               "benchmark stands for `--config <label>`):\n")
     for pair in pairs:
