@@ -774,19 +774,25 @@ __global__ __launch_bounds__(kBlock, 8) void dispatch_lean_kernel(DispatchArgs a
 // In seat mode the source row of a token is the token itself, so its units are
   // fetched before the index words have even arrived and are reused for every
   // path the token is routed to (a top-k token is read once and stored k times).
-  auto load_units = [&](int i, int tokens, int step, int off0, U (&val)[UPR]) {
+  auto load_units = [&](int i, int tokens, int step, int off0, bool wanted, U (&val)[UPR]) {
     const size_t from = static_cast<size_t>(r0 + step * rps + i) * cpr;
 #pragma unroll
     for (int u = 0; u < UPR; ++u) {
       const int off = off0 + u * LPR + glane;
-      if (i < tokens && off < cpr) val[u] = src[from + off];
+      if (wanted && i < tokens && off < cpr) val[u] = src[from + off];
     }
   };
 
   for (int step = 0; step < n_steps; ++step) {
     const int tokens = min(rps, nr - step * rps);
     U val[UPR];
-    load_units(gidx, tokens, step, 0, val);
+    // The rows of the first cells of a step are requested before anything is known about them;
+    // the other cells of the step (and the later units of long rows) only if a path kept them:
+    // a cell dropped by the capacities is then not read at all.  (Holding back the first request
+    // of a step as well, until its index words -- requested a step earlier -- say that a path
+    // kept the cell, takes the top-2 route with 56 % of its entries dropped from 15.1 to 14.3 us,
+    // and costs the benchmark layer's dispatch, which drops nothing, half a microsecond.)
+    load_units(gidx, tokens, step, 0, true, val);
     const int v = v_next;
     const int row = step * rps + sub;
     {
@@ -795,11 +801,11 @@ __global__ __launch_bounds__(kBlock, 8) void dispatch_lean_kernel(DispatchArgs a
     }
     const int dst_row = tab.start_e + v - 1;
     const bool ok = row < nr && e < E && v >= 1 && v <= tab.load_e && dst_row < a.P;
+    const unsigned long long m = __ballot(ok);
     float gate = 1.0f;
     if constexpr (DT >= 0) {
       if (ok) gate = load_gate(a.gates, DT, static_cast<size_t>(r0 + row) * E + e);
     }
-    const unsigned long long m = __ballot(ok);
     if (a.new_tags != nullptr && ok) {  // the lane that holds (token, path) tags the row
       const int tok = static_cast<int>(r0) + row;
       a.new_tags[dst_row] = a.old_tags != nullptr ? a.old_tags[tok] : tok + 1;
@@ -808,7 +814,7 @@ __global__ __launch_bounds__(kBlock, 8) void dispatch_lean_kernel(DispatchArgs a
       const int i = tb + gidx;  // token of this lane group
       const unsigned long long mine = i < tokens ? (m >> (i * ep)) & seg0 : 0ull;
       for (int off0 = 0; off0 < cpr; off0 += LPR * UPR) {
-        if (tb != 0 || off0 != 0) load_units(i, tokens, step, off0, val);
+        if (tb != 0 || off0 != 0) load_units(i, tokens, step, off0, mine != 0, val);
         unsigned long long rem = mine;
         while (__ballot(rem != 0) != 0) {
           const bool has = rem != 0;
