@@ -518,7 +518,8 @@ def phase_ceilings(gpu):
     """What the machine gives the same run, for the figures of this line to be read against: the
     library's dense bf16 GEMM (torch.matmul, a hipBLASLt kernel) on the two shapes of the
     compute-bound probe, on the same N(0,1) x N(0,0.02) data, and the runtime's device-to-device
-    copy of 512 MiB (read + written: 1 GiB of traffic).  Eager launches between two events on the
+    copy of 512 MiB (read + written: 1 GiB of traffic), and the matrix pipes with nothing but MFMAs
+    to do.  Eager launches between two events on the
     benchmark's stream, 10 per interval, best of 3 intervals; none of it goes into a graph."""
     torch, dev = gpu.torch, gpu.dev
     g = torch.Generator(device="cuda").manual_seed(6)
@@ -557,6 +558,21 @@ def phase_ceilings(gpu):
                                  "GBps": round(2 * src.numel() / t_us / 1e3, 1),
                                  "hbm_frac": round(2 * src.numel() / t_us / 1e3 / HBM_PEAK_GBPS, 4)}
     del src, dst
+    # nothing but MFMAs on register operands of random bits, one wavefront per SIMD: the rate the
+    # power limit leaves of the nominal peak, and the shader clock the pipes sustain it at
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    iters = 40000
+    clocks = torch.zeros(2, dtype=torch.int64, device=dev)
+    t_us = eager_us(lambda: gpu.check(gpu.L.brt_hip_probe_mfma_rate(cus, iters, clocks.data_ptr(), gpu.sptr())), per=2)
+    flop = cus * 4.0 * iters * 8 * 32768
+    out["mfma_only_random_operands"] = {
+        "us": round(t_us, 1), "TFLOPs": round(flop / t_us / 1e6, 1),
+        "mfma_frac": round(flop / t_us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4),
+        "shader_clock_GHz": round(int(clocks[0].item()) / t_us / 1e3, 3),
+        "clocks_per_mfma": round(int(clocks[0].item()) / (iters * 8.0), 2),
+        "note": "brt_hip_probe_mfma_rate: v_mfma_f32_32x32x16_bf16 only, no memory traffic; the clock is "
+                "the loop's shader clocks (s_memtime) over the launch time",
+    }
     torch.cuda.empty_cache()
     return out
 

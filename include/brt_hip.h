@@ -439,6 +439,17 @@ int brt_hip_combine_by_rows(const void* src, void* dst, const float* weights,
                             int cell, int P, int is_residual, int in_dtype, int out_dtype,
                             void* stream);
 
+/*
+ * Measurement aid (no counterpart in the reference; bench.py's `ceilings` uses it): `workgroups`
+ * workgroups of four wavefronts, one per SIMD, each issue iters x 8 v_mfma_f32_32x32x16_bf16
+ * (32768 flop per wavefront and instruction) on register operands of random bit patterns and touch
+ * no memory.  clocks[0] (device, 8-byte aligned) receives the shader clocks the first wavefront
+ * spent in its loop; clocks[1] is reserved and never written in practice.  Launch time and
+ * clocks[0] give the rate the matrix pipes sustain under the part's power limit and the shader
+ * clock they sustain it at.  workgroups 1..65536, iters >= 1.
+ */
+int brt_hip_probe_mfma_rate(int workgroups, int iters, long long* clocks, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -728,3 +728,22 @@ def test_top2_weighted_combine_folded_at_full_size():
             ref[j] += y2[row].double() * float(gates_np[c, e])
     assert (out[cells].double() - ref).abs().max() <= 1e-6 * ref.abs().max()
     del w2
+
+
+def test_mfma_rate_probe_counts_its_clocks():
+    """The measurement aid behind bench.py's `ceilings`: every wavefront issues iters x 8 MFMAs of
+    32 clocks each and nothing else, so the loop's shader clocks are iters x 8 x 32 plus a few per
+    iteration, and bad arguments are refused before anything is launched."""
+    from brainstorm_amd import _lib
+
+    L = _lib.lib()
+    iters = 2000
+    clocks = torch.zeros(2, dtype=torch.int64, device="cuda")
+    _lib.check(L.brt_hip_probe_mfma_rate(64, iters, clocks.data_ptr(), torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    per_mfma = int(clocks[0]) / (iters * 8)
+    assert 31.5 <= per_mfma <= 40.0, per_mfma
+    assert int(clocks[1]) == 0
+    assert L.brt_hip_probe_mfma_rate(0, iters, clocks.data_ptr(), None) == -1  # BRT_E_INVALID
+    assert L.brt_hip_probe_mfma_rate(64, 0, clocks.data_ptr(), None) == -1  # BRT_E_INVALID
+    assert L.brt_hip_probe_mfma_rate(64, iters, None, None) == -1  # BRT_E_INVALID
