@@ -726,10 +726,11 @@ def routing_config(gpu, name, c):
     return res
 
 
-def ffn_config(gpu, loads_np, d, dff, seed, spot_checks=3):
+def ffn_config(gpu, loads_np, d, dff, seed, spot_checks=3, k_loop_clocks=False):
     """Both grouped GEMMs of an expert FFN over the given ragged loads: d -> dff with GELU, then
     dff -> d.  Weights ~ N(0, 0.02) drawn on the device.  A few experts are checked against
-    F.linear in fp32 before the launches are timed."""
+    F.linear in fp32 before the launches are timed.  `k_loop_clocks`: for shapes that the host
+    sends to the ping-pong kernel, also read that kernel's own clocks of the first tile's K loop."""
     torch, L, lib, dev = gpu.torch, gpu.L, gpu._lib, gpu.dev
     En, rows = len(loads_np), int(loads_np.sum())
     g = torch.Generator(device="cuda").manual_seed(seed)
@@ -783,6 +784,22 @@ def ffn_config(gpu, loads_np, d, dff, seed, spot_checks=3):
             "GBps": round(nbytes / t_us / 1e3, 1),
             "hbm_frac": round(nbytes / t_us / 1e3 / HBM_PEAK_GBPS, 4),
         }
+    if k_loop_clocks and d % 64 == 0 and dff % 64 == 0 and int(loads_np[loads_np > 0][0]) >= 256:
+        # the first tile's K loop as the kernel itself clocks it (the timed form of the call runs
+        # the 256 x 256 ping-pong kernel): 2048 of the clocks of a K-step issue MFMAs
+        clocks = torch.zeros(3, dtype=torch.int64, device=dev)
+        for name, args, act in (("gemm1_gelu", (x, t1, h, d, dff), lib.ACT_GELU), ("gemm2", (h, t2, y, dff, d), lib.ACT_NONE)):
+            a_in, tab, a_out, kk, nn = args
+            for _ in range(3):  # the last launch's reading, with the clocks settled
+                gpu.run(lambda: gpu.check(L.brt_hip_grouped_gemm_timed(
+                    a_in.data_ptr(), tab.data_ptr(), None, a_out.data_ptr(), loads.data_ptr(), En, rows, kk, nn,
+                    act, clocks.data_ptr(), gpu.sptr())))
+            shader, ticks, k_steps = (int(v) for v in clocks.tolist())
+            res[name]["k_loop_of_the_first_tile"] = {
+                "k_steps": k_steps, "shader_clocks_per_k_step": round(shader / k_steps, 1),
+                "mfma_issue_frac": round(2048.0 * k_steps / shader, 4),
+                "shader_clock_GHz": round(shader / (ticks * 10.0), 3),
+                "us_per_k_step": round(ticks / 100.0 / k_steps, 3)}
     # which roofline bounds this shape: time at the MFMA peak against time at the HBM peak
     t_mfma, t_hbm = flop / MFMA_BF16_PEAK_TFLOPS / 1e6, nbytes / HBM_PEAK_GBPS / 1e3
     res["bound"] = "mfma" if t_mfma > t_hbm else "hbm"
@@ -873,14 +890,15 @@ def phase_configs(gpu, only=None):
         out["cfg3_ffn_32e_1024_4096"] = ffn_config(gpu, loads3.astype(np.int64), 1024, 4096, seed=3)
     if want("cfg5_task_moe_ffn_128e_2048_8192"):
         loads5 = workloads.dirichlet_loads(32768, 128, 0.3, seed=5)
-        out["cfg5_task_moe_ffn_128e_2048_8192"] = ffn_config(gpu, loads5.astype(np.int64), 2048, 8192, seed=5)
+        out["cfg5_task_moe_ffn_128e_2048_8192"] = ffn_config(gpu, loads5.astype(np.int64), 2048, 8192, seed=5,
+                                                             k_loop_clocks=True)
     if want("cfg3_top2_combine_folded_into_gemm2"):
         out["cfg3_top2_combine_folded_into_gemm2"] = accumulate_config(gpu)
     # what the same kernel does when the shape lets the matrix units be the bound: the same rows
     # and feature sizes over 8 experts of 4096 rows (weights 268 MB per GEMM)
     if want("compute_bound_probe_8e_x_4096_rows_2048_8192"):
         out["compute_bound_probe_8e_x_4096_rows_2048_8192"] = ffn_config(
-            gpu, np.full(8, 4096, dtype=np.int64), 2048, 8192, seed=6, spot_checks=1)
+            gpu, np.full(8, 4096, dtype=np.int64), 2048, 8192, seed=6, spot_checks=1, k_loop_clocks=True)
     return out
 
 

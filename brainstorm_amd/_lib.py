@@ -132,6 +132,10 @@ SIGNATURES = {
          _c_ptr],
     ),
     "brt_hip_probe_mfma_rate": (_c_int, [_c_int, _c_int, _c_ptr, _c_ptr]),
+    "brt_hip_grouped_gemm_timed": (
+        _c_int,
+        [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr],
+    ),
 }
 
 _lib = None

@@ -693,7 +693,7 @@ int grouped_gemm_impl(const void* x, const void* const* weights, const void* con
                       const int32_t* loads, const int32_t* tags, int entries_per_cell, int E, int P,
                       int T, int K, int N, int act, int gather_in, int scatter_out, void* stream,
                       bool out_is_f32 = false, int32_t* row_tags_out = nullptr,
-                      const float* gates = nullptr) {
+                      const float* gates = nullptr, long long* clocks = nullptr) {
   if (E <= 0 || P < 0 || K <= 0 || N <= 0 || T < 0)
     return fail(BRT_E_INVALID, "bad shape E=%d P=%d T=%d K=%d N=%d", E, P, T, K, N);
   if (K % 8 != 0 || N % 8 != 0)
@@ -731,6 +731,12 @@ int grouped_gemm_impl(const void* x, const void* const* weights, const void* con
   // 4.9 us instead of 5.9 us and the GEMM itself nothing (measured inside the step; with ordinary
   // stores in the expanding GEMM that GEMM takes 102 us instead of 87 us).
   a.plain_out = N < K && static_cast<size_t>(P) * N * 2 <= (size_t{32} << 20);
+  if (clocks != nullptr) {  // the timed form: the ping-pong kernel or nothing
+    if (!pingpong_gemm_applies(a) || out_is_f32)
+      return fail(BRT_E_UNSUPPORTED, "the timed form runs the ping-pong kernel only (bf16 output, no tags, K a multiple of 64 and >= 128)");
+    a.clocks = clocks;
+    return launch_pingpong_gemm(a, act, as_stream(stream));
+  }
   if (out_is_f32) {
     if (act == BRT_ACT_GELU) return launch_f32<BRT_ACT_GELU>(a, as_stream(stream));
     if (act == BRT_ACT_RELU) return launch_f32<BRT_ACT_RELU>(a, as_stream(stream));
@@ -783,6 +789,14 @@ extern "C" int brt_hip_grouped_gemm(const void* x, const void* const* weights,
                                     const void* const* biases, void* out, const int32_t* loads,
                                     int E, int P, int K, int N, int act, void* stream) {
   return grouped_gemm_impl(x, weights, biases, out, loads, nullptr, 0, E, P, 0, K, N, act, 0, 0, stream);
+}
+
+extern "C" int brt_hip_grouped_gemm_timed(const void* x, const void* const* weights, const void* const* biases,
+                                          void* out, const int32_t* loads, int E, int P, int K, int N, int act,
+                                          long long* clocks, void* stream) {
+  if (clocks == nullptr) return fail(BRT_E_INVALID, "grouped_gemm_timed: clocks is null");
+  return grouped_gemm_impl(x, weights, biases, out, loads, nullptr, 0, E, P, 0, K, N, act, 0, 0, stream, false,
+                                nullptr, nullptr, clocks);
 }
 
 extern "C" int brt_hip_grouped_gemm_f32out(const void* x, const void* const* weights,

@@ -28,6 +28,10 @@ struct GemmArgs {
   int tiles_n, tiles_m_max;
   int walk, groups_n;  // column tiles one workgroup walks, ceil(tiles_n / walk)
   int patch;           // workgroups in patch order (experts with several row blocks), see the kernel
+  // measurement aid (ping-pong kernel only): non-null, the workgroup of the first tile writes the
+  // shader clocks (s_memtime) and the ticks of the constant 100 MHz counter (s_memrealtime) its
+  // first wavefront spent in the K loop, and the number of K-steps, into clocks[0..2]
+  long long* clocks;
 };
 
 // The 256 x 256 ping-pong kernel (grouped_gemm_pingpong.hip): the shapes it takes, and its launch.

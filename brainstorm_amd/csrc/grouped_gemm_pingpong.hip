@@ -325,9 +325,15 @@ __global__ __launch_bounds__(kWaves * 64) void grouped_gemm_pingpong_kernel(Gemm
       a_load = a_load == 2 * kTileB ? 0 : a_load + kTileB;
     }
   };
+  const long long clock0 = __builtin_amdgcn_s_memtime(), tick0 = __builtin_amdgcn_s_memrealtime();
   if (n_i > 2) k_loop(std::integral_constant<int, 4>{});
   else if (n_i > 0) k_loop(std::integral_constant<int, 2>{});
   else k_loop(std::integral_constant<int, 0>{});
+  if (a.clocks != nullptr && t == 0 && tid == 0) {  // measurement aid: this wavefront's K loop
+    a.clocks[0] = __builtin_amdgcn_s_memtime() - clock0;
+    a.clocks[1] = __builtin_amdgcn_s_memrealtime() - tick0;
+    a.clocks[2] = k_tiles;
+  }
   if (wm == 0) block_barrier();  // group 1's last C phase
   block_barrier();               // no wavefront reads a stage any more: the epilogue may write over them
 

@@ -440,6 +440,21 @@ int brt_hip_combine_by_rows(const void* src, void* dst, const float* weights,
                             void* stream);
 
 /*
+ * Measurement aid (no counterpart in the reference; bench.py reports what it reads beside the
+ * compute-bound shapes): brt_hip_grouped_gemm through the 256 x 256 ping-pong kernel, whatever the
+ * shape (BRT_E_UNSUPPORTED when that kernel does not take it: K must be a multiple of 64 and at
+ * least 128), which also writes into clocks[0..2] (device, 8-byte aligned) what the first
+ * wavefront of the first tile's workgroup spent in its K loop: shader clocks (s_memtime), ticks of
+ * the constant 100 MHz counter (s_memrealtime), and the number of K-steps of 64.  A full tile
+ * issues 2 x 1024 clocks of MFMA per SIMD and K-step, so clocks[0] / clocks[2] says how much of
+ * the loop is matrix work and clocks[0] / clocks[1] at which clock the part ran it.  The output is
+ * that of brt_hip_grouped_gemm, bit for bit.
+ */
+int brt_hip_grouped_gemm_timed(const void* x, const void* const* weights, const void* const* biases,
+                               void* out, const int32_t* loads, int E, int P, int K, int N, int act,
+                               long long* clocks, void* stream);
+
+/*
  * Measurement aid (no counterpart in the reference; bench.py's `ceilings` uses it): `workgroups`
  * workgroups of four wavefronts, one per SIMD, each issue iters x 8 v_mfma_f32_32x32x16_bf16
  * (32768 flop per wavefront and instruction) on register operands of random bit patterns and touch

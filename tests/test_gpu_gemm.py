@@ -747,3 +747,40 @@ def test_mfma_rate_probe_counts_its_clocks():
     assert L.brt_hip_probe_mfma_rate(0, iters, clocks.data_ptr(), None) == -1  # BRT_E_INVALID
     assert L.brt_hip_probe_mfma_rate(64, 0, clocks.data_ptr(), None) == -1  # BRT_E_INVALID
     assert L.brt_hip_probe_mfma_rate(64, iters, None, None) == -1  # BRT_E_INVALID
+
+
+def test_timed_grouped_gemm_gives_the_same_rows_and_plausible_clocks():
+    """The timed form (a measurement aid) runs the ping-pong kernel: its output must be the plain
+    call's, bit for bit, and the K loop of a full 256 x 256 tile cannot take fewer shader clocks
+    than its 2 x 1024 clocks of MFMA per K-step; shapes that kernel does not take are refused."""
+    from brainstorm_amd import _lib
+
+    L = _lib.lib()
+    loads, K, N = [1024] * 8, 512, 2048
+    E, P = len(loads), sum(loads)
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(P, K, generator=g).to(torch.bfloat16).cuda()
+    ws = [(torch.randn(N, K, generator=g) * 0.05).to(torch.bfloat16).cuda() for _ in range(E)]
+    bs = [torch.randn(N, generator=g).to(torch.bfloat16).cuda() for _ in range(E)]
+    wt = torch.tensor([w.data_ptr() for w in ws], dtype=torch.int64, device="cuda")
+    bt = torch.tensor([b.data_ptr() for b in bs], dtype=torch.int64, device="cuda")
+    d_loads = torch.tensor(loads, dtype=torch.int32, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+    plain = torch.full((P, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    timed = torch.full((P, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    clocks = torch.zeros(3, dtype=torch.int64, device="cuda")
+    _lib.check(L.brt_hip_grouped_gemm(x.data_ptr(), wt.data_ptr(), bt.data_ptr(), plain.data_ptr(),
+                                      d_loads.data_ptr(), E, P, K, N, ACT["gelu"], st))
+    _lib.check(L.brt_hip_grouped_gemm_timed(x.data_ptr(), wt.data_ptr(), bt.data_ptr(), timed.data_ptr(),
+                                            d_loads.data_ptr(), E, P, K, N, ACT["gelu"], clocks.data_ptr(), st))
+    torch.cuda.synchronize()
+    assert torch.equal(plain.view(torch.int16), timed.view(torch.int16))
+    shader, ticks, k_steps = (int(v) for v in clocks)
+    assert k_steps == K // 64
+    assert 2048 * k_steps <= shader <= 6000 * k_steps, (shader, k_steps)
+    assert 0.5 <= shader / (ticks * 10.0) <= 2.5, (shader, ticks)  # GHz: the counter behind `ticks` runs at 100 MHz
+    # K = 72 is not a whole number of K-steps of 64: the timed form has no other kernel to fall back to
+    assert L.brt_hip_grouped_gemm_timed(x.data_ptr(), wt.data_ptr(), bt.data_ptr(), timed.data_ptr(),
+                                        d_loads.data_ptr(), E, P, 72, N, ACT["none"], clocks.data_ptr(), st) == -4
+    assert L.brt_hip_grouped_gemm_timed(x.data_ptr(), wt.data_ptr(), bt.data_ptr(), timed.data_ptr(),
+                                        d_loads.data_ptr(), E, P, K, N, ACT["none"], None, st) == -1
