@@ -25,7 +25,7 @@
 //     three to four phases to land, and each wavefront issues its 8 loads of a K-step in its M
 //     phase, between fragment reads.  A K-step is 2 x 1024 clocks of MFMA per SIMD and measures
 //     about 2100 (s_memtime at the phase boundaries: M phase 820-865, C phase's MFMAs back to back),
-//     at a shader clock of 1.3-1.45 GHz under this load: time, not clocks, is what is left to win,
+//     at a shader clock of 1.3-1.6 GHz under this load (boxes differ): time, not clocks, is what is left to win,
 //     i.e. less energy per K-step.  Its 64 KB of loads alone take 0.62 us per CU when the rows are up to 8 KB apart and 1.08 us when they
 //     are 16 KB apart (K = 8192: the 512 rows of a tile pair then lie in 128 regions of 64 KB,
 //     more than a CU's address translation holds), so the load stream has to be fed in every
